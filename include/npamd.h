@@ -1,0 +1,159 @@
+/*
+ * npamd.h -- C ABI of libnpamd.so: the MI355X (gfx950) backend for
+ * neuropress's quantized-linear forward path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says otherwise;
+ *   - the library never allocates, frees or keeps a pointer after return;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     launches are asynchronous, nothing here synchronises;
+ *   - return value 0 = success, negative = NPAMD_ERR_*; npamd_last_error()
+ *     then returns a thread-local human-readable message;
+ *   - dtype codes: NPAMD_F16 / NPAMD_BF16 / NPAMD_F32;
+ *   - x is [M, K] with row stride ldx (elements), y is [M, N] with row stride
+ *     ldy; weights are never materialised by the gemv / gemm_tile entry points.
+ *
+ * Index bit-stream ("packed"): index i occupies bits [i*bits, (i+1)*bits) of a
+ * byte stream, LSB first; flat index of (row n, group g) is n*(K/VL)+g.
+ * Codebooks are fp16 [NC, VL] row-major (NPAMD_F16), or -- for the gemv /
+ * gemm_tile entry points only -- already cast to the activation dtype.
+ *
+ * Paths are relative to the reference repository (DreamerMind/neuropress).
+ */
+#ifndef NPAMD_H
+#define NPAMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NPAMD_F16 0
+#define NPAMD_BF16 1
+#define NPAMD_F32 2
+
+#define NPAMD_OK 0
+#define NPAMD_ERR_INVALID (-1)     /* bad argument (shape, dtype, null, alignment) */
+#define NPAMD_ERR_UNSUPPORTED (-2) /* valid request this build has no kernel for */
+#define NPAMD_ERR_LAUNCH (-3)      /* HIP reported an error at launch */
+
+/* Largest token count the fused decode-GEMV entry points accept. */
+#define NPAMD_GEMV_MAX_M 16
+
+/* Library ABI version (bumped on any signature change). */
+int npamd_version(void);
+
+/* Thread-local message for the last failing call on this thread ("" if none). */
+const char* npamd_last_error(void);
+
+/* ---------------------------------------------------------------- VQ ---- */
+
+/*
+ * One-pass decode: out.flat[v*VL + j] = cast(codebook[idx(v), j]).
+ * Replaces vq_dequant (neuropress/kernels/vq_dequant.cu:105-146) and
+ * dequantize_vq_weight (neuropress/kernels/vq_linear.cu:458-479).
+ * bits in [4, 20]; out_dtype any of the three; out holds n_vectors*VL elements.
+ */
+int npamd_vq_dequant(const uint8_t* packed, int64_t n_bytes, int bits,
+                     const void* codebook_f16, int nc, int vl,
+                     int64_t n_vectors, void* out, int out_dtype, void* stream);
+
+/*
+ * Fused decode GEMV, M <= NPAMD_GEMV_MAX_M:
+ *   y[m, n] = sum_k x[m, k] * codebook[idx(n, k/VL), k%VL] (+ bias[n]), f32 accumulate.
+ * Replaces vq_linear (neuropress/kernels/vq_linear.cu:344-424) and the GEMV
+ * branch of vq_linear_wmma (neuropress/kernels/vq_linear_wmma.cu:187-240, 468-540).
+ * act_dtype: NPAMD_F16 or NPAMD_BF16 (x and y).  codebook_dtype: NPAMD_F16, or
+ * the activation dtype when the caller pre-cast the codebook.  bias: f32 [N] or NULL.
+ */
+int npamd_vq_gemv(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_bytes,
+                  int bits, const void* codebook, int codebook_dtype, int nc, int vl,
+                  const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                  int act_dtype, void* stream);
+
+/*
+ * Tile-decode MFMA GEMM, any M >= 1: same contraction, weight tiles decoded
+ * inside the kernel, dense weight never written.
+ * Replaces vq_gemm_triton (neuropress/kernels/vq_triton.py:119-179) and the
+ * WMMA GEMM branch of vq_linear_wmma (neuropress/kernels/vq_linear_wmma.cu:261-394).
+ */
+int npamd_vq_gemm_tile(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_bytes,
+                       int bits, const void* codebook, int codebook_dtype, int nc, int vl,
+                       const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                       int act_dtype, void* stream);
+
+/*
+ * Widen a bit-stream to one uint16 per index (the layout the fast kernels
+ * stream at bits=16).  Same stream semantics as unpack_indices
+ * (neuropress/kernels/kmeans_assign.cu:405-451); bits in [4, 16].
+ */
+int npamd_vq_widen_u16(const uint8_t* packed, int64_t n_bytes, int bits,
+                       int64_t n_indices, uint16_t* out, void* stream);
+
+/* ------------------------------------------------- residual VQ (RVQ) ---- */
+/*
+ * Two codebooks + per-output-row fp16 scale and bias (no counterpart in the
+ * reference; BASELINE config 4):
+ *   W[n, g*VL+j] = f16(f16(f16(Cm[im(n,g),j] + Cr[ir(n,g),j]) * s[n]) + b[n])
+ * row_scale / row_bias: fp16 [N] or NULL.  Both codebooks fp16, same VL.
+ */
+int npamd_rvq_dequant(const uint8_t* packed_main, int64_t n_bytes_main, int bits_main,
+                      const uint8_t* packed_res, int64_t n_bytes_res, int bits_res,
+                      const void* cb_main_f16, int nc_main, const void* cb_res_f16, int nc_res,
+                      const void* row_scale_f16, const void* row_bias_f16, int vl,
+                      int N, int K, void* out, int out_dtype, void* stream);
+
+int npamd_rvq_gemv(const void* x, int64_t ldx,
+                   const uint8_t* packed_main, int64_t n_bytes_main, int bits_main,
+                   const uint8_t* packed_res, int64_t n_bytes_res, int bits_res,
+                   const void* cb_main_f16, int nc_main, const void* cb_res_f16, int nc_res,
+                   const void* row_scale_f16, const void* row_bias_f16, int vl,
+                   const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                   int act_dtype, void* stream);
+
+int npamd_rvq_gemm_tile(const void* x, int64_t ldx,
+                        const uint8_t* packed_main, int64_t n_bytes_main, int bits_main,
+                        const uint8_t* packed_res, int64_t n_bytes_res, int bits_res,
+                        const void* cb_main_f16, int nc_main, const void* cb_res_f16, int nc_res,
+                        const void* row_scale_f16, const void* row_bias_f16, int vl,
+                        const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                        int act_dtype, void* stream);
+
+/* ------------------------------------------- group-affine n-bit (Q4) ---- */
+/*
+ * w_pack: uint8 [N, K/vpb], vpb = 8/nbits, value k of row n =
+ *   (w_pack[n, k/vpb] >> ((k%vpb)*nbits)) & mask   (low nibble = even k);
+ * scale: fp16 [N*(K/group_size)]; zero_point: fp16 same shape or NULL
+ * (symmetric: zp = 2^(nbits-1));  w = (float(q) - zp) * float(scale), f32.
+ */
+
+/*
+ * Decode to a dense [N, K] weight, one RNE rounding to out_dtype.
+ * Restates the decode half of _q_dequant_linear (neuropress/nn/np_linear.py:333-353).
+ */
+int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, const void* zero_point_f16,
+                    int N, int K, int nbits, int group_size, void* out, int out_dtype,
+                    void* stream);
+
+/*
+ * Fused dequant GEMV, M <= NPAMD_GEMV_MAX_M.
+ * Replaces q_linear (neuropress/kernels/q4_linear.cu:80-131, 179-253).
+ */
+int npamd_q_gemv(const void* x, int64_t ldx, const uint8_t* w_pack, const void* scale_f16,
+                 const void* zero_point_f16, const float* bias, void* y, int64_t ldy,
+                 int M, int N, int K, int nbits, int group_size, int act_dtype, void* stream);
+
+/*
+ * Fused dequant MFMA GEMM, any M.  The reference has no kernel of its own here
+ * (it defers to the third-party gemlite: neuropress/nn/np_linear.py:763-776).
+ */
+int npamd_q_gemm_tile(const void* x, int64_t ldx, const uint8_t* w_pack, const void* scale_f16,
+                      const void* zero_point_f16, const float* bias, void* y, int64_t ldy,
+                      int M, int N, int K, int nbits, int group_size, int act_dtype,
+                      void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NPAMD_H */

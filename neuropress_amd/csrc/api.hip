@@ -1,0 +1,104 @@
+// Library-level entry points: version, thread-local error text, launch check.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <stdlib.h>
+
+#include "gemm_tile.hpp"
+#include "gemv.hpp"
+
+namespace npamd {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(NPAMD_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return NPAMD_OK;
+}
+
+const char* error_text() { return g_err; }
+
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : dflt;
+}
+
+static int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+// One "job" = one 16-row tile x one 256-k step.  The kernel lasts about one
+// HBM round trip, so the plan aims at every job's packed bytes being requested
+// as soon as the grid starts: jobs per wave is kept near jobs / (16 waves * CUs).
+// NPAMD_GEMV_R / NPAMD_GEMV_SPW override the choice (tuning aid).
+GemvPlan plan_gemv(int N, int chunks) {
+  const int steps = (chunks + 3) / 4;
+  const int tiles = (N + 15) / 16;
+  const int64_t jobs = (int64_t)tiles * steps;
+  const int64_t target_waves = (int64_t)device_cu_count() * 16;
+  int jpw = (int)((jobs + target_waves - 1) / target_waves);
+  if (jpw < 1) jpw = 1;
+  GemvPlan p;
+  p.R = (jpw >= 2 && tiles >= 2) ? 2 : 1;
+  int spw = (jpw + p.R - 1) / p.R;
+  const int r_env = env_int("NPAMD_GEMV_R", 0);
+  if (r_env == 1 || r_env == 2 || r_env == 4) p.R = r_env;
+  const int spw_env = env_int("NPAMD_GEMV_SPW", 0);
+  if (spw_env > 0) spw = spw_env;
+  const int max_waves = p.R >= 4 ? 8 : 16;
+  if ((steps + spw - 1) / spw > max_waves) spw = (steps + max_waves - 1) / max_waves;
+  p.steps_per_wave = spw;
+  p.waves = (steps + spw - 1) / spw;
+  return p;
+}
+
+// NPAMD_TILE_MT overrides the choice (tuning aid).
+int plan_tile_mt(int M, int N) {
+  const int mt_env = env_int("NPAMD_TILE_MT", 0);
+  if (mt_env >= 1 && mt_env <= 4) return mt_env;
+  const int cus = device_cu_count();
+  const int n_blocks = (N + kTileCols - 1) / kTileCols;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int mt = 1; mt <= 4; ++mt) {
+    const int m_blocks = (M + 32 * mt - 1) / (32 * mt);
+    const int64_t blocks = (int64_t)m_blocks * n_blocks;
+    const int64_t passes = (blocks + cus - 1) / cus;
+    const double cost = (double)passes * (mt + 1.0);
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = mt;
+    }
+  }
+  return best;
+}
+
+}  // namespace npamd
+
+extern "C" int npamd_version(void) { return 1; }
+
+extern "C" const char* npamd_last_error(void) { return npamd::error_text(); }

@@ -1,0 +1,245 @@
+// Fused decode GEMV for small token counts (M <= 16), wave64 + MFMA 16x16x32.
+//
+// The contraction y[m, n] = sum_k x[m, k] * W[n, k] is issued as
+// D[16 x 16] += A[16 x 32] * B[32 x 16] with A = x (rows m, zero beyond M) and
+// B = W^T (columns n).  Lane l = (c = l % 16, q = l / 16) supplies
+//   A: x[m = c][8 consecutive k of k-slot q]      (16 bytes, zero if c >= M)
+//   B: W[n = n0 + c][the same 8 k]                (16 bytes = one VQ codebook row)
+// so a gathered codebook row is already a B-operand: no LDS, no VALU work on
+// the weights, and M = 1 ... 16 all cost the same.  The kernel is bound by the
+// packed-weight stream from HBM plus, for codebooks larger than L1, the
+// 16-byte gathers out of L2.
+//
+// Work split: a "chunk" is 64 k of one row (8 operands); one "step" is the 4
+// k-slots of a wave = 256 k.  A block owns 16*R rows and all of K; its S waves
+// split the steps and their partial tiles are summed through LDS.
+#pragma once
+
+#include "providers.hpp"
+
+namespace npamd {
+
+struct GemvShape {
+  const void* x;
+  int64_t ldx;
+  const float* bias;
+  void* y;
+  int64_t ldy;
+  int M, N;
+  int chunks;          // K / 64 (K % 64 == 0 is a precondition of this kernel)
+  int steps;           // ceil(chunks / 4)
+  int steps_per_wave;  // steps each wave of the block covers
+};
+
+// R = 4 keeps 32 gathered operands (128 registers) live per lane, so it is
+// limited to 8 waves per block; R <= 2 fits the 128-register budget of 16 waves.
+template <int R>
+constexpr int kGemvMaxWaves = (R >= 4) ? 8 : 16;
+
+template <int ACT, class Provider, int R>
+__global__ void __launch_bounds__(kGemvMaxWaves<R> * 64)
+fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
+  extern __shared__ float red[];  // [waves][M][16*R]
+  const Provider prov(pargs);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n_waves = blockDim.x >> 6;
+  const int c = lane & 15;
+  const int q = lane >> 4;
+  const int row0 = blockIdx.x * (16 * R);
+
+  f32x4 acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int step_begin = wave * s.steps_per_wave;
+  const int step_end = min(step_begin + s.steps_per_wave, s.steps);
+  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(s.x) + (int64_t)c * s.ldx;
+  const bool x_lane = c < s.M;
+
+  for (int step = step_begin; step < step_end; ++step) {
+    const int kc = step * 4 + q;
+    const bool kvalid = kc < s.chunks;
+
+    typename Provider::Raw raw[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = row0 + 16 * r + c;
+      prov.load(raw[r], n, kc, kvalid && n < s.N);
+    }
+
+    u32x4 xa[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      xa[j] = u32x4{0, 0, 0, 0};
+      if (x_lane && kvalid) {
+        xa[j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)kc * 64 + j * 8);
+        if constexpr (Provider::kPermuteA) xa[j] = permute_a_0415(xa[j]);
+      }
+    }
+
+    u32x4 b[R][8];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const bool valid = kvalid && (row0 + 16 * r + c) < s.N;
+      b[r][0] = prov.template operand<0>(raw[r], valid);
+      b[r][1] = prov.template operand<1>(raw[r], valid);
+      b[r][2] = prov.template operand<2>(raw[r], valid);
+      b[r][3] = prov.template operand<3>(raw[r], valid);
+      b[r][4] = prov.template operand<4>(raw[r], valid);
+      b[r][5] = prov.template operand<5>(raw[r], valid);
+      b[r][6] = prov.template operand<6>(raw[r], valid);
+      b[r][7] = prov.template operand<7>(raw[r], valid);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = mfma16<ACT>(xa[j], b[r][j], acc[r]);
+  }
+
+  // D layout: lane (c, q) holds D[m = 4q + i][n = c], i = 0..3.
+  const int cols = 16 * R;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * q + i;
+      if (m < s.M) red[((int64_t)wave * s.M + m) * cols + r * 16 + c] = acc[r][i];
+    }
+  }
+  __syncthreads();
+  for (int o = threadIdx.x; o < s.M * cols; o += blockDim.x) {
+    const int m = o / cols;
+    const int col = o - m * cols;
+    const int n = row0 + col;
+    if (n >= s.N) continue;
+    float v = 0.f;
+    for (int w = 0; w < n_waves; ++w) v += red[((int64_t)w * s.M + m) * cols + col];
+    if (s.bias) v += s.bias[n];
+    store_from_f32<ACT>(s.y, (int64_t)m * s.ldy + n, v);
+  }
+}
+
+// Launch geometry: enough waves to put the whole packed stream in flight at
+// once (the kernel lasts a few microseconds, about one HBM round trip), capped
+// at 16 waves per block.
+struct GemvPlan {
+  int R;               // row tiles (of 16) per block
+  int waves;           // waves per block
+  int steps_per_wave;
+};
+
+GemvPlan plan_gemv(int N, int chunks);
+
+template <int ACT, class Provider, int R>
+int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const GemvPlan& plan,
+                        hipStream_t st, const char* what) {
+  s.steps_per_wave = plan.steps_per_wave;
+  const int blocks = (s.N + 16 * R - 1) / (16 * R);
+  const size_t lds = (size_t)plan.waves * s.M * 16 * R * sizeof(float);
+  fused_gemv_kernel<ACT, Provider, R><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
+  return check_launch(what);
+}
+
+template <int ACT, class Provider>
+int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStream_t st,
+                      const char* what) {
+  s.steps = (s.chunks + 3) / 4;
+  const GemvPlan plan = plan_gemv(s.N, s.chunks);
+  if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4>(s, pargs, plan, st, what);
+  if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2>(s, pargs, plan, st, what);
+  return launch_fused_gemv_r<ACT, Provider, 1>(s, pargs, plan, st, what);
+}
+
+// ---------------------------------------------------------------------------
+// Fallback for shapes the MFMA kernel does not take (odd vector length or index
+// width, K not a multiple of 64, unaligned buffers): one wave per output
+// element, lanes stride over k, every weight element decoded on its own.
+// Slow by design; exists so that every valid input has a HIP path.
+//   Elem::get(n, k) -> float weight value in the activation dtype's rounding.
+// ---------------------------------------------------------------------------
+template <int ACT, class Elem>
+__global__ void __launch_bounds__(256)
+generic_gemv_kernel(const void* __restrict__ x, int64_t ldx, const float* __restrict__ bias,
+                    void* __restrict__ y, int64_t ldy, int M, int N, int K, const Elem elem) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int m = blockIdx.y;
+  if (n >= N || m >= M) return;
+  float acc = 0.f;
+  for (int k = lane; k < K; k += 64)
+    acc = __builtin_fmaf(load_as_f32<ACT>(x, (int64_t)m * ldx + k), elem.get(n, k), acc);
+  acc = wave_reduce_sum(acc);
+  if (lane == 0) {
+    if (bias) acc += bias[n];
+    store_from_f32<ACT>(y, (int64_t)m * ldy + n, acc);
+  }
+}
+
+template <int ACT, class Elem>
+int launch_generic_gemv(const void* x, int64_t ldx, const float* bias, void* y, int64_t ldy,
+                        int M, int N, int K, const Elem& elem, hipStream_t st, const char* what) {
+  const dim3 grid((N + 3) / 4, M);
+  generic_gemv_kernel<ACT, Elem><<<grid, 256, 0, st>>>(x, ldx, bias, y, ldy, M, N, K, elem);
+  return check_launch(what);
+}
+
+// Weight element of a (residual) VQ layer, any VL / index width.
+struct VqElem {
+  const uint8_t* packed;
+  int64_t n_bytes;
+  int bits;
+  const uint16_t* cb;
+  uint32_t nc_minus_1;
+  int vl, groups;
+  int act;       // activation dtype the weight is rounded to
+  int cb_dtype;  // NPAMD_F16, or NPAMD_BF16 when the caller pre-cast the codebook
+  // residual part (packed_r == nullptr -> plain VQ)
+  const uint8_t* packed_r;
+  int64_t n_bytes_r;
+  int bits_r;
+  const uint16_t* cb_r;
+  uint32_t ncr_minus_1;
+  const uint16_t* row_scale;
+  const uint16_t* row_bias;
+
+  __device__ __forceinline__ float get(int n, int k) const {
+#pragma clang fp contract(off)
+    const int g = k / vl, v = k - g * vl;
+    const int64_t flat = (int64_t)n * groups + g;
+    const uint32_t i = min(read_index(packed, n_bytes, flat, bits), nc_minus_1);
+    if (cb_dtype == NPAMD_BF16) return bf16_bits_to_f32(cb[(int64_t)i * vl + v]);
+    _Float16 h = __builtin_bit_cast(_Float16, cb[(int64_t)i * vl + v]);
+    if (packed_r) {
+      const uint32_t ir = min(read_index(packed_r, n_bytes_r, flat, bits_r), ncr_minus_1);
+      h = h + __builtin_bit_cast(_Float16, cb_r[(int64_t)ir * vl + v]);
+      if (row_scale) h = h * __builtin_bit_cast(_Float16, row_scale[n]);
+      if (row_bias) h = h + __builtin_bit_cast(_Float16, row_bias[n]);
+    }
+    const float f = (float)h;
+    return act == NPAMD_BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(f)) : f;
+  }
+};
+
+// Weight element of a group-affine n-bit layer, any nbits in {1,2,4,8}, sym or asym.
+struct QElem {
+  const uint8_t* w_pack;
+  const uint16_t* scale;
+  const uint16_t* zero_point;  // may be null
+  int K, nbits, group_size;
+  int act;
+
+  __device__ __forceinline__ float get(int n, int k) const {
+#pragma clang fp contract(off)
+    const int vpb = 8 / nbits;
+    const int q = (w_pack[(int64_t)n * (K / vpb) + k / vpb] >> ((k % vpb) * nbits)) & ((1 << nbits) - 1);
+    const int64_t sidx = (int64_t)n * (K / group_size) + k / group_size;
+    const float zp = zero_point ? f16_bits_to_f32(zero_point[sidx]) : (float)(1 << (nbits - 1));
+    const float d = (float)q - zp;
+    const float w = d * f16_bits_to_f32(scale[sidx]);
+    return act == NPAMD_BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(w))
+                             : f16_bits_to_f32(f32_to_f16_bits(w));
+  }
+};
+
+}  // namespace npamd

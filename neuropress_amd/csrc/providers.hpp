@@ -1,0 +1,193 @@
+// Weight-operand providers for the fused kernels.
+//
+// The fused GEMV and the tile GEMM never see a dense weight.  Each lane owns a
+// "chunk": 64 consecutive k of one weight row n, i.e. eight MFMA B-operands of
+// eight 16-bit values.  A provider turns the packed bytes of that chunk into
+// those operands:
+//
+//   load(raw, n, kc, valid)   -- global loads of the packed chunk kc of row n
+//   operand<j>(raw, valid)    -- B-operand j (k = 64*kc + 8*j .. +7) in the
+//                                activation dtype, zero when !valid
+//
+// A B-operand of a VQ weight with VL = 8 is exactly one codebook row, so the
+// 16-byte gather lands in MFMA layout with no shuffling.  For int4 the eight
+// nibbles of one dword are one operand, produced in the k-order
+// (0,4,1,5,2,6,3,7); the A-operand is permuted the same way (kPermuteA).
+#pragma once
+
+#include "common.hpp"
+
+namespace npamd {
+
+// ---------------------------------------------------------------------------
+// Single-codebook VQ, VL = 8, fast index widths.
+//   CONV : codebook is fp16 but activations are bf16 -> convert per gather.
+// ---------------------------------------------------------------------------
+template <int ACT, int BITS, bool CONV>
+struct VqProvider {
+  static constexpr bool kPermuteA = false;
+  struct Args {
+    const uint8_t* packed;
+    const u32x4* cb;
+    uint32_t nc_minus_1;
+    int chunks;  // K / 64
+  };
+  struct Raw {
+    u32x4 idx;
+  };
+  const Args& a;
+  __device__ explicit VqProvider(const Args& args) : a(args) {}
+
+  __device__ __forceinline__ void load(Raw& r, int n, int kc, bool valid) const {
+    r.idx = u32x4{0, 0, 0, 0};
+    if (valid) r.idx = load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8);
+  }
+  template <int J>
+  __device__ __forceinline__ u32x4 operand(const Raw& r, bool valid) const {
+    u32x4 c{0, 0, 0, 0};
+    if (valid) {
+      const uint32_t idx = min(idx8_get(r.idx, J), a.nc_minus_1);
+      c = a.cb[idx];
+      if constexpr (CONV) c = cb_to_act<ACT>(c);
+    }
+    return c;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Residual VQ: main + residual codebook (fp16), per-row fp16 scale and bias.
+//   w = f16(f16(f16(cm + cr) * s) + b), each op rounded separately.
+// ---------------------------------------------------------------------------
+template <int ACT, int BITS_M, int BITS_R>
+struct RvqProvider {
+  static constexpr bool kPermuteA = false;
+  struct Args {
+    const uint8_t* packed_m;
+    const uint8_t* packed_r;
+    const u32x4* cb_m;
+    const u32x4* cb_r;
+    const uint16_t* row_scale;  // may be null
+    const uint16_t* row_bias;   // may be null
+    uint32_t ncm_minus_1, ncr_minus_1;
+    int chunks;
+  };
+  struct Raw {
+    u32x4 im, ir;
+    uint32_t s2, b2;  // scale / bias replicated in both halves
+  };
+  const Args& a;
+  __device__ explicit RvqProvider(const Args& args) : a(args) {}
+
+  __device__ __forceinline__ void load(Raw& r, int n, int kc, bool valid) const {
+    r.im = u32x4{0, 0, 0, 0};
+    r.ir = u32x4{0, 0, 0, 0};
+    r.s2 = 0x3C003C00u;  // 1.0, 1.0
+    r.b2 = 0u;
+    if (valid) {
+      const int64_t i0 = ((int64_t)n * a.chunks + kc) * 8;
+      r.im = load_idx8<BITS_M>(a.packed_m, i0);
+      r.ir = load_idx8<BITS_R>(a.packed_r, i0);
+      if (a.row_scale) r.s2 = (uint32_t)a.row_scale[n] * 0x10001u;
+      if (a.row_bias) r.b2 = (uint32_t)a.row_bias[n] * 0x10001u;
+    }
+  }
+  template <int J>
+  __device__ __forceinline__ u32x4 operand(const Raw& r, bool valid) const {
+#pragma clang fp contract(off)
+    u32x4 c{0, 0, 0, 0};
+    if (valid) {
+      const u32x4 cm = a.cb_m[min(idx8_get(r.im, J), a.ncm_minus_1)];
+      const u32x4 cr = a.cb_r[min(idx8_get(r.ir, J), a.ncr_minus_1)];
+      const f16x2 s = __builtin_bit_cast(f16x2, r.s2);
+      const f16x2 b = __builtin_bit_cast(f16x2, r.b2);
+      const bool has_s = a.row_scale != nullptr, has_b = a.row_bias != nullptr;
+      uint32_t o[4];
+      const uint32_t m4[4] = {cm.x, cm.y, cm.z, cm.w};
+      const uint32_t r4[4] = {cr.x, cr.y, cr.z, cr.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        f16x2 h = __builtin_bit_cast(f16x2, m4[i]) + __builtin_bit_cast(f16x2, r4[i]);
+        if (has_s) h = h * s;
+        if (has_b) h = h + b;
+        o[i] = __builtin_bit_cast(uint32_t, h);
+      }
+      c = cb_to_act<ACT>(u32x4{o[0], o[1], o[2], o[3]});
+    }
+    return c;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Symmetric int4, zero point 8, group size a multiple of 32.
+// One dword of nibbles = one operand, emitted in k-order (0,4,1,5,2,6,3,7).
+// f16: w = f16((q-8) * s) -- exact product, one rounding: the oracle's weight.
+// bf16: w = bf16((q-8) * s) with the product taken in f32.
+// ---------------------------------------------------------------------------
+template <int ACT>
+struct Q4Provider {
+  static constexpr bool kPermuteA = true;
+  struct Args {
+    const uint8_t* w_pack;   // [N, K/2]
+    const uint16_t* scale;   // [N, K/gs]
+    int chunks;              // K / 64
+    int groups_per_row;      // K / gs
+    int gs_shift_chunks;     // log2(gs/32): scale index = (2*kc + half) >> gs_shift_chunks
+  };
+  struct Raw {
+    u32x4 w0, w1;
+    uint32_t s_lo, s_hi;  // scale (replicated pair) for operands 0-3 and 4-7
+  };
+  const Args& a;
+  __device__ explicit Q4Provider(const Args& args) : a(args) {}
+
+  __device__ __forceinline__ void load(Raw& r, int n, int kc, bool valid) const {
+    r.w0 = u32x4{0, 0, 0, 0};
+    r.w1 = u32x4{0, 0, 0, 0};
+    r.s_lo = r.s_hi = 0;
+    if (valid) {
+      const u32x4* p = reinterpret_cast<const u32x4*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 32);
+      r.w0 = p[0];
+      r.w1 = p[1];
+      const uint16_t* s = a.scale + (int64_t)n * a.groups_per_row;
+      r.s_lo = (uint32_t)s[(2 * kc) >> a.gs_shift_chunks] * 0x10001u;
+      r.s_hi = (uint32_t)s[(2 * kc + 1) >> a.gs_shift_chunks] * 0x10001u;
+    }
+  }
+  template <int J>
+  __device__ __forceinline__ u32x4 operand(const Raw& r, bool valid) const {
+#pragma clang fp contract(off)
+    (void)valid;  // raw words and scales are zero when invalid -> (0-8)*0 = -0: harmless, x is 0 there
+    const u32x4& ww = (J < 4) ? r.w0 : r.w1;
+    const uint32_t w = (J % 4 == 0) ? ww.x : (J % 4 == 1) ? ww.y : (J % 4 == 2) ? ww.z : ww.w;
+    const uint32_t s2 = (J < 4) ? r.s_lo : r.s_hi;
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // (1024 + q) as fp16 via the exponent trick, then subtract 1032 -> q - 8 exactly.
+      const uint32_t pair = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+      const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, 0x64086408u);
+      if constexpr (ACT == NPAMD_F16) {
+        o[i] = __builtin_bit_cast(uint32_t, q * __builtin_bit_cast(f16x2, s2));
+      } else {
+        const float sf = f16_bits_to_f32(s2 & 0xFFFFu);
+        bf16x2 b;
+        b.x = (__bf16)((float)q.x * sf);
+        b.y = (__bf16)((float)q.y * sf);
+        o[i] = __builtin_bit_cast(uint32_t, b);
+      }
+    }
+    return u32x4{o[0], o[1], o[2], o[3]};
+  }
+};
+
+// A-operand (x) permutation matching Q4Provider's k-order.
+__device__ __forceinline__ u32x4 permute_a_0415(u32x4 x) {
+  u32x4 r;
+  r.x = (x.x & 0xFFFFu) | (x.z << 16);
+  r.y = (x.x >> 16) | (x.z & 0xFFFF0000u);
+  r.z = (x.y & 0xFFFFu) | (x.w << 16);
+  r.w = (x.y >> 16) | (x.w & 0xFFFF0000u);
+  return r;
+}
+
+}  // namespace npamd

@@ -1,0 +1,197 @@
+// One-pass VQ decode kernels: packed index stream + fp16 codebook -> dense weight.
+//
+//   out.flat[v*VL + j] = cast(codebook[idx(v), j])
+//
+// HBM-bound byte work: one thread per vector, coalesced index reads (2 B/lane
+// at 16 bits), one 16-byte codebook gather (L2-resident table), one vector
+// store.  Traffic = index stream + output; the codebook is read from cache.
+#include "common.hpp"
+
+namespace npamd {
+
+#pragma clang fp contract(off)
+
+// Index of vector v.  BITS is 8 or 16 for the byte-aligned widths, 0 for the
+// bounds-checked window reader.
+template <int BITS>
+__device__ __forceinline__ uint32_t vec_index(const uint8_t* __restrict__ packed, int64_t n_bytes,
+                                              int64_t v, int bits) {
+  if constexpr (BITS == 16) return reinterpret_cast<const uint16_t*>(packed)[v];
+  else if constexpr (BITS == 8) return packed[v];
+  else return read_index(packed, n_bytes, v, bits);
+}
+
+template <int OUT>
+__device__ __forceinline__ void store8(void* out, int64_t v, u32x4 c) {
+  if constexpr (OUT == NPAMD_F16) {
+    reinterpret_cast<u32x4*>(out)[v] = c;
+  } else if constexpr (OUT == NPAMD_BF16) {
+    reinterpret_cast<u32x4*>(out)[v] = cb_to_act<NPAMD_BF16>(c);
+  } else {
+    f32x4 lo, hi;
+    lo.x = f16_bits_to_f32(c.x & 0xFFFFu); lo.y = f16_bits_to_f32(c.x >> 16);
+    lo.z = f16_bits_to_f32(c.y & 0xFFFFu); lo.w = f16_bits_to_f32(c.y >> 16);
+    hi.x = f16_bits_to_f32(c.z & 0xFFFFu); hi.y = f16_bits_to_f32(c.z >> 16);
+    hi.z = f16_bits_to_f32(c.w & 0xFFFFu); hi.w = f16_bits_to_f32(c.w >> 16);
+    reinterpret_cast<f32x4*>(out)[2 * v] = lo;
+    reinterpret_cast<f32x4*>(out)[2 * v + 1] = hi;
+  }
+}
+
+// VL = 8: one 16-byte gather and one vector store per thread.
+template <int BITS, int OUT>
+__global__ void __launch_bounds__(256)
+vq_dequant_vl8_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int bits,
+                      const u32x4* __restrict__ codebook, uint32_t nc, void* __restrict__ out,
+                      int64_t n_vectors) {
+  const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (v >= n_vectors) return;
+  // An index past the codebook is clamped to the last row so a corrupt stream
+  // cannot read outside the table.
+  const uint32_t idx = min(vec_index<BITS>(packed, n_bytes, v, bits), nc - 1u);
+  store8<OUT>(out, v, codebook[idx]);
+}
+
+// Any VL: scalar copy of the codebook row.
+template <int OUT>
+__global__ void __launch_bounds__(256)
+vq_dequant_generic_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int bits,
+                          const uint16_t* __restrict__ codebook, uint32_t nc,
+                          void* __restrict__ out, int64_t n_vectors, int vl) {
+  const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (v >= n_vectors) return;
+  const uint32_t idx = min(read_index(packed, n_bytes, v, bits), nc - 1u);
+  const uint16_t* c = codebook + (int64_t)idx * vl;
+  for (int j = 0; j < vl; ++j) store_from_f16_bits<OUT>(out, v * vl + j, c[j]);
+}
+
+__global__ void __launch_bounds__(256)
+vq_widen_u16_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int bits,
+                    int64_t n_indices, uint16_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_indices) return;
+  out[i] = (uint16_t)read_index(packed, n_bytes, i, bits);
+}
+
+// Residual VQ: three separately rounded fp16 operations per element.
+__device__ __forceinline__ uint32_t rvq_elem(uint32_t cm, uint32_t cr, bool has_s, _Float16 s,
+                                             bool has_b, _Float16 b) {
+  _Float16 h = __builtin_bit_cast(_Float16, (uint16_t)cm) + __builtin_bit_cast(_Float16, (uint16_t)cr);
+  if (has_s) h = h * s;
+  if (has_b) h = h + b;
+  return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(256)
+rvq_dequant_kernel(const uint8_t* __restrict__ pm, int64_t nbm, int bits_m,
+                   const uint8_t* __restrict__ pr, int64_t nbr, int bits_r,
+                   const uint16_t* __restrict__ cbm, uint32_t ncm,
+                   const uint16_t* __restrict__ cbr, uint32_t ncr,
+                   const uint16_t* __restrict__ row_scale, const uint16_t* __restrict__ row_bias,
+                   int vl, int64_t groups, int64_t n_vectors, void* __restrict__ out) {
+  const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (v >= n_vectors) return;
+  const uint32_t im = min(read_index(pm, nbm, v, bits_m), ncm - 1u);
+  const uint32_t ir = min(read_index(pr, nbr, v, bits_r), ncr - 1u);
+  const int64_t n = v / groups;
+  const bool has_s = row_scale != nullptr, has_b = row_bias != nullptr;
+  const _Float16 s = has_s ? __builtin_bit_cast(_Float16, row_scale[n]) : (_Float16)1.0f;
+  const _Float16 b = has_b ? __builtin_bit_cast(_Float16, row_bias[n]) : (_Float16)0.0f;
+  const uint16_t* cm = cbm + (int64_t)im * vl;
+  const uint16_t* cr = cbr + (int64_t)ir * vl;
+  for (int j = 0; j < vl; ++j)
+    store_from_f16_bits<OUT>(out, v * vl + j, rvq_elem(cm[j], cr[j], has_s, s, has_b, b));
+}
+
+template <int OUT>
+static int launch_vq_dequant(const uint8_t* packed, int64_t n_bytes, int bits, const void* cb,
+                             uint32_t nc, int vl, int64_t n_vectors, void* out, hipStream_t st) {
+  const unsigned blocks = (unsigned)((n_vectors + 255) / 256);
+  const bool cb_aligned = (reinterpret_cast<uintptr_t>(cb) % 16) == 0;
+  const bool out_aligned = (reinterpret_cast<uintptr_t>(out) % 16) == 0;
+  if (vl == 8 && cb_aligned && out_aligned) {
+    const u32x4* c = reinterpret_cast<const u32x4*>(cb);
+    if (bits == 16 && (reinterpret_cast<uintptr_t>(packed) % 2) == 0)
+      vq_dequant_vl8_kernel<16, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
+    else if (bits == 8)
+      vq_dequant_vl8_kernel<8, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
+    else
+      vq_dequant_vl8_kernel<0, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
+  } else {
+    vq_dequant_generic_kernel<OUT><<<blocks, 256, 0, st>>>(
+        packed, n_bytes, bits, reinterpret_cast<const uint16_t*>(cb), nc, out, n_vectors, vl);
+  }
+  return check_launch("npamd_vq_dequant");
+}
+
+}  // namespace npamd
+
+using namespace npamd;
+
+extern "C" int npamd_vq_dequant(const uint8_t* packed, int64_t n_bytes, int bits,
+                                const void* codebook_f16, int nc, int vl, int64_t n_vectors,
+                                void* out, int out_dtype, void* stream) {
+  NPAMD_REQUIRE(bits >= 4 && bits <= 20, "npamd_vq_dequant: bits must be in [4, 20], got %d", bits);
+  NPAMD_REQUIRE(vl >= 1 && nc >= 1, "npamd_vq_dequant: bad codebook shape [%d, %d]", nc, vl);
+  NPAMD_REQUIRE(n_vectors >= 0, "npamd_vq_dequant: negative n_vectors");
+  NPAMD_REQUIRE((n_vectors * bits + 7) / 8 <= n_bytes,
+                "npamd_vq_dequant: packed buffer too short for %lld indices of %d bits",
+                (long long)n_vectors, bits);
+  if (n_vectors == 0) return NPAMD_OK;
+  NPAMD_REQUIRE(packed && codebook_f16 && out, "npamd_vq_dequant: null pointer");
+  NPAMD_REQUIRE(n_vectors <= (int64_t)0x7FFFFFFF * 256, "npamd_vq_dequant: too many vectors");
+  hipStream_t st = (hipStream_t)stream;
+  switch (out_dtype) {
+    case NPAMD_F16: return launch_vq_dequant<NPAMD_F16>(packed, n_bytes, bits, codebook_f16, (uint32_t)nc, vl, n_vectors, out, st);
+    case NPAMD_BF16: return launch_vq_dequant<NPAMD_BF16>(packed, n_bytes, bits, codebook_f16, (uint32_t)nc, vl, n_vectors, out, st);
+    case NPAMD_F32: return launch_vq_dequant<NPAMD_F32>(packed, n_bytes, bits, codebook_f16, (uint32_t)nc, vl, n_vectors, out, st);
+  }
+  return fail(NPAMD_ERR_INVALID, "npamd_vq_dequant: out_dtype must be f16, bf16 or f32");
+}
+
+extern "C" int npamd_vq_widen_u16(const uint8_t* packed, int64_t n_bytes, int bits,
+                                  int64_t n_indices, uint16_t* out, void* stream) {
+  NPAMD_REQUIRE(bits >= 4 && bits <= 16, "npamd_vq_widen_u16: bits must be in [4, 16], got %d", bits);
+  NPAMD_REQUIRE(n_indices >= 0 && (n_indices * bits + 7) / 8 <= n_bytes,
+                "npamd_vq_widen_u16: packed buffer too short");
+  if (n_indices == 0) return NPAMD_OK;
+  NPAMD_REQUIRE(packed && out, "npamd_vq_widen_u16: null pointer");
+  const unsigned blocks = (unsigned)((n_indices + 255) / 256);
+  vq_widen_u16_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(packed, n_bytes, bits, n_indices, out);
+  return check_launch("npamd_vq_widen_u16");
+}
+
+extern "C" int npamd_rvq_dequant(const uint8_t* packed_main, int64_t n_bytes_main, int bits_main,
+                                 const uint8_t* packed_res, int64_t n_bytes_res, int bits_res,
+                                 const void* cb_main_f16, int nc_main, const void* cb_res_f16,
+                                 int nc_res, const void* row_scale_f16, const void* row_bias_f16,
+                                 int vl, int N, int K, void* out, int out_dtype, void* stream) {
+  NPAMD_REQUIRE(bits_main >= 4 && bits_main <= 20 && bits_res >= 4 && bits_res <= 20,
+                "npamd_rvq_dequant: bits must be in [4, 20]");
+  NPAMD_REQUIRE(vl >= 1 && nc_main >= 1 && nc_res >= 1, "npamd_rvq_dequant: bad codebook shape");
+  NPAMD_REQUIRE(N >= 0 && K >= 0 && K % vl == 0, "npamd_rvq_dequant: K=%d not divisible by VL=%d", K, vl);
+  const int64_t groups = K / vl, n_vectors = (int64_t)N * groups;
+  NPAMD_REQUIRE((n_vectors * bits_main + 7) / 8 <= n_bytes_main &&
+                    (n_vectors * bits_res + 7) / 8 <= n_bytes_res,
+                "npamd_rvq_dequant: packed buffer too short");
+  if (n_vectors == 0) return NPAMD_OK;
+  NPAMD_REQUIRE(packed_main && packed_res && cb_main_f16 && cb_res_f16 && out,
+                "npamd_rvq_dequant: null pointer");
+  const unsigned blocks = (unsigned)((n_vectors + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+#define NPAMD_RVQ_LAUNCH(OUT)                                                                   \
+  rvq_dequant_kernel<OUT><<<blocks, 256, 0, st>>>(                                              \
+      packed_main, n_bytes_main, bits_main, packed_res, n_bytes_res, bits_res,                  \
+      (const uint16_t*)cb_main_f16, (uint32_t)nc_main, (const uint16_t*)cb_res_f16,             \
+      (uint32_t)nc_res, (const uint16_t*)row_scale_f16, \
+      (const uint16_t*)row_bias_f16, vl, groups, n_vectors, out)
+  switch (out_dtype) {
+    case NPAMD_F16: NPAMD_RVQ_LAUNCH(NPAMD_F16); break;
+    case NPAMD_BF16: NPAMD_RVQ_LAUNCH(NPAMD_BF16); break;
+    case NPAMD_F32: NPAMD_RVQ_LAUNCH(NPAMD_F32); break;
+    default: return fail(NPAMD_ERR_INVALID, "npamd_rvq_dequant: out_dtype must be f16, bf16 or f32");
+  }
+#undef NPAMD_RVQ_LAUNCH
+  return check_launch("npamd_rvq_dequant");
+}

@@ -1,0 +1,86 @@
+// C-ABI entry points of the fused decode GEMV (plain and residual VQ).
+#include "vq_call.hpp"
+
+using namespace npamd;
+
+namespace {
+
+template <int ACT, int BITS>
+int run_vq(const VqCall& c, const GemvShape& s) {
+  if constexpr (ACT == NPAMD_BF16) {
+    if (c.cb_dtype == NPAMD_F16) {
+      using P = VqProvider<ACT, BITS, true>;
+      typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
+      return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+    }
+  }
+  using P = VqProvider<ACT, BITS, false>;
+  typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
+  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+}
+
+template <int ACT>
+int run_vq_bits(const VqCall& c, const GemvShape& s) {
+  switch (c.bits) {
+    case 4: return run_vq<ACT, 4>(c, s);
+    case 8: return run_vq<ACT, 8>(c, s);
+    case 12: return run_vq<ACT, 12>(c, s);
+    default: return run_vq<ACT, 16>(c, s);
+  }
+}
+
+template <int ACT, int BM_, int BR_>
+int run_rvq(const VqCall& c, const GemvShape& s) {
+  using P = RvqProvider<ACT, BM_, BR_>;
+  typename P::Args a{c.packed, c.packed_r, (const u32x4*)c.cb, (const u32x4*)c.cb_r,
+                     (const uint16_t*)c.row_scale, (const uint16_t*)c.row_bias,
+                     (uint32_t)c.nc - 1u, (uint32_t)c.nc_r - 1u, s.chunks};
+  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+}
+
+template <int ACT>
+int dispatch(const VqCall& c) {
+  GemvShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K / 64, 0, 0};
+  if (fast_ok(c)) {
+    if (!c.packed_r) return run_vq_bits<ACT>(c, s);
+    const bool res_ok = aligned(c.packed_r, 16) && aligned(c.cb_r, 16);
+    if (res_ok && c.bits == 16 && c.bits_r == 8) return run_rvq<ACT, 16, 8>(c, s);
+    if (res_ok && c.bits == 16 && c.bits_r == 16) return run_rvq<ACT, 16, 16>(c, s);
+    if (res_ok && c.bits == 12 && c.bits_r == 8) return run_rvq<ACT, 12, 8>(c, s);
+    if (res_ok && c.bits == 8 && c.bits_r == 8) return run_rvq<ACT, 8, 8>(c, s);
+  }
+  return launch_generic_gemv<ACT>(c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, make_elem(c), c.st, c.what);
+}
+
+int run(const VqCall& c) {
+  const int rc = validate(c, NPAMD_GEMV_MAX_M);
+  if (rc < 0) return rc;
+  if (rc == 1) return NPAMD_OK;
+  return c.act == NPAMD_BF16 ? dispatch<NPAMD_BF16>(c) : dispatch<NPAMD_F16>(c);
+}
+
+}  // namespace
+
+extern "C" int npamd_vq_gemv(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_bytes,
+                             int bits, const void* codebook, int codebook_dtype, int nc, int vl,
+                             const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                             int act_dtype, void* stream) {
+  VqCall c{x, ldx, packed, n_bytes, bits, codebook, codebook_dtype, nc, vl,
+               nullptr, 0, 0, nullptr, 0, nullptr, nullptr,
+               bias, y, ldy, M, N, K, act_dtype, (hipStream_t)stream, "npamd_vq_gemv"};
+  return run(c);
+}
+
+extern "C" int npamd_rvq_gemv(const void* x, int64_t ldx,
+                              const uint8_t* packed_main, int64_t n_bytes_main, int bits_main,
+                              const uint8_t* packed_res, int64_t n_bytes_res, int bits_res,
+                              const void* cb_main_f16, int nc_main, const void* cb_res_f16, int nc_res,
+                              const void* row_scale_f16, const void* row_bias_f16, int vl,
+                              const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                              int act_dtype, void* stream) {
+  if (!packed_res) return fail(NPAMD_ERR_INVALID, "npamd_rvq_gemv: residual stream is null");
+  VqCall c{x, ldx, packed_main, n_bytes_main, bits_main, cb_main_f16, NPAMD_F16, nc_main, vl,
+               packed_res, n_bytes_res, bits_res, cb_res_f16, nc_res, row_scale_f16, row_bias_f16,
+               bias, y, ldy, M, N, K, act_dtype, (hipStream_t)stream, "npamd_rvq_gemv"};
+  return run(c);
+}

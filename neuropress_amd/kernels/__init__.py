@@ -1,0 +1,436 @@
+"""Kernel wrappers: torch tensors in, HIP kernels through the C ABI, torch tensors out.
+
+Mirrors the function surface of the reference's ``neuropress.kernels``
+(neuropress/kernels/__init__.py): ``vq_linear`` (:209-216), ``vq_linear_wmma``
+(:335-342), ``vq_dequant`` (:497-504), ``dequantize_vq_weight`` (:248-255),
+``q_linear`` (:109-117), ``unpack_indices`` (:947), ``warn_kernel_fallback``
+(:436-453) -- same names, argument order and error type (``RuntimeError``).
+``vq_gemm_tile`` takes the place of the reference's Triton GEMM
+(neuropress/kernels/vq_triton.py:119-179); ``q_dequant`` / ``q_gemm_tile`` and
+the ``rvq_*`` functions have no reference counterpart.
+
+Every function here launches on torch's current stream, allocates its output
+with torch, and raises if the HIP library is missing: there is no CPU fallback
+at this level (callers that want one catch ``RuntimeError`` and say so through
+:func:`warn_kernel_fallback`).
+"""
+
+from __future__ import annotations
+
+import logging
+
+import torch
+
+from .. import _lib
+
+log = logging.getLogger(__name__)
+
+_DT = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+
+
+def _dt(dtype: torch.dtype, what: str) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise RuntimeError(f"{what}: dtype must be bfloat16, float16 or float32, got {dtype}") from None
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _check_device(what: str, *tensors: torch.Tensor | None) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(f"{what}: all tensors must be on the GPU (got a {t.device} tensor)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"{what}: tensors are on different devices ({dev} vs {t.device})")
+    assert dev is not None
+    return dev
+
+
+def _packed_u8(packed: torch.Tensor, what: str) -> torch.Tensor:
+    if packed.dtype != torch.uint8:
+        raise RuntimeError(f"{what}: packed indices must be uint8, got {packed.dtype}")
+    return packed.contiguous().reshape(-1)
+
+
+def _centroids_f16(centroids: torch.Tensor, what: str) -> torch.Tensor:
+    if centroids.dim() != 2:
+        raise RuntimeError(f"{what}: centroids must be [NC, VL]")
+    return centroids.contiguous()
+
+
+def _bias_f32(bias: torch.Tensor | None) -> torch.Tensor | None:
+    if bias is None:
+        return None
+    return bias.contiguous() if bias.dtype == torch.float32 else bias.to(torch.float32).contiguous()
+
+
+def _x2d(x: torch.Tensor, what: str) -> torch.Tensor:
+    if x.dim() != 2:
+        raise RuntimeError(f"{what}: x must be 2-D [M, K]")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    return x
+
+
+# ---------------------------------------------------------------------------
+# VQ
+# ---------------------------------------------------------------------------
+
+
+def vq_dequant(
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    out_features: int,
+    in_features: int,
+    dtype: torch.dtype,
+) -> torch.Tensor:
+    """Decode a packed VQ weight to a dense ``[out_features, in_features]`` tensor.
+
+    Same contract as the reference's ``vq_dequant`` (neuropress/kernels/__init__.py:497-529,
+    neuropress/kernels/vq_dequant.cu:105-146); the result equals
+    ``centroids[idx].reshape(N, K).to(dtype)`` bit for bit.
+    """
+    what = "vq_dequant"
+    _check_device(what, packed_indices, centroids)
+    packed = _packed_u8(packed_indices, what)
+    cb = _centroids_f16(centroids, what)
+    if cb.dtype != torch.float16:
+        raise RuntimeError(f"{what}: centroids must be float16")
+    vl = cb.shape[1]
+    numel = out_features * in_features
+    if numel % vl:
+        raise RuntimeError(f"{what}: weight size not divisible by VL={vl}")
+    out = torch.empty((out_features, in_features), device=packed.device, dtype=dtype)
+    _lib.call(
+        "npamd_vq_dequant", packed.data_ptr(), packed.numel(), int(bits), cb.data_ptr(),
+        cb.shape[0], vl, numel // vl, out.data_ptr(), _dt(dtype, what), _stream(out),
+    )  # fmt: skip
+    return out
+
+
+def dequantize_vq_weight(
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    vector_len: int,
+    out_features: int,
+    in_features: int,
+) -> torch.Tensor:
+    """fp16 decode (reference: neuropress/kernels/__init__.py:248-283); no tail padding needed."""
+    if centroids.shape[1] != vector_len:
+        raise RuntimeError("dequantize_vq_weight: vector_len does not match the codebook")
+    return vq_dequant(packed_indices, centroids, bits, out_features, in_features, torch.float16)
+
+
+def unpack_indices(packed: torch.Tensor, n_indices: int, bits: int) -> torch.Tensor:
+    """Bit-stream -> int64 indices on the GPU (reference: neuropress/kernels/__init__.py:947)."""
+    return widen_indices_u16(packed, n_indices, bits).view(torch.int16).to(torch.int64) & 0xFFFF
+
+
+def widen_indices_u16(packed: torch.Tensor, n_indices: int, bits: int) -> torch.Tensor:
+    """Bit-stream -> one uint16 per index, returned as a uint8 view (a 16-bit stream)."""
+    what = "widen_indices_u16"
+    _check_device(what, packed)
+    p = _packed_u8(packed, what)
+    out = torch.empty(2 * n_indices, device=p.device, dtype=torch.uint8)
+    _lib.call("npamd_vq_widen_u16", p.data_ptr(), p.numel(), int(bits), int(n_indices),
+              out.data_ptr(), _stream(out))  # fmt: skip
+    return out
+
+
+def _vq_fused(
+    entry: str,
+    x: torch.Tensor,
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    out_features: int | None,
+    bias: torch.Tensor | None,
+) -> torch.Tensor:
+    _check_device(entry, x, packed_indices, centroids, bias)
+    x = _x2d(x, entry)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"{entry}: x must be float16 or bfloat16, got {x.dtype}")
+    packed = _packed_u8(packed_indices, entry)
+    cb = _centroids_f16(centroids, entry)
+    if cb.dtype not in (torch.float16, x.dtype):
+        raise RuntimeError(f"{entry}: centroids must be float16 or x's dtype")
+    m, k = x.shape
+    vl = cb.shape[1]
+    if k % vl:
+        raise RuntimeError(f"{entry}: K={k} not divisible by VL={vl}")
+    groups = k // vl
+    if out_features is None:
+        # N from the stream length, as the reference kernels do (vq_linear_wmma.cu:501-506).
+        total = packed.numel() * 8 // bits
+        if groups == 0 or total % groups:
+            raise RuntimeError(f"{entry}: packed_indices size does not evenly divide into rows")
+        out_features = total // groups
+    y = torch.empty((m, out_features), device=x.device, dtype=x.dtype)
+    b32 = _bias_f32(bias)
+    _lib.call(
+        entry, x.data_ptr(), x.stride(0), packed.data_ptr(), packed.numel(), int(bits),
+        cb.data_ptr(), _DT[cb.dtype], cb.shape[0], vl, _ptr(b32), y.data_ptr(), y.stride(0),
+        m, out_features, k, _DT[x.dtype], _stream(x),
+    )  # fmt: skip
+    return y
+
+
+def vq_linear(
+    x: torch.Tensor,
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    vector_len: int,
+    bias: torch.Tensor | None = None,
+    out_features: int | None = None,
+) -> torch.Tensor:
+    """Fused decode GEMV, ``M <= 16`` (reference: neuropress/kernels/__init__.py:209-245)."""
+    if centroids.dim() == 2 and centroids.shape[1] != vector_len:
+        raise RuntimeError("vq_linear: vector_len does not match the codebook")
+    return _vq_fused("npamd_vq_gemv", x, packed_indices, centroids, bits, out_features, bias)
+
+
+def vq_linear_wmma(
+    x: torch.Tensor,
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    vector_len: int,
+    bias: torch.Tensor | None = None,
+    out_features: int | None = None,
+) -> torch.Tensor:
+    """GEMV/GEMM auto-dispatch on M (reference: neuropress/kernels/__init__.py:335-354).
+
+    ``M <= 16`` runs the fused GEMV, larger M the tile-decode MFMA GEMM.
+    """
+    if centroids.dim() == 2 and centroids.shape[1] != vector_len:
+        raise RuntimeError("vq_linear_wmma: vector_len does not match the codebook")
+    entry = "npamd_vq_gemv" if x.shape[0] <= _lib.GEMV_MAX_M else "npamd_vq_gemm_tile"
+    return _vq_fused(entry, x, packed_indices, centroids, bits, out_features, bias)
+
+
+def vq_gemm_tile(
+    x: torch.Tensor,
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    out_features: int,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``x @ W.T (+ bias)`` with W decoded tile by tile inside an MFMA GEMM.
+
+    Signature of the reference's ``vq_gemm_triton`` (neuropress/kernels/vq_triton.py:119-126).
+    """
+    return _vq_fused("npamd_vq_gemm_tile", x, packed_indices, centroids, bits, out_features, bias)
+
+
+# ---------------------------------------------------------------------------
+# Residual VQ (two codebooks, per-row scale / bias)
+# ---------------------------------------------------------------------------
+
+
+def _f16_or_none(t: torch.Tensor | None, what: str) -> torch.Tensor | None:
+    if t is None:
+        return None
+    if t.dtype != torch.float16:
+        raise RuntimeError(f"{what}: per-row scale / bias must be float16")
+    return t.contiguous()
+
+
+def rvq_dequant(
+    packed_main: torch.Tensor,
+    bits_main: int,
+    packed_res: torch.Tensor,
+    bits_res: int,
+    centroids_main: torch.Tensor,
+    centroids_res: torch.Tensor,
+    row_scale: torch.Tensor | None,
+    row_bias: torch.Tensor | None,
+    out_features: int,
+    in_features: int,
+    dtype: torch.dtype,
+) -> torch.Tensor:
+    what = "rvq_dequant"
+    _check_device(what, packed_main, packed_res, centroids_main, centroids_res, row_scale, row_bias)
+    pm, pr = _packed_u8(packed_main, what), _packed_u8(packed_res, what)
+    cm, cr = _centroids_f16(centroids_main, what), _centroids_f16(centroids_res, what)
+    if cm.dtype != torch.float16 or cr.dtype != torch.float16 or cm.shape[1] != cr.shape[1]:
+        raise RuntimeError(f"{what}: codebooks must be float16 with the same vector length")
+    sc, rb = _f16_or_none(row_scale, what), _f16_or_none(row_bias, what)
+    out = torch.empty((out_features, in_features), device=pm.device, dtype=dtype)
+    _lib.call(
+        "npamd_rvq_dequant", pm.data_ptr(), pm.numel(), int(bits_main), pr.data_ptr(), pr.numel(),
+        int(bits_res), cm.data_ptr(), cm.shape[0], cr.data_ptr(), cr.shape[0], _ptr(sc), _ptr(rb),
+        cm.shape[1], out_features, in_features, out.data_ptr(), _dt(dtype, what), _stream(out),
+    )  # fmt: skip
+    return out
+
+
+def rvq_linear(
+    x: torch.Tensor,
+    packed_main: torch.Tensor,
+    bits_main: int,
+    packed_res: torch.Tensor,
+    bits_res: int,
+    centroids_main: torch.Tensor,
+    centroids_res: torch.Tensor,
+    row_scale: torch.Tensor | None,
+    row_bias: torch.Tensor | None,
+    out_features: int,
+    bias: torch.Tensor | None = None,
+    tile: bool | None = None,
+) -> torch.Tensor:
+    """Fused residual-VQ linear; ``tile=None`` picks GEMV for ``M <= 16`` else the tile GEMM."""
+    what = "rvq_linear"
+    _check_device(what, x, packed_main, packed_res, centroids_main, centroids_res)
+    x = _x2d(x, what)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"{what}: x must be float16 or bfloat16, got {x.dtype}")
+    pm, pr = _packed_u8(packed_main, what), _packed_u8(packed_res, what)
+    cm, cr = _centroids_f16(centroids_main, what), _centroids_f16(centroids_res, what)
+    if cm.dtype != torch.float16 or cr.dtype != torch.float16 or cm.shape[1] != cr.shape[1]:
+        raise RuntimeError(f"{what}: codebooks must be float16 with the same vector length")
+    sc, rb = _f16_or_none(row_scale, what), _f16_or_none(row_bias, what)
+    m, k = x.shape
+    if tile is None:
+        tile = m > _lib.GEMV_MAX_M
+    y = torch.empty((m, out_features), device=x.device, dtype=x.dtype)
+    b32 = _bias_f32(bias)
+    _lib.call(
+        "npamd_rvq_gemm_tile" if tile else "npamd_rvq_gemv",
+        x.data_ptr(), x.stride(0), pm.data_ptr(), pm.numel(), int(bits_main), pr.data_ptr(),
+        pr.numel(), int(bits_res), cm.data_ptr(), cm.shape[0], cr.data_ptr(), cr.shape[0],
+        _ptr(sc), _ptr(rb), cm.shape[1], _ptr(b32), y.data_ptr(), y.stride(0), m, out_features, k,
+        _DT[x.dtype], _stream(x),
+    )  # fmt: skip
+    return y
+
+
+# ---------------------------------------------------------------------------
+# Group-affine n-bit
+# ---------------------------------------------------------------------------
+
+
+def _q_args(what, w_pack, scale, zero_point, nbits, group_size):
+    if w_pack.dtype != torch.uint8 or w_pack.dim() != 2:
+        raise RuntimeError(f"{what}: w_pack must be a 2-D uint8 tensor [N, K/vpb]")
+    if scale.dtype != torch.float16:
+        raise RuntimeError(f"{what}: scale must be float16")
+    if zero_point is not None and zero_point.dtype != torch.float16:
+        raise RuntimeError(f"{what}: zero_point must be float16")
+    if nbits not in (1, 2, 4, 8):
+        raise RuntimeError(f"{what}: nbits must be one of {{1, 2, 4, 8}}, got {nbits}")
+    n = w_pack.shape[0]
+    k = w_pack.shape[1] * (8 // nbits)
+    if group_size <= 0 or k % group_size:
+        raise RuntimeError(f"{what}: K={k} not divisible by group_size={group_size}")
+    sc = scale.contiguous().reshape(-1)
+    if sc.numel() != n * (k // group_size):
+        raise RuntimeError(f"{what}: scale has {sc.numel()} entries, expected {n * (k // group_size)}")
+    zp = None
+    if zero_point is not None:
+        zp = zero_point.contiguous().reshape(-1)
+        if zp.numel() != sc.numel():
+            raise RuntimeError(f"{what}: zero_point must have the same number of entries as scale")
+    return w_pack.contiguous(), sc, zp, n, k
+
+
+def q_dequant(
+    w_pack: torch.Tensor,
+    scale: torch.Tensor,
+    nbits: int,
+    group_size: int,
+    zero_point: torch.Tensor | None = None,
+    dtype: torch.dtype = torch.float16,
+) -> torch.Tensor:
+    """Decode ``[N, K/vpb]`` packed codes to a dense ``[N, K]`` weight of *dtype*."""
+    what = "q_dequant"
+    _check_device(what, w_pack, scale, zero_point)
+    wp, sc, zp, n, k = _q_args(what, w_pack, scale, zero_point, nbits, group_size)
+    out = torch.empty((n, k), device=wp.device, dtype=dtype)
+    _lib.call("npamd_q_dequant", wp.data_ptr(), sc.data_ptr(), _ptr(zp), n, k, int(nbits),
+              int(group_size), out.data_ptr(), _dt(dtype, what), _stream(out))  # fmt: skip
+    return out
+
+
+def _q_fused(entry, x, w_pack, scale, nbits, group_size, zero_point, bias):
+    _check_device(entry, x, w_pack, scale, zero_point, bias)
+    wp, sc, zp, n, k = _q_args(entry, w_pack, scale, zero_point, nbits, group_size)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"{entry}: x must be float16 or bfloat16, got {x.dtype}")
+    if x.shape[-1] != k:
+        raise RuntimeError(f"{entry}: x has K={x.shape[-1]}, the packed weight has K={k}")
+    lead = x.shape[:-1]
+    x2 = _x2d(x.reshape(-1, k), entry)
+    m = x2.shape[0]
+    y = torch.empty((m, n), device=x.device, dtype=x.dtype)
+    b32 = _bias_f32(bias)
+    _lib.call(entry, x2.data_ptr(), x2.stride(0), wp.data_ptr(), sc.data_ptr(), _ptr(zp), _ptr(b32),
+              y.data_ptr(), y.stride(0), m, n, k, int(nbits), int(group_size), _DT[x.dtype],
+              _stream(x))  # fmt: skip
+    return y.reshape(*lead, n)
+
+
+def q_linear(
+    x: torch.Tensor,
+    w_pack: torch.Tensor,
+    scale: torch.Tensor,
+    nbits: int,
+    group_size: int,
+    zero_point: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Fused group-quantized dequant + linear (reference: neuropress/kernels/__init__.py:109-151).
+
+    ``M <= 16`` runs the fused GEMV, larger M the fused MFMA GEMM; the reference
+    runs its GEMV at every M (neuropress/kernels/q4_linear.cu:137-139).
+    """
+    m = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    entry = "npamd_q_gemv" if m <= _lib.GEMV_MAX_M else "npamd_q_gemm_tile"
+    return _q_fused(entry, x, w_pack, scale, nbits, group_size, zero_point, bias)
+
+
+def q_gemm_tile(x, w_pack, scale, nbits, group_size, zero_point=None, bias=None) -> torch.Tensor:
+    """Fused dequant MFMA GEMM at any M."""
+    return _q_fused("npamd_q_gemm_tile", x, w_pack, scale, nbits, group_size, zero_point, bias)
+
+
+# ---------------------------------------------------------------------------
+# Fallback reporting
+# ---------------------------------------------------------------------------
+
+_warned_fallbacks: set[str] = set()
+
+
+def warn_kernel_fallback(kernel: str, fallback: str, exc: BaseException) -> None:
+    """Warn once per *kernel* that it is unavailable and *fallback* runs instead.
+
+    Same behaviour as the reference (neuropress/kernels/__init__.py:436-453):
+    one WARNING per kernel name carrying the cause and the fix; later calls for
+    the same kernel are silent.
+    """
+    if kernel in _warned_fallbacks:
+        return
+    _warned_fallbacks.add(kernel)
+    log.warning(
+        "HIP kernel %s unavailable (%s); using %s instead, which can be much slower. "
+        "Build the library with `python -m neuropress_amd.build` (needs hipcc from ROCm) "
+        "and run on a gfx950 GPU.",
+        kernel,
+        exc,
+        fallback,
+    )

@@ -1,0 +1,108 @@
+"""Backend enumerations for the quantized inference modules.
+
+String values are the reference's (neuropress/nn/backends.py:102-159) so that
+recipes, YAML lowering configs and saved checkpoints keep working.  The names
+that say "cuda" select the HIP kernels of this package:
+
+===================  =========================================================
+``cuda`` / ``cuda_wmma``  fused decode GEMV -> tile-decode MFMA GEMM -> decode + GEMM,
+                          by token count
+``cuda_lut``              decode + GEMM at every token count unless the LUT
+                          threshold is raised (the routing the reference gives
+                          large-codebook layers)
+``compile`` / ``default`` gather + ``F.linear`` with torch ops (CPU or GPU)
+===================  =========================================================
+
+``is_cuda_jit_available`` keeps its name; here it answers "can the HIP kernel
+library run": the shared object loads and a GPU is visible.
+"""
+
+from __future__ import annotations
+
+import enum
+import logging
+import os
+
+_log = logging.getLogger(__name__)
+
+_hip_ok: bool | None = None
+
+
+def is_hip_backend_available() -> bool:
+    """True when ``libnpamd.so`` loads and torch sees a GPU.  Cached.
+
+    ``NEUROPRESS_FORCE_CUDA_JIT=1`` skips the probe and answers True, as the
+    reference's switch of the same name does (neuropress/nn/backends.py:40).
+    """
+    global _hip_ok
+    if _hip_ok is not None:
+        return _hip_ok
+    if os.environ.get("NEUROPRESS_FORCE_CUDA_JIT", "").strip() in ("1", "true", "yes"):
+        _hip_ok = True
+        return True
+    import torch
+
+    from .. import _lib
+
+    if not torch.cuda.is_available():
+        _hip_ok = False
+        return False
+    _hip_ok = _lib.is_available()
+    if not _hip_ok:
+        _log.warning(
+            "libnpamd.so could not be loaded; HIP backends disabled, falling back to torch ops"
+        )
+    return _hip_ok
+
+
+# Name kept for drop-in compatibility with code written against the reference.
+is_cuda_jit_available = is_hip_backend_available
+
+
+class _StrEnum(str, enum.Enum):
+    """``enum.StrEnum`` for Python < 3.11: members compare and format as their value."""
+
+    def __str__(self) -> str:
+        return str(self.value)
+
+    def __format__(self, spec: str) -> str:
+        return format(str(self.value), spec)
+
+
+class LinearBackend(_StrEnum):
+    """Valid backends for scalar-quantized ``nn.Linear`` (:class:`.NPLinear`)."""
+
+    AUTO = "auto"
+    DEFAULT = "default"
+    COMPILE = "compile"
+    CUDA = "cuda"
+    GEMLITE = "gemlite"
+
+
+class VQBackend(_StrEnum):
+    """Valid backends for vector-quantized ``nn.Linear`` (:class:`.NPVQLinear`)."""
+
+    AUTO = "auto"
+    DEFAULT = "default"
+    COMPILE = "compile"
+    CUDA = "cuda"
+    CUDA_WMMA = "cuda_wmma"
+    CUDA_LUT = "cuda_lut"
+    CUDA_TIERED = "cuda_tiered"
+    CUDA_NTIER = "cuda_ntier"
+    CUDA_ZERO_ESCAPE = "cuda_zero_escape"
+
+
+class Backend(_StrEnum):
+    """Superset enum kept for backward compatibility."""
+
+    DEFAULT = "default"
+    COMPILE = "compile"
+    CUDA = "cuda"
+    CUDA_WMMA = "cuda_wmma"
+    CUDA_LUT = "cuda_lut"
+    CUDA_TIERED = "cuda_tiered"
+    CUDA_NTIER = "cuda_ntier"
+    CUDA_ZERO_ESCAPE = "cuda_zero_escape"
+    GEMLITE = "gemlite"
+    AUTO = "auto"

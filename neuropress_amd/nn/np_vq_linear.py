@@ -1,0 +1,686 @@
+"""NPVQLinear: drop-in ``nn.Linear`` replacement with a VQ-compressed weight.
+
+The weight is a packed stream of codebook indices plus a codebook shared
+through a :class:`VQProxy`:
+
+    ``W[n, g*VL + v] = centroids[idx[n * n_groups + g], v]``
+
+Same module surface as the reference (neuropress/nn/np_vq_linear.py:399-1517):
+``VQProxy``, ``NPVQLinear(proxy, packed_indices, bits, out_features, in_features,
+vector_len, backend, bias, column_perm, ...)``, ``from_qtensor_linear``,
+``to_qtensor``, ``forward``, ``linearize_vq_weights``.  What differs is what runs
+underneath: hand-written gfx950 kernels instead of CUDA/Triton, selected by
+token count ``m = x.numel() // in_features``:
+
+====================  ==============================  ==========================
+band                  condition                        kernel
+====================  ==============================  ==========================
+(a) fused GEMV        ``m <= _FUSED_MAX_TOKENS``       ``kernels.vq_linear``
+(b) tile-decode GEMM  ``m <= _TILE_MAX_TOKENS``        ``kernels.vq_gemm_tile``
+(c) decode + GEMM     otherwise                        ``kernels.vq_dequant`` + ``F.linear``
+====================  ==============================  ==========================
+
+The dispatch rule itself is the reference's (np_vq_linear.py:1014-1058); the
+thresholds are re-derived for one MI355X and stay overridable through the same
+environment variables.  Entropy-coded index formats (tiered / n-tier /
+zero-escape) are not supported and are rejected at construction.
+"""
+
+from __future__ import annotations
+
+import logging
+import os
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from ..qweights import VQScheme, VQWeight, is_vq_weight
+from ..transforms.vq_packing import IndexPacking
+from .backends import Backend, VQBackend, is_hip_backend_available
+
+log = logging.getLogger(__name__)
+
+
+def _env_int(names: tuple[str, ...], default: int) -> int:
+    for name in names:
+        v = os.environ.get(name)
+        if v is not None and v.strip():
+            return int(v)
+    return default
+
+
+# Token-count bands (tokens = rows of the flattened input), read once at import
+# like the reference's (np_vq_linear.py:73-87).  The fused GEMV issues the
+# contraction as 16-row MFMA tiles, so 1..16 tokens cost the same: the fused
+# band ends at 16 here (2 in the reference, whose GEMV re-reads the weight per token).
+_FUSED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_FUSED_MAX_TOKENS",), 16)
+
+# cuda_lut layers: 0 = always decode + GEMM, the reference's default routing.
+_LUT_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_LUT_MAX_TOKENS",), 0)
+
+# Upper end of the tile-decode GEMM band.  NEUROPRESS_VQ_TRITON_MAX_TOKENS is the
+# reference's name for the same knob and is honoured too.  0 disables the band.
+_TILE_MAX_TOKENS: int = _env_int(
+    ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 1024
+)
+
+# Opt-in: when a HIP kernel call fails, warn once and run torch ops instead (the
+# reference's behaviour).  Off by default so a missing or broken kernel library
+# is an error, not a silent slow path.
+_ALLOW_FALLBACK: bool = os.environ.get("NEUROPRESS_ALLOW_KERNEL_FALLBACK", "").strip() in (
+    "1", "true", "yes",
+)  # fmt: skip
+
+_FUSED_BACKENDS = frozenset({VQBackend.CUDA_WMMA, VQBackend.CUDA_LUT, VQBackend.CUDA})
+_UNSUPPORTED_BACKENDS = frozenset(
+    {VQBackend.CUDA_TIERED, VQBackend.CUDA_NTIER, VQBackend.CUDA_ZERO_ESCAPE}
+)
+
+# Latched once the tile GEMM fails with fallback allowed, so later calls go
+# straight to decode + GEMM (reference: np_vq_linear.py:91-93).
+_tile_failed: bool = False
+
+# Index widths the fast kernels stream directly; other widths are widened to
+# 16 bits once, on first GPU use.
+_FAST_BITS = frozenset({4, 8, 12, 16})
+
+
+def _fused_max_tokens(backend: VQBackend) -> int:
+    """Largest token count for which *backend*'s fused kernel is used."""
+    return _LUT_MAX_TOKENS if backend == VQBackend.CUDA_LUT else _FUSED_MAX_TOKENS
+
+
+def _resolve_vq_backend(
+    backend: str | VQBackend | Backend | None,
+    use_tiered: bool = False,
+    use_ntier: bool = False,
+    use_zero_escape: bool = False,
+    bits: int = 8,
+    out_features: int = 0,
+    num_centroids: int = 0,
+    vector_len: int = 8,
+) -> VQBackend:
+    """Resolve a backend alias to a concrete :class:`VQBackend` (never ``AUTO``).
+
+    Signature and alias handling follow the reference
+    (neuropress/nn/np_vq_linear.py:101-170): ``None`` / ``"torch"`` ->
+    ``DEFAULT``, unknown strings raise ``ValueError``.  ``"auto"`` on a machine
+    where the HIP library can run resolves to ``CUDA_WMMA`` -- the three-band
+    path -- for every codebook size and vector length: the reference's detours
+    (vector_len != 4 -> COMPILE, bits > 12 -> CUDA_LUT) exist because its
+    tensor-core kernels are fixed to VL = 4 and a 4096-entry shared-memory
+    codebook; the kernels here have neither limit.  Without a GPU ``"auto"``
+    resolves to ``COMPILE`` as in the reference.
+    """
+    if backend is None or backend == "torch":
+        return VQBackend.DEFAULT
+    if isinstance(backend, (VQBackend, Backend)):
+        val = backend.value
+    elif isinstance(backend, str):
+        val = backend
+    else:
+        val = str(backend)
+    if val != "auto":
+        return VQBackend(val)  # raises ValueError for unknown strings
+    if use_tiered or use_ntier or use_zero_escape:
+        return VQBackend.COMPILE
+    if torch.cuda.is_available() and is_hip_backend_available():
+        return VQBackend.CUDA_WMMA
+    return VQBackend.COMPILE
+
+
+def _vq_dequant_linear(
+    x: torch.Tensor,
+    packed_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    bits: int,
+    n_vectors: int,
+    out_features: int,
+    in_features: int,
+    bias: torch.Tensor | None,
+) -> torch.Tensor:
+    """Unpack, gather, ``F.linear`` with torch ops: the specification of the layer.
+
+    Follows neuropress/nn/np_vq_linear.py:178-211.  Runs on whatever device the
+    buffers live on; used by the ``default`` / ``compile`` backends.
+    """
+    indices = IndexPacking.unpack(packed_indices, bits, n_vectors)
+    w = centroids[indices].reshape(out_features, in_features)
+    return F.linear(x, w.to(x.dtype), bias)
+
+
+# ---------------------------------------------------------------------------
+# VQProxy — shared codebook
+# ---------------------------------------------------------------------------
+
+
+class VQProxy(nn.Module):
+    """Shared VQ codebook holder (reference: neuropress/nn/np_vq_linear.py:399-455).
+
+    Holds ``centroids`` ``[num_centroids, vector_len]`` as a float16 buffer.
+    One instance is shared by every :class:`NPVQLinear` of a quantization group
+    and is registered on the model root, not on each layer.
+    """
+
+    centroids: torch.Tensor
+
+    def __init__(self, centroids: torch.Tensor) -> None:
+        super().__init__()
+        self.register_buffer("centroids", centroids.to(torch.float16))
+        self._cast_cache: dict = {}
+
+    @property
+    def num_centroids(self) -> int:
+        return self.centroids.shape[0]
+
+    @property
+    def vector_len(self) -> int:
+        return self.centroids.shape[1]
+
+    def centroids_as(self, dtype: torch.dtype) -> torch.Tensor:
+        """The codebook cast to *dtype*, cached until the buffer moves or changes.
+
+        A bf16 model multiplies by bf16-rounded codebook rows (that is what
+        ``W.to(x.dtype)`` means); casting the table once keeps that conversion
+        out of the kernels' inner loops.
+        """
+        c = self.centroids
+        if dtype == c.dtype:
+            return c
+        key = (dtype, c.device, c.data_ptr(), c._version)
+        hit = self._cast_cache.get("entry")
+        if hit is None or hit[0] != key:
+            hit = (key, c.to(dtype).contiguous())
+            self._cast_cache["entry"] = hit
+        return hit[1]
+
+    def extra_repr(self) -> str:
+        return f"num_centroids={self.num_centroids}, vector_len={self.vector_len}"
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise RuntimeError(
+            "VQProxy.forward() should not be called.  Access centroids "
+            "directly via self.proxy.centroids."
+        )
+
+
+# ---------------------------------------------------------------------------
+# NPVQLinear
+# ---------------------------------------------------------------------------
+
+
+class NPVQLinear(nn.Module):
+    """Linear layer with a VQ-compressed weight and a shared codebook proxy.
+
+    Constructor arguments up to ``column_perm`` are the reference's
+    (neuropress/nn/np_vq_linear.py:493-513).  The entropy-coded-format arguments
+    are accepted for signature compatibility and rejected when set.  The
+    ``residual_*`` / ``row_*`` arguments add an optional residual codebook and
+    a per-output-row fp16 scale and bias on the decoded weight:
+
+        ``W[n, :] = ((Cm[im] + Cr[ir]) * row_scale[n]) + row_bias[n]``
+
+    each operation rounded to fp16 (BASELINE config 4; not in the reference).
+    """
+
+    def __init__(
+        self,
+        proxy: VQProxy,
+        packed_indices: torch.Tensor,
+        bits: int,
+        out_features: int,
+        in_features: int,
+        vector_len: int,
+        backend: str | VQBackend | None,
+        bias: torch.Tensor | None = None,
+        column_perm: torch.Tensor | None = None,
+        use_tiered: bool = False,
+        cold_bits: int = 8,
+        hot_row_offsets: torch.Tensor | None = None,
+        cold_row_offsets: torch.Tensor | None = None,
+        qtensor_meta: dict[str, str] | None = None,
+        tier_bits: list[int] | None = None,
+        ntier_row_offsets: list[torch.Tensor] | None = None,
+        zero_escape: bool = False,
+        zesc_row_offsets: list[torch.Tensor] | None = None,
+        residual_proxy: VQProxy | None = None,
+        packed_residual: torch.Tensor | None = None,
+        residual_bits: int = 0,
+        row_scale: torch.Tensor | None = None,
+        row_bias: torch.Tensor | None = None,
+    ) -> None:
+        super().__init__()
+        if use_tiered or tier_bits is not None or zero_escape:
+            raise NotImplementedError(
+                "NPVQLinear: entropy-coded index formats (tiered / n-tier / zero-escape) "
+                "are not supported by this backend; use fixed-width IndexPacking."
+            )
+        if in_features % vector_len:
+            raise ValueError(f"in_features={in_features} not divisible by vector_len={vector_len}")
+        if proxy.vector_len != vector_len:
+            raise ValueError(f"vector_len={vector_len} does not match the codebook ({proxy.vector_len})")
+        self._qtensor_meta = qtensor_meta
+        self.out_features = out_features
+        self.in_features = in_features
+        self.vector_len = vector_len
+        self.bits = bits
+        self.n_vectors = out_features * (in_features // vector_len)
+        self.use_tiered = False
+        self.cold_bits = cold_bits
+        self.tier_bits = None
+        self.zero_escape = False
+        self.backend = _resolve_vq_backend(
+            backend,
+            bits=bits,
+            out_features=out_features,
+            num_centroids=proxy.num_centroids,
+            vector_len=vector_len,
+        )
+        if self.backend in _UNSUPPORTED_BACKENDS:
+            raise NotImplementedError(f"backend {self.backend.value!r} is not supported")
+        need = IndexPacking.packed_nbytes(self.n_vectors, bits)
+        if packed_indices.numel() < need:
+            raise ValueError(
+                f"packed_indices holds {packed_indices.numel()} bytes, {need} needed for "
+                f"{self.n_vectors} indices of {bits} bits"
+            )
+
+        # The proxy is a plain attribute, not a sub-module: it must not appear
+        # once per layer in state_dict (reference: np_vq_linear.py:588-590).
+        object.__setattr__(self, "proxy", proxy)
+        object.__setattr__(self, "residual_proxy", residual_proxy)
+
+        self.register_buffer("packed_indices", packed_indices.contiguous())
+        self._register_optional("bias", bias)
+        self._register_optional(
+            "column_perm", None if column_perm is None else column_perm.to(torch.int64)
+        )
+        self.residual_bits = residual_bits
+        if residual_proxy is not None:
+            if packed_residual is None:
+                raise ValueError("residual_proxy given without packed_residual")
+            if residual_proxy.vector_len != vector_len:
+                raise ValueError("residual codebook must have the same vector length")
+            self.residual_bits = residual_bits or IndexPacking.bits_for(residual_proxy.num_centroids)
+        self._register_optional("packed_residual", packed_residual)
+        self._register_optional("row_scale", None if row_scale is None else row_scale.to(torch.float16))
+        self._register_optional("row_bias", None if row_bias is None else row_bias.to(torch.float16))
+        # Derived, rebuilt on demand: f32 bias for the kernels, widened index stream.
+        self._derived: dict = {}
+
+    def _register_optional(self, name: str, t: torch.Tensor | None) -> None:
+        if t is not None:
+            self.register_buffer(name, t.contiguous())
+        else:
+            setattr(self, name, None)
+
+    def _apply(self, fn, recurse: bool = True):
+        result = super()._apply(fn, recurse)
+        self._derived = {}
+        return result
+
+    # ------------------------------------------------------------------
+    # Factory / inverse
+    # ------------------------------------------------------------------
+
+    @classmethod
+    def from_qtensor_linear(
+        cls,
+        linear: nn.Linear,
+        proxy: VQProxy,
+        backend: str | VQBackend | None = VQBackend.AUTO,
+        residual_proxy: VQProxy | None = None,
+    ) -> NPVQLinear:
+        """Build from an ``nn.Linear`` whose ``weight`` is a VQ weight.
+
+        Follows neuropress/nn/np_vq_linear.py:831-921.  Raises ``TypeError``
+        (message naming ``QTensorTractVQ``, as the reference does) when the
+        weight is not vector-quantized.
+        """
+        weight_q = linear.weight
+        if not is_vq_weight(weight_q):
+            raise TypeError(
+                f"Expected a VQ weight (QTensorTractVQ / VQWeight), got {type(weight_q).__name__!r}."
+            )
+        qs = weight_q.qscheme
+        bias = linear.bias.detach().clone() if linear.bias is not None else None
+        perm = getattr(qs, "column_permutation", None)
+        res_c = getattr(qs, "residual_centroids", None)
+        if res_c is not None and residual_proxy is None:
+            residual_proxy = VQProxy(res_c)
+        row_scale = getattr(qs, "row_scale", None)
+        row_bias = getattr(qs, "row_bias", None)
+        return cls(
+            proxy=proxy,
+            packed_indices=weight_q.u8_blob.detach().clone(),
+            bits=qs.is_packed_indices,
+            out_features=linear.out_features,
+            in_features=linear.in_features,
+            vector_len=qs.vector_len,
+            backend=backend,
+            bias=bias,
+            column_perm=perm.detach().clone() if perm is not None else None,
+            use_tiered=bool(getattr(qs, "use_tiered", False)),
+            tier_bits=getattr(qs, "tier_bits", None),
+            zero_escape=bool(getattr(qs, "zero_escape", False)),
+            qtensor_meta={"original_shape": tuple(getattr(qs, "original_shape", ()))},
+            residual_proxy=residual_proxy,
+            packed_residual=getattr(weight_q, "residual_blob", None),
+            residual_bits=getattr(qs, "residual_bits", 0),
+            row_scale=row_scale,
+            row_bias=row_bias,
+        )
+
+    def to_qtensor(self) -> VQWeight:
+        """Rebuild the VQ weight this module was lowered from (for unlowering / saving).
+
+        Same contract as neuropress/nn/np_vq_linear.py:977-1008: raises
+        ``RuntimeError`` when the module was not built by :meth:`from_qtensor_linear`.
+        """
+        if self._qtensor_meta is None:
+            raise RuntimeError(
+                "Cannot reconstruct QTensor: no serde metadata stored. "
+                "Build via NPVQLinear.from_qtensor_linear() to enable to_qtensor()."
+            )
+        scheme = VQScheme(
+            centroids=self.proxy.centroids,
+            original_shape=(self.out_features, self.in_features),
+            is_packed_indices=self.bits,
+            column_permutation=self.column_perm,
+            residual_centroids=None if self.residual_proxy is None else self.residual_proxy.centroids,
+            residual_bits=self.residual_bits,
+            row_scale=self.row_scale,
+            row_bias=self.row_bias,
+        )
+        return VQWeight(self.packed_indices, scheme, self.packed_residual)
+
+    # ------------------------------------------------------------------
+    # Derived buffers
+    # ------------------------------------------------------------------
+
+    @property
+    def is_residual(self) -> bool:
+        return self.residual_proxy is not None or self.row_scale is not None or self.row_bias is not None
+
+    def _bias_f32(self) -> torch.Tensor | None:
+        if self.bias is None:
+            return None
+        b = self._derived.get("bias_f32")
+        if b is None or b.device != self.bias.device:
+            b = self.bias.detach().to(torch.float32).contiguous()
+            self._derived["bias_f32"] = b
+        return b
+
+    def _kernel_stream(self) -> tuple[torch.Tensor, int]:
+        """Index stream and width the fused kernels read.
+
+        Widths outside {4, 8, 12, 16} are widened to a 16-bit stream once per
+        device so they take the vectorised index loads (precedent: the
+        reference re-lays index streams out at construction, np_vq_linear.py:644-696).
+        """
+        if self.bits in _FAST_BITS or self.bits > 16:
+            return self.packed_indices, self.bits
+        wide = self._derived.get("wide")
+        if wide is None or wide.device != self.packed_indices.device:
+            from .. import kernels
+
+            wide = kernels.widen_indices_u16(self.packed_indices, self.n_vectors, self.bits)
+            self._derived["wide"] = wide
+        return wide, 16
+
+    # ------------------------------------------------------------------
+    # Forward
+    # ------------------------------------------------------------------
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """Band dispatch by token count (reference: neuropress/nn/np_vq_linear.py:1014-1058)."""
+        if self.column_perm is not None:
+            x = x[..., self.column_perm]
+        if self.backend in _FUSED_BACKENDS:
+            if x.dtype not in (torch.float16, torch.bfloat16):
+                return self._forward_dequant_gemm(x)  # fp32 activations: decode + GEMM
+            m = x.numel() // self.in_features
+            if m > _fused_max_tokens(self.backend):
+                if self.backend != VQBackend.CUDA_LUT and m <= _TILE_MAX_TOKENS:
+                    return self._forward_tile_gemm(x)
+                return self._forward_dequant_gemm(x)
+        if self.backend == VQBackend.CUDA_LUT:
+            return self._forward_cuda_lut(x)
+        if self.backend == VQBackend.CUDA_WMMA:
+            return self._forward_cuda_wmma(x)
+        if self.backend == VQBackend.CUDA:
+            return self._forward_cuda(x)
+        if self.backend == VQBackend.COMPILE:
+            return self._forward_compile(x)
+        return self._forward_default(x)
+
+    # -- torch-op paths ---------------------------------------------------
+
+    def _dense_weight_torch(self, dtype: torch.dtype) -> torch.Tensor:
+        idx = IndexPacking.unpack(self.packed_indices, self.bits, self.n_vectors)
+        w = self.proxy.centroids[idx]
+        if self.is_residual:
+            if self.residual_proxy is not None:
+                ir = IndexPacking.unpack(self.packed_residual, self.residual_bits, self.n_vectors)
+                w = w + self.residual_proxy.centroids[ir]
+            w = w.reshape(self.out_features, self.in_features)
+            if self.row_scale is not None:
+                w = w * self.row_scale[:, None]
+            if self.row_bias is not None:
+                w = w + self.row_bias[:, None]
+        return w.reshape(self.out_features, self.in_features).to(dtype)
+
+    def _forward_default(self, x: torch.Tensor) -> torch.Tensor:
+        """Follows neuropress/nn/np_vq_linear.py:1091-1095."""
+        if self.is_residual:
+            return F.linear(x, self._dense_weight_torch(x.dtype), self.bias)
+        return _vq_dequant_linear(
+            x, self.packed_indices, self.proxy.centroids, self.bits, self.n_vectors,
+            self.out_features, self.in_features, self.bias,
+        )  # fmt: skip
+
+    def _forward_compile(self, x: torch.Tensor) -> torch.Tensor:
+        """The reference compiles the gather path with a tracing compiler
+        (np_vq_linear.py:1150-1160); here the same ops run eagerly."""
+        return self._forward_default(x)
+
+    # -- HIP paths --------------------------------------------------------
+
+    def _fallback(self, kernel: str, fallback: str, exc: Exception) -> None:
+        """Re-raise unless fallbacks were opted into; then warn once per kernel."""
+        if not _ALLOW_FALLBACK:
+            raise exc
+        from .. import kernels
+
+        kernels.warn_kernel_fallback(kernel, fallback, exc)
+
+    def _forward_dequant_gemm(self, x: torch.Tensor) -> torch.Tensor:
+        """Band (c): decode the weight in one kernel pass, then a dense GEMM.
+
+        Follows neuropress/nn/np_vq_linear.py:1127-1148.  The decoded ``[N, K]``
+        weight is a temporary returned to the allocator after the matmul.
+        """
+        from .. import kernels
+
+        try:
+            if self.is_residual:
+                w = kernels.rvq_dequant(
+                    self.packed_indices, self.bits, self._res_stream(), self._res_bits(),
+                    self.proxy.centroids, self._res_centroids(), self.row_scale, self.row_bias,
+                    self.out_features, self.in_features, x.dtype,
+                )  # fmt: skip
+            else:
+                w = kernels.vq_dequant(
+                    self.packed_indices, self.proxy.centroids, self.bits,
+                    self.out_features, self.in_features, x.dtype,
+                )  # fmt: skip
+        except RuntimeError as exc:
+            self._fallback("vq_dequant", "the gather path", exc)
+            return self._forward_compile(x)
+        return F.linear(x, w, self.bias)
+
+    def _forward_tile_gemm(self, x: torch.Tensor) -> torch.Tensor:
+        """Band (b): MFMA GEMM decoding weight tiles in-kernel.
+
+        Takes the place of the reference's Triton band (np_vq_linear.py:1097-1125).
+        """
+        global _tile_failed
+        if _tile_failed or x.dtype not in (torch.bfloat16, torch.float16):
+            return self._forward_dequant_gemm(x)
+        try:
+            y = self._fused(x, tile=True)
+        except RuntimeError as exc:
+            self._fallback("vq_gemm_tile", "decode + GEMM", exc)
+            _tile_failed = True
+            return self._forward_dequant_gemm(x)
+        return y
+
+    def _res_stream(self) -> torch.Tensor:
+        if self.packed_residual is not None:
+            return self.packed_residual
+        z = self._derived.get("zero_res")
+        if z is None or z.device != self.packed_indices.device:
+            z = torch.zeros(self.n_vectors, dtype=torch.uint8, device=self.packed_indices.device)
+            self._derived["zero_res"] = z
+        return z
+
+    def _res_bits(self) -> int:
+        return self.residual_bits if self.packed_residual is not None else 8
+
+    def _res_centroids(self) -> torch.Tensor:
+        if self.residual_proxy is not None:
+            return self.residual_proxy.centroids
+        z = self._derived.get("zero_cb")
+        if z is None or z.device != self.packed_indices.device:
+            z = torch.zeros(
+                (1, self.vector_len), dtype=torch.float16, device=self.packed_indices.device
+            )
+            self._derived["zero_cb"] = z
+        return z
+
+    def _fused(self, x: torch.Tensor, tile: bool) -> torch.Tensor:
+        from .. import kernels
+
+        *leading, _ = x.shape
+        x2d = x.reshape(-1, self.in_features)
+        if self.is_residual:
+            y = kernels.rvq_linear(
+                x2d, self.packed_indices, self.bits, self._res_stream(), self._res_bits(),
+                self.proxy.centroids, self._res_centroids(), self.row_scale, self.row_bias,
+                self.out_features, self._bias_f32(), tile=tile,
+            )  # fmt: skip
+        else:
+            stream, bits = self._kernel_stream()
+            cb = self.proxy.centroids_as(x.dtype)
+            fn = kernels.vq_gemm_tile if tile else kernels.vq_linear
+            if tile:
+                y = fn(x2d, stream, cb, bits, self.out_features, self._bias_f32())
+            else:
+                y = fn(x2d, stream, cb, bits, self.vector_len, self._bias_f32(), self.out_features)
+        return y.reshape(*leading, self.out_features)
+
+    def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:
+        """Band (a) (reference: np_vq_linear.py:1173-1187).  Above the kernel's
+        16-token limit (reachable only with a raised threshold) the tile GEMM runs."""
+        m = x.numel() // self.in_features
+        return self._fused(x, tile=m > 16)
+
+    def _forward_cuda_wmma(self, x: torch.Tensor) -> torch.Tensor:
+        """GEMV / GEMM by token count (reference: np_vq_linear.py:1250-1267)."""
+        m = x.numel() // self.in_features
+        return self._fused(x, tile=m > 16)
+
+    def _forward_cuda_lut(self, x: torch.Tensor) -> torch.Tensor:
+        """Reached only when ``_LUT_MAX_TOKENS`` was raised above 0.
+
+        The reference's LUT kernel (np_vq_linear.py:1192-1248) builds an
+        ``[M, n_groups, NC]`` table, which for the codebooks it is chosen for is
+        larger than the weight and loses at every M (np_vq_linear.py:75-79);
+        it is not rebuilt.  The same result is produced by the fused kernels.
+        """
+        m = x.numel() // self.in_features
+        return self._fused(x, tile=m > 16)
+
+    # ------------------------------------------------------------------
+
+    def extra_repr(self) -> str:
+        perm_str = ", perm=True" if self.column_perm is not None else ""
+        res_str = ", residual=True" if self.is_residual else ""
+        return (
+            f"in={self.in_features}, out={self.out_features}, "
+            f"vector_len={self.vector_len}, "
+            f"num_centroids={self.proxy.num_centroids}, "
+            f"bits={self.bits}, backend={self.backend.value}"
+            f"{perm_str}{res_str}"
+        )
+
+
+# ---------------------------------------------------------------------------
+# Model-level transform
+# ---------------------------------------------------------------------------
+
+
+def linearize_vq_weights(
+    model: nn.Module,
+    backend: str | VQBackend | None = VQBackend.AUTO,
+) -> nn.Module:
+    """Replace every ``nn.Linear`` carrying a VQ weight with an :class:`NPVQLinear`.
+
+    Follows neuropress/nn/np_vq_linear.py:1432-1517: layers whose codebook is
+    the same tensor object share one :class:`VQProxy`; each unique proxy is
+    registered on the model root as ``_vq_proxy_<i>`` (residual codebooks as
+    ``_vq_res_proxy_<i>``).  The model is mutated in place and returned.
+    """
+    proxy_cache: dict[int, VQProxy] = {}
+    res_cache: dict[int, VQProxy] = {}
+    replacements: list[tuple[str, NPVQLinear]] = []
+
+    for name, module in model.named_modules():
+        if not isinstance(module, nn.Linear) or not is_vq_weight(module.weight):
+            continue
+        qs = module.weight.qscheme
+        cid = id(qs.centroids)
+        if cid not in proxy_cache:
+            proxy_cache[cid] = VQProxy(qs.centroids)
+        res_proxy = None
+        res_c = getattr(qs, "residual_centroids", None)
+        if res_c is not None:
+            if id(res_c) not in res_cache:
+                res_cache[id(res_c)] = VQProxy(res_c)
+            res_proxy = res_cache[id(res_c)]
+        try:
+            layer = NPVQLinear.from_qtensor_linear(module, proxy_cache[cid], backend, res_proxy)
+        except (TypeError, ValueError, NotImplementedError) as exc:
+            log.warning("linearize_vq_weights: skipping %s — %s", name, exc)
+            continue
+        replacements.append((name, layer))
+
+    if not replacements:
+        log.info("linearize_vq_weights: no VQ-weight linear layers found.")
+        return model
+
+    for i, proxy in enumerate(proxy_cache.values()):
+        model.add_module(f"_vq_proxy_{i}", proxy)
+    for i, proxy in enumerate(res_cache.values()):
+        model.add_module(f"_vq_res_proxy_{i}", proxy)
+
+    for name, layer in replacements:
+        if "." in name:
+            parent_name, attr = name.rsplit(".", 1)
+            parent = model.get_submodule(parent_name)
+        else:
+            parent, attr = model, name
+        setattr(parent, attr, layer)
+
+    counts: dict[str, int] = {}
+    for _, layer in replacements:
+        counts[layer.backend.value] = counts.get(layer.backend.value, 0) + 1
+    summary = ", ".join(f"{v}x{k}" for k, v in sorted(counts.items()))
+    log.info(
+        "linearize_vq_weights: replaced %d layer(s) [%s], %d unique proxy/ies",
+        len(replacements),
+        summary,
+        len(proxy_cache),
+    )
+    return model
