@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-sweep]
+
+One "step" = one call of the fused decode GEMV on BASELINE config 3's up/gate
+layer (Llama-3-8B MLP, N=14336, K=4096, vector length 8, 65536-entry fp16
+codebook, 16-bit indices, bf16 activations, M=1 token) on synthetic seeded
+data already resident in HBM.  K steps are recorded into one HIP graph over a
+rotating pool of weight/activation buffers larger than L2 + Infinity Cache and
+timed with HIP events on the launch stream, so `value` is kernel throughput,
+not Python launch overhead, and the index stream really comes from HBM.
+
+Prints ONE JSON line: the headline value (algorithmic GB/s of the M=1 GEMV),
+`roofline` for that kernel, `cpu_baseline` (the reference's CPU path restated
+with torch ops, timed on this host), and a `sweep` over the other bands /
+configs (us per call, GB/s, TFLOP/s, fraction of peak).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0      # dense bf16 / fp16
+METRIC = "VQ-linear µs/call + HBM GB/s (M=1), TFLOP/s (M=384), Llama-3-8B shapes"
+POOL_BYTES = 640 << 20         # rotate through more than L2 (32 MB) + Infinity Cache (256 MB)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
+    return ap.parse_args()
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def time_graph(fn, n_rot, steps, warmup, dev):
+    """Average microseconds per call of fn(i), `steps` calls recorded in one HIP graph.
+
+    Events are recorded on the stream the graph is launched on (torch's current
+    stream), before and after the replay.
+    """
+    for i in range(max(warmup, 1)):
+        fn(i % n_rot)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(steps):
+            fn(i % n_rot)
+    graph.replay()  # untimed: first replay uploads the graph
+    torch.cuda.synchronize(dev)
+    best = float("inf")
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize(dev)
+        best = min(best, e0.elapsed_time(e1) * 1e3 / steps)
+    return best
+
+
+def vq_case(dev, seed, n, k, nc, bits, act, n_rot):
+    from neuropress_amd.transforms.vq_packing import IndexPacking
+
+    g = gen(seed)
+    cb = (torch.randn(nc, 8, generator=g) * 0.02).to(torch.float16)
+    n_idx = n * (k // 8)
+    if bits == 16:
+        base = torch.randint(0, 65536, (n_idx,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8)
+    else:
+        base = IndexPacking.pack(torch.randint(0, nc, (n_idx,), generator=g), bits)
+    x = torch.randn(16, k, generator=g).to(act)
+    d_base = base.to(dev)
+    pool = [d_base] + [d_base.clone() for _ in range(n_rot - 1)]
+    return dict(cb=cb, packed=base, x=x, d_cb=cb.to(dev), d_cb_act=cb.to(act).to(dev), pool=pool,
+                n=n, k=k, nc=nc, bits=bits, act=act, idx_bytes=base.numel())
+
+
+def vq_alg_bytes(c, m):
+    return c["idx_bytes"] + c["nc"] * 16 + m * c["k"] * 2 + m * c["n"] * 2
+
+
+def check_against_cpu(y_gpu, y_cpu):
+    err = (y_gpu.float().cpu() - y_cpu.float()).abs()
+    bound = 1e-2 + 1e-2 * y_cpu.float().abs()
+    return bool((err <= bound).all()), float(err.max())
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: the path has no multi-GPU component (got --gpus {args.gpus}). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False).", file=sys.stderr)
+        sys.exit(2)
+    from neuropress_amd import _lib, kernels
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---------------- headline: config 3 up/gate, M = 1, fused GEMV -------------
+    n, k = 14336, 4096
+    n_rot = max(2, POOL_BYTES // (n * k // 8 * 2))
+    c3 = vq_case(dev, 1003, n, k, 65536, 16, torch.bfloat16, n_rot)
+    xs = [torch.randn(1, k, generator=gen(7 + i)).to(torch.bfloat16).to(dev) for i in range(n_rot)]
+    ys = [None] * n_rot
+
+    def step(i):
+        ys[i] = kernels.vq_linear(xs[i], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n)
+
+    us = time_graph(step, n_rot, args.steps, args.warmup, dev)
+    alg = vq_alg_bytes(c3, 1)
+    gbs = alg / us / 1e3
+
+    # correctness gate on the timed configuration (decode bit-exact, output within 1e-2)
+    w_gpu = kernels.vq_dequant(c3["pool"][0], c3["d_cb"], 16, n, k, torch.bfloat16)
+    idx = (c3["packed"].view(torch.int16).to(torch.int64) & 0xFFFF)
+    decode_exact = bool(torch.equal(w_gpu.cpu(), c3["cb"][idx].reshape(n, k).to(torch.bfloat16)))
+    y_ref = xs[0].float() @ w_gpu.float().T
+    ok, max_abs = check_against_cpu(ys[0], y_ref.cpu())
+
+    result = {
+        "metric": METRIC,
+        "value": round(gbs, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us / 1e3, 6),
+        "us_per_call": round(us, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seed 1003; uniform 16-bit indices, N(0,0.02) fp16 codebook, N(0,1) bf16 activations)",
+        "config": {
+            "workload": "BASELINE config 3: Llama-3-8B MLP up/gate 14336x4096, VL=8, 65536-entry fp16 codebook, "
+                        "16-bit indices, bf16, M=1 (fused decode GEMV, band a)",
+            "N": n, "K": k, "M": 1, "rotating_pool_MB": round(n_rot * c3["idx_bytes"] / 2**20),
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "fused_gemv_kernel (vq, 16-bit)", "algorithmic_bytes_per_launch": alg,
+            "avg_launch_us": round(us, 3),
+        },
+        "checks": {"decode_bit_exact": decode_exact, "output_within_1e-2": ok, "max_abs_err": max_abs},
+    }
+
+    # ---------------- sweep over the other bands / configs ----------------------
+    sweep = []
+    if not args.no_sweep:
+        def add(name, band, m, us_, alg_bytes, flops):
+            sweep.append({"case": name, "band": band, "M": m, "us": round(us_, 2),
+                          "GBps": round(alg_bytes / us_ / 1e3, 1), "hbm_frac": round(alg_bytes / us_ / 1e3 / HBM_PEAK_GBS, 4),
+                          "TFLOPs": round(flops / us_ / 1e6, 1), "mfma_frac": round(flops / us_ / 1e6 / MFMA_PEAK_TFLOPS, 4)})
+
+        steps_s = max(10, args.steps // 10)
+        for m in (2, 16):
+            xm = [torch.randn(m, k, generator=gen(50 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
+            t = time_graph(lambda i: kernels.vq_linear(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n),
+                           n_rot, steps_s * 2, 3, dev)
+            add("cfg3 14336x4096 bf16", "a:gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+        for m in (64, 384, 1024):
+            xm = [torch.randn(m, k, generator=gen(60 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
+            t = time_graph(lambda i: kernels.vq_gemm_tile(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, n, None),
+                           n_rot, steps_s, 2, dev)
+            add("cfg3 14336x4096 bf16", "b:tile-gemm", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+            t = time_graph(lambda i: torch.nn.functional.linear(
+                xm[i % 2], kernels.vq_dequant(c3["pool"][i], c3["d_cb"], 16, n, k, torch.bfloat16)),
+                n_rot, steps_s, 2, dev)
+            add("cfg3 14336x4096 bf16", "c:decode+gemm", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+        del c3["pool"][1:]
+        torch.cuda.empty_cache()
+        # config 3 down-proj shape
+        c3d = vq_case(dev, 1003, 4096, 14336, 65536, 16, torch.bfloat16, n_rot)
+        for m, fn, band in ((1, kernels.vq_linear, "a:gemv"), (384, None, "b:tile-gemm")):
+            xm = [torch.randn(m, 14336, generator=gen(70 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
+            if fn is not None:
+                f = lambda i: kernels.vq_linear(xm[i % 2], c3d["pool"][i], c3d["d_cb_act"], 16, 8, None, 4096)
+            else:
+                f = lambda i: kernels.vq_gemm_tile(xm[i % 2], c3d["pool"][i], c3d["d_cb_act"], 16, 4096, None)
+            t = time_graph(f, n_rot, steps_s * (2 if m == 1 else 1), 2, dev)
+            add("cfg3 4096x14336 bf16", band, m, t, vq_alg_bytes(c3d, m), 2.0 * m * 4096 * 14336)
+        del c3d
+        torch.cuda.empty_cache()
+        # config 2 gate/up (12-bit stream, 4096-entry codebook) and config 1
+        for name, (nn_, kk, nc, bits), ms in (("cfg2 8192x2048 f16 12-bit", (8192, 2048, 4096, 12), (1, 2)),
+                                              ("cfg1 2048x640 f16 8-bit", (2048, 640, 256, 8), (1, 16))):
+            rot = max(2, min(256, POOL_BYTES // (nn_ * kk // 8 * bits // 8)))
+            cc = vq_case(dev, 1002, nn_, kk, nc, bits, torch.float16, rot)
+            for m in ms:
+                xm = [torch.randn(m, kk, generator=gen(80 + m)).to(torch.float16).to(dev) for _ in range(2)]
+                t = time_graph(lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_),
+                               rot, steps_s * 2, 3, dev)
+                add(name, "a:gemv", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
+            del cc
+            torch.cuda.empty_cache()
+        # config 5: int4 group-affine, 14336x4096 fp16
+        from neuropress_amd.t2n.packing import BitPacking4
+
+        g = gen(1005)
+        nn_, kk = 14336, 4096
+        blob = BitPacking4.compress(torch.randint(0, 16, (nn_, kk), generator=g, dtype=torch.int64).to(torch.uint8))
+        sc = (torch.rand(nn_ * kk // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
+        rot = max(2, POOL_BYTES // blob.numel())
+        blobs = [blob.to(dev)]
+        blobs += [blobs[0].clone() for _ in range(rot - 1)]
+        for m in (1, 16, 256):
+            xm = [torch.randn(m, kk, generator=gen(90 + m)).to(torch.float16).to(dev) for _ in range(2)]
+            t = time_graph(lambda i: kernels.q_linear(xm[i % 2], blobs[i], sc, 4, 32), rot, steps_s, 2, dev)
+            algq = nn_ * kk // 2 + nn_ * kk // 32 * 2 + m * kk * 2 + m * nn_ * 2
+            add("cfg5 int4 14336x4096 f16", "a:gemv" if m <= 16 else "b:tile-gemm", m, t, algq, 2.0 * m * nn_ * kk)
+        del blobs
+        torch.cuda.empty_cache()
+    result["sweep"] = sweep
+
+    # ---------------- CPU baseline: the reference's CPU path, same workload ------
+    if not args.no_cpu:
+        from oracle import torch_path  # test infrastructure, used here only as the timed CPU baseline
+
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        x_cpu = xs[0].cpu()
+        reps = []
+        for it in range(4):  # first iteration is warm-up
+            t0 = time.perf_counter()
+            y_cpu = torch_path.vq_linear_cpu(x_cpu, c3["packed"], c3["cb"], 16, n, k, None, fast_unpack=True)
+            reps.append(time.perf_counter() - t0)
+        t_cpu = sorted(reps[1:])[len(reps[1:]) // 2]
+        ok_cpu, max_abs_cpu = check_against_cpu(ys[0], y_cpu)
+        cpu_model = ""
+        try:
+            with open("/proc/cpuinfo") as fh:
+                for ln in fh:
+                    if ln.startswith("model name"):
+                        cpu_model = ln.split(":", 1)[1].strip()
+                        break
+        except OSError:
+            pass
+        result["cpu_baseline"] = {
+            "value": round(alg / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "the full config-3 up/gate layer at M=1, 3 timed calls (median) of unpack (vectorised "
+                      "16-bit view) + codebook gather + cast + torch F.linear in bf16",
+            "ms_per_call": round(t_cpu * 1e3, 2), "cpu": cpu_model,
+            "gpu_matches_cpu_within_1e-2": ok_cpu, "max_abs_diff": max_abs_cpu,
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,64 @@
+"""Seeded synthetic layers shared by the tests (same generators as bench.py)."""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from neuropress_amd.transforms.vq_packing import IndexPacking
+
+
+def gen(seed: int) -> torch.Generator:
+    return torch.Generator().manual_seed(seed)
+
+
+def vq_layer(seed, n, k, nc, vl=8, bits=None, act=torch.float16, m=1, bias=False, std=0.02):
+    g = gen(seed)
+    bits = bits or IndexPacking.bits_for(nc)
+    cb = (torch.randn(nc, vl, generator=g) * std).to(torch.float16)
+    idx = torch.randint(0, nc, (n * (k // vl),), generator=g)
+    packed = IndexPacking.pack(idx, bits)
+    x = torch.randn(m, k, generator=g).to(act)
+    b = torch.randn(n, generator=g).to(act) if bias else None
+    return dict(cb=cb, idx=idx, packed=packed, bits=bits, x=x, bias=b, n=n, k=k, vl=vl, nc=nc)
+
+
+def zipf_indices(g, nc, count, s=1.1):
+    p = 1.0 / torch.arange(1, nc + 1, dtype=torch.float64) ** s
+    return torch.multinomial(p / p.sum(), count, replacement=True, generator=g)
+
+
+def rvq_layer(seed, n, k, nc_main=65536, nc_res=256, vl=8, act=torch.float16, m=1, zipf=True):
+    g = gen(seed)
+    cbm = (torch.randn(nc_main, vl, generator=g) * 0.02).to(torch.float16)
+    cbr = (torch.randn(nc_res, vl, generator=g) * 0.02).to(torch.float16)
+    cnt = n * (k // vl)
+    im = zipf_indices(g, nc_main, cnt) if zipf else torch.randint(0, nc_main, (cnt,), generator=g)
+    ir = zipf_indices(g, nc_res, cnt) if zipf else torch.randint(0, nc_res, (cnt,), generator=g)
+    bm, br = IndexPacking.bits_for(nc_main), IndexPacking.bits_for(nc_res)
+    scale = (torch.rand(n, generator=g) + 0.5).to(torch.float16)
+    wbias = (torch.randn(n, generator=g) * 0.01).to(torch.float16)
+    x = torch.randn(m, k, generator=g).to(act)
+    return dict(cbm=cbm, cbr=cbr, im=im, ir=ir, pm=IndexPacking.pack(im, bm), pr=IndexPacking.pack(ir, br),
+                bm=bm, br=br, scale=scale, wbias=wbias, x=x, n=n, k=k, vl=vl)
+
+
+def q4_layer(seed, n, k, nbits=4, gs=32, act=torch.float16, m=1, asym=False, bias=False):
+    from neuropress_amd.t2n.packing import BitPacking
+
+    g = gen(seed)
+    codes = torch.randint(0, 1 << nbits, (n, k), generator=g, dtype=torch.int64).to(torch.uint8)
+    blob = BitPacking(nbits).compress(codes)
+    scale = (torch.rand(n * (k // gs), generator=g) * 0.019 + 0.001).to(torch.float16)
+    zp = (torch.rand(n * (k // gs), generator=g) * ((1 << nbits) - 1)).to(torch.float16) if asym else None
+    x = torch.randn(m, k, generator=g).to(act)
+    b = torch.randn(n, generator=g).to(act) if bias else None
+    return dict(codes=codes, blob=blob, scale=scale, zp=zp, x=x, bias=b, n=n, k=k, nbits=nbits, gs=gs)
+
+
+def within_tol(y: np.ndarray, ref: np.ndarray, atol=1e-2, rtol=1e-2):
+    """The output bar of the path: |y - ref| <= 1e-2 + 1e-2 * |ref| against an
+    f32-or-better accumulated reference.  Returns (ok, max_abs, max_rel_excess)."""
+    err = np.abs(y.astype(np.float64) - ref)
+    bound = atol + rtol * np.abs(ref)
+    return bool((err <= bound).all()), float(err.max(initial=0.0)), float((err / bound).max(initial=0.0))

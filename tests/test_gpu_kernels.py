@@ -1,0 +1,291 @@
+"""Parity of the HIP kernels against the CPU oracle, through the C ABI (ctypes wrappers).
+
+Bars: decoded weights bit-exact; layer outputs within 1e-2 abs + 1e-2 rel of
+the oracle's double-accumulated contraction of the oracle-decoded weight.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+def _bits_equal(t: torch.Tensor, ref: np.ndarray):
+    got = orc.to_bits(t)
+    assert got.dtype == ref.dtype and got.shape == ref.shape
+    assert np.array_equal(got, ref), f"{(got != ref).sum()} of {ref.size} elements differ"
+
+
+# ------------------------------------------------------------------ decode ---
+
+
+@pytest.mark.parametrize("vl", [4, 8, 6])
+@pytest.mark.parametrize("bits", [4, 8, 10, 12, 14, 16])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_vq_dequant_bit_exact(gpu, oracle_lib, bits, dtype, vl):
+    # Odd N so the last index ends mid-byte (the reference's own case:
+    # tests/nn/test_np_vq_linear.py:546-562 of the reference).
+    from neuropress_amd import kernels
+
+    n, k = 37, 16 * vl
+    nc = min(1 << bits, 4096)
+    L = cases.vq_layer(100 + bits, n, k, nc, vl=vl, bits=bits, std=1.0)
+    ref = oracle_lib.vq_decode(L["packed"].numpy(), bits, orc.to_bits(L["cb"]), n, k, orc.torch_dtype_code(dtype))
+    out = kernels.vq_dequant(L["packed"].to(gpu), L["cb"].to(gpu), bits, n, k, dtype)
+    assert out.dtype == dtype and out.shape == (n, k)
+    _bits_equal(out, ref)
+
+
+def test_vq_dequant_special_values(gpu, oracle_lib):
+    """Codebook holding inf, subnormals, the largest finite half and signed zeros."""
+    from neuropress_amd import kernels
+
+    bits_pat = np.array([0x0000, 0x8000, 0x7C00, 0xFC00, 0x0001, 0x8001, 0x03FF, 0x7BFF,
+                         0x3555, 0xB555, 0x0400, 0x3C01, 0x3BFF, 0x1234, 0xABCD, 0x4321], dtype=np.uint16)
+    cb = orc.from_bits(bits_pat.reshape(2, 8), torch.float16)
+    idx = torch.tensor([0, 1, 1, 0, 1, 0])
+    from neuropress_amd.transforms.vq_packing import IndexPacking
+
+    packed = IndexPacking.pack(idx, 4)
+    for dtype in DTYPES:
+        ref = oracle_lib.vq_decode(packed.numpy(), 4, bits_pat.reshape(2, 8), 2, 24, orc.torch_dtype_code(dtype))
+        out = kernels.vq_dequant(packed.to(gpu), cb.to(gpu), 4, 2, 24, dtype)
+        _bits_equal(out, ref)
+
+
+@pytest.mark.parametrize("bits", [4, 5, 7, 9, 12, 13, 16])
+def test_widen_indices(gpu, bits):
+    from neuropress_amd import kernels
+    from neuropress_amd.transforms.vq_packing import IndexPacking
+
+    idx = torch.randint(0, 1 << bits, (1001 if bits != 4 else 1002,), generator=cases.gen(bits))
+    packed = IndexPacking.pack(idx, bits).to(gpu)
+    got = kernels.unpack_indices(packed, idx.numel(), bits).cpu()
+    assert torch.equal(got, idx)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("with_affine", [True, False])
+def test_rvq_dequant_bit_exact(gpu, oracle_lib, dtype, with_affine):
+    from neuropress_amd import kernels
+
+    L = cases.rvq_layer(7, 24, 128, nc_main=4096, nc_res=256)
+    sc = L["scale"] if with_affine else None
+    wb = L["wbias"] if with_affine else None
+    ref = oracle_lib.rvq_decode(
+        L["pm"].numpy(), L["bm"], L["pr"].numpy(), L["br"], orc.to_bits(L["cbm"]), orc.to_bits(L["cbr"]),
+        None if sc is None else orc.to_bits(sc), None if wb is None else orc.to_bits(wb),
+        24, 128, orc.torch_dtype_code(dtype))
+    out = kernels.rvq_dequant(
+        L["pm"].to(gpu), L["bm"], L["pr"].to(gpu), L["br"], L["cbm"].to(gpu), L["cbr"].to(gpu),
+        None if sc is None else sc.to(gpu), None if wb is None else wb.to(gpu), 24, 128, dtype)
+    _bits_equal(out, ref)
+
+
+@pytest.mark.parametrize("nbits,gs", [(4, 32), (4, 128), (8, 32), (2, 16), (1, 8), (4, 24)])
+@pytest.mark.parametrize("asym", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_q_dequant_bit_exact(gpu, oracle_lib, nbits, gs, asym, dtype):
+    from neuropress_amd import kernels
+
+    n, k = 19, gs * 8
+    L = cases.q4_layer(50 + nbits, n, k, nbits=nbits, gs=gs, asym=asym)
+    ref = oracle_lib.q_decode(L["blob"].numpy(), orc.to_bits(L["scale"]),
+                              None if L["zp"] is None else orc.to_bits(L["zp"]), nbits, gs,
+                              orc.torch_dtype_code(dtype))
+    out = kernels.q_dequant(L["blob"].to(gpu), L["scale"].to(gpu), nbits, gs,
+                            None if L["zp"] is None else L["zp"].to(gpu), dtype)
+    _bits_equal(out, ref)
+
+
+# ---------------------------------------------------------------- contraction ---
+
+
+def _vq_ref(oracle_lib, L, act):
+    code = orc.torch_dtype_code(act)
+    w = oracle_lib.vq_decode(L["packed"].numpy(), L["bits"], orc.to_bits(L["cb"]), L["n"], L["k"], code)
+    bias = None if L["bias"] is None else orc.to_bits(L["bias"])
+    return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
+
+
+def _check(y: torch.Tensor, ref: np.ndarray):
+    ok, max_abs, excess = cases.within_tol(y.float().cpu().numpy(), ref)
+    assert ok, f"max abs err {max_abs:.3e}, {excess:.2f}x the 1e-2 bound"
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,nc", [(4, 16), (8, 256), (12, 4096), (16, 65536)])
+@pytest.mark.parametrize("m", [1, 2, 5, 16])
+def test_vq_gemv_fast_path(gpu, oracle_lib, act, bits, nc, m):
+    from neuropress_amd import kernels
+
+    # N not a multiple of 16, K = 5 chunks of 64 (not a multiple of the 256-k step).
+    L = cases.vq_layer(200 + bits + m, 100, 320, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
+    y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 8,
+                          L["bias"].to(gpu), out_features=100)
+    assert y.shape == (m, 100) and y.dtype == act
+    _check(y, _vq_ref(oracle_lib, L, act))
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+def test_vq_gemv_precast_codebook(gpu, oracle_lib, act):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(31, 64, 512, 4096, act=act, m=2, std=0.05)
+    y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(act).to(gpu), 12, 8, None, 64)
+    _check(y, _vq_ref(oracle_lib, L, act))
+
+
+@pytest.mark.parametrize("vl,bits,nc,k", [(4, 10, 1024, 96), (8, 14, 16384, 72), (8, 16, 65536, 200), (2, 4, 16, 64)])
+@pytest.mark.parametrize("m", [1, 3])
+def test_vq_gemv_generic_path(gpu, oracle_lib, vl, bits, nc, k, m):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(300 + bits, 37, k, nc, vl=vl, bits=bits, act=torch.float16, m=m, bias=True, std=0.05)
+    y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, vl, L["bias"].to(gpu), 37)
+    _check(y, _vq_ref(oracle_lib, L, torch.float16))
+
+
+@pytest.mark.parametrize("bits", [4, 8, 10, 12, 14, 16])
+@pytest.mark.parametrize("m", [1, 17, 130])
+def test_vq_gemm_tile_reference_shapes(gpu, oracle_lib, bits, m):
+    """The reference's Triton test shapes (tests/nn/test_vq_triton.py:11-29): N=72, K=96, VL=4, bf16."""
+    from neuropress_amd import kernels
+
+    nc = min(1 << bits, 4096)
+    L = cases.vq_layer(400 + bits, 72, 96, nc, vl=4, bits=bits, act=torch.bfloat16, m=m, bias=True, std=1.0)
+    y = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 72, L["bias"].to(gpu))
+    ref = _vq_ref(oracle_lib, L, torch.bfloat16)
+    # K=96 with unit-variance weights: the reference's own tolerance for this case.
+    assert np.allclose(y.float().cpu().numpy(), ref, rtol=2e-2, atol=5e-2)
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,nc", [(8, 256), (12, 4096), (16, 65536)])
+@pytest.mark.parametrize("m", [1, 17, 96, 130, 300])
+def test_vq_gemm_tile_fast_path(gpu, oracle_lib, act, bits, nc, m):
+    from neuropress_amd import kernels
+
+    # N = 300 spans two 256-column blocks with a ragged tail; K = 448 = 3.5 macro-steps.
+    L = cases.vq_layer(500 + bits + m, 300, 448, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
+    y = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 300, L["bias"].to(gpu))
+    _check(y, _vq_ref(oracle_lib, L, act))
+
+
+def _rvq_ref(oracle_lib, L, act):
+    code = orc.torch_dtype_code(act)
+    w = oracle_lib.rvq_decode(L["pm"].numpy(), L["bm"], L["pr"].numpy(), L["br"], orc.to_bits(L["cbm"]),
+                              orc.to_bits(L["cbr"]), orc.to_bits(L["scale"]), orc.to_bits(L["wbias"]),
+                              L["n"], L["k"], code)
+    return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code)
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,tile", [(1, False), (4, False), (4, True), (150, True)])
+def test_rvq_linear(gpu, oracle_lib, act, m, tile):
+    from neuropress_amd import kernels
+
+    L = cases.rvq_layer(9, 80, 256, act=act, m=m)
+    y = kernels.rvq_linear(L["x"].to(gpu), L["pm"].to(gpu), L["bm"], L["pr"].to(gpu), L["br"], L["cbm"].to(gpu),
+                           L["cbr"].to(gpu), L["scale"].to(gpu), L["wbias"].to(gpu), 80, None, tile=tile)
+    _check(y, _rvq_ref(oracle_lib, L, act))
+
+
+def _q_ref(oracle_lib, L, act):
+    code = orc.torch_dtype_code(act)
+    w = oracle_lib.q_decode(L["blob"].numpy(), orc.to_bits(L["scale"]),
+                            None if L["zp"] is None else orc.to_bits(L["zp"]), L["nbits"], L["gs"], code)
+    bias = None if L["bias"] is None else orc.to_bits(L["bias"])
+    return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("m", [1, 16, 17, 200])
+def test_q4_linear_fast_path(gpu, oracle_lib, act, gs, m):
+    from neuropress_amd import kernels
+
+    L = cases.q4_layer(600 + gs + m, 300, 384, gs=gs, act=act, m=m, bias=True)
+    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
+    assert y.shape == (m, 300)
+    _check(y, _q_ref(oracle_lib, L, act))
+
+
+@pytest.mark.parametrize("nbits,gs,asym", [(4, 32, True), (8, 32, False), (2, 16, True), (1, 8, False), (4, 24, False)])
+@pytest.mark.parametrize("m", [2, 20])
+def test_q_linear_generic_path(gpu, oracle_lib, nbits, gs, asym, m):
+    from neuropress_amd import kernels
+
+    L = cases.q4_layer(700 + nbits, 21, gs * 4, nbits=nbits, gs=gs, act=torch.float16, m=m, asym=asym, bias=True)
+    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), nbits, gs,
+                         None if L["zp"] is None else L["zp"].to(gpu), L["bias"].to(gpu))
+    _check(y, _q_ref(oracle_lib, L, torch.float16))
+
+
+def test_q_known_answers(gpu):
+    """Reference KATs (tests/test_quantized_weight_regressions.py:848-859 of the reference):
+    code 15, zero point 2, scale 1 -> 13; an underflowed scale decodes the block to 0."""
+    from neuropress_amd import kernels
+
+    codes = torch.full((2, 32), 15, dtype=torch.uint8)
+    from neuropress_amd.t2n.packing import BitPacking4
+
+    blob = BitPacking4.compress(codes).to(gpu)
+    scale = torch.tensor([1e-12, 1.0]).to(torch.float16).to(gpu)
+    zp = torch.full((2,), 2.0, dtype=torch.float16, device=gpu)
+    w = kernels.q_dequant(blob, scale, 4, 32, zp, torch.float32).cpu()
+    assert torch.all(w[0] == 0) and torch.all(w[1] == 13)
+
+
+# ------------------------------------------------------------------ edges ---
+
+
+def test_empty_and_error_paths(gpu):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(1, 16, 64, 256)
+    cb, packed = L["cb"].to(gpu), L["packed"].to(gpu)
+    y = kernels.vq_linear(torch.empty(0, 64, device=gpu, dtype=torch.float16), packed, cb, 8, 8, None, 16)
+    assert y.shape == (0, 16)
+    with pytest.raises(RuntimeError, match="too short"):
+        kernels.vq_dequant(packed[:10], cb, 8, 16, 64, torch.float16)
+    with pytest.raises(RuntimeError, match="bits"):
+        kernels.vq_dequant(packed, cb, 3, 16, 64, torch.float16)
+    with pytest.raises(RuntimeError, match="exceeds the fused limit"):
+        kernels.vq_linear(torch.zeros(17, 64, device=gpu, dtype=torch.float16), packed, cb, 8, 8, None, 16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        kernels.vq_dequant(L["packed"], L["cb"], 8, 16, 64, torch.float16)
+    with pytest.raises(RuntimeError, match="float16 or bfloat16"):
+        kernels.vq_linear(torch.zeros(1, 64, device=gpu), packed, cb, 8, 8, None, 16)
+
+
+def test_out_of_range_index_is_clamped(gpu):
+    """A 16-bit stream pointing past a small codebook must not read outside it."""
+    from neuropress_amd import kernels
+    from neuropress_amd.transforms.vq_packing import IndexPacking
+
+    cb = torch.arange(4 * 8, dtype=torch.float16).reshape(4, 8).to(gpu)
+    packed = IndexPacking.pack(torch.tensor([0, 3, 60000, 65535] * 2), 16).to(gpu)
+    w = kernels.vq_dequant(packed, cb, 16, 1, 64, torch.float16)
+    assert torch.equal(w.reshape(8, 8)[2], cb[3]) and torch.equal(w.reshape(8, 8)[3], cb[3])
+
+
+def test_strided_x_and_stream(gpu, oracle_lib):
+    """Row-strided activations and a non-default stream."""
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(77, 48, 256, 256, m=3)
+    xbig = torch.zeros(3, 512, dtype=torch.float16, device=gpu)
+    xbig[:, :256] = L["x"].to(gpu)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        y = kernels.vq_linear(xbig[:, :256], L["packed"].to(gpu), L["cb"].to(gpu), 8, 8, None, 48)
+    s.synchronize()
+    _check(y, _vq_ref(oracle_lib, L, torch.float16))

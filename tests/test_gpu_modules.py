@@ -1,0 +1,212 @@
+"""GPU tests of the drop-in modules and of the full BASELINE sizes.
+
+Module tests: every band of NPVQLinear / NPLinear on the GPU against the
+torch-op specification of the same layer on the CPU.  Full-size tests use
+size-independent properties: decode equals torch's own gather on the device
+(a library routine), codebook-permutation invariance (bit-exact), a zero
+codebook yields exactly the bias, M-split invariance, linearity.
+"""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import neuropress_amd.nn.np_vq_linear as vqmod
+from neuropress_amd import AutoKernelLowering
+from neuropress_amd.nn import NPLinear, NPVQLinear, VQProxy
+from neuropress_amd.qweights import ScalarQWeight, VQWeight, attach_quantized_weight
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(y_gpu, y_ref):
+    ok, max_abs, excess = cases.within_tol(y_gpu.float().cpu().numpy(), y_ref.double().cpu().numpy())
+    assert ok, f"max abs err {max_abs:.3e} = {excess:.2f}x the 1e-2 bound"
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("bits,nc", [(8, 256), (10, 1024), (12, 4096), (16, 65536)])
+def test_npvqlinear_all_bands_match_default(gpu, act, bits, nc, monkeypatch):
+    monkeypatch.setattr(vqmod, "_FUSED_MAX_TOKENS", 16)
+    monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    L = cases.vq_layer(40 + bits, 96, 256, nc, bits=bits, bias=True, std=0.05)
+    ref_layer = NPVQLinear(VQProxy(L["cb"]), L["packed"], bits, 96, 256, 8, "default", bias=L["bias"].float())
+    proxy = VQProxy(L["cb"]).to(gpu)
+    layer = NPVQLinear(proxy, L["packed"], bits, 96, 256, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
+    for shape in [(1, 256), (2, 8, 256), (40, 256), (3, 50, 256)]:  # fused, fused(16), tile, dense
+        x = torch.randn(*shape, generator=cases.gen(1)).to(act)
+        y = layer(x.to(gpu))
+        assert y.shape == (*shape[:-1], 96) and y.dtype == act
+        # specification: gather + F.linear in f32 with the weight rounded to the activation dtype
+        w = L["cb"][L["idx"]].reshape(96, 256).to(act).float()
+        _close(y, torch.nn.functional.linear(x.float(), w, L["bias"].float()))
+        if act == torch.float32:
+            assert torch.allclose(y.cpu(), ref_layer(x), atol=1e-4)
+
+
+def test_lowering_auto_runs_hip_backends_on_gpu(gpu):
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            L = cases.vq_layer(5, 64, 128, 4096, bias=False)
+            self.fc = attach_quantized_weight(nn.Linear(128, 64, bias=True),
+                                              VQWeight.from_indices(L["idx"], L["cb"], 64, 128))
+            Q = cases.q4_layer(6, 64, 128)
+            self.q = attach_quantized_weight(nn.Linear(128, 64, bias=False),
+                                             ScalarQWeight.from_codes(Q["codes"], Q["scale"], 4, 32))
+
+        def forward(self, x):
+            return self.fc(x) + self.q(x)
+
+    torch.manual_seed(0)
+    m = M()
+    x = torch.randn(5, 128).half()
+    AutoKernelLowering(vq_backend="default", linear_backend="compile").apply(m)
+    ref = m(x.float())
+    from neuropress_amd import unlower_model
+
+    unlower_model(m)
+    m = m.to(gpu)
+    AutoKernelLowering().apply(m)
+    m = m.to(gpu)
+    assert m.fc.backend.value == "cuda_wmma" and m.q.backend.value == "cuda"
+    _close(m(x.to(gpu)), ref)
+    _close(m(torch.cat([x] * 8).to(gpu))[:5], ref)  # 40 tokens: tile bands
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+def test_nplinear_bands(gpu, act, monkeypatch):
+    import neuropress_amd.nn.np_linear as qmod
+
+    monkeypatch.setattr(qmod, "_Q_TILE_MAX_TOKENS", 64)
+    Q = cases.q4_layer(8, 80, 256, bias=True)
+    layer = NPLinear(Q["blob"], Q["scale"], 80, 256, 32, 4, "sym", "cuda", bias=Q["bias"].float()).to(gpu)
+    w = ((Q["codes"].float() - 8).reshape(80, 8, 32) * Q["scale"].float().reshape(80, 8, 1)).reshape(80, 256)
+    for m in (1, 16, 40, 100):
+        x = torch.randn(m, 256, generator=cases.gen(m)).to(act)
+        _close(layer(x.to(gpu)), torch.nn.functional.linear(x.float(), w.to(act).float(), Q["bias"].float()))
+
+
+def test_residual_module_bands(gpu, monkeypatch):
+    monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    L = cases.rvq_layer(12, 48, 256, nc_main=65536, nc_res=256)
+    mk = lambda backend: NPVQLinear(VQProxy(L["cbm"]), L["pm"], L["bm"], 48, 256, 8, backend,
+                                    residual_proxy=VQProxy(L["cbr"]), packed_residual=L["pr"],
+                                    residual_bits=L["br"], row_scale=L["scale"], row_bias=L["wbias"])
+    ref_layer = mk("default")
+    layer = mk("cuda_wmma").to(gpu)
+    layer.proxy.to(gpu), layer.residual_proxy.to(gpu)
+    w = ref_layer._dense_weight_torch(torch.float16).float()
+    for m in (1, 30, 100):
+        x = torch.randn(m, 256, generator=cases.gen(m)).half()
+        _close(layer(x.to(gpu)), x.float() @ w.T)
+
+
+# ------------------------------------------------------- BASELINE full sizes ---
+
+
+@pytest.fixture(scope="module")
+def cfg3(gpu):
+    """Config 3, up/gate shape: 14336 x 4096, 65536 x 8 codebook, 16-bit indices, seed 1003."""
+    g = cases.gen(1003)
+    cb = (torch.randn(65536, 8, generator=g) * 0.02).half()
+    idx16 = torch.randint(0, 65536, (14336 * 512,), generator=g, dtype=torch.int32).to(torch.int16)
+    return dict(cb=cb.to(gpu), idx16=idx16.to(gpu), packed=idx16.view(torch.uint8).to(gpu), n=14336, k=4096)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_cfg3_decode_equals_device_gather(gpu, cfg3, dtype):
+    from neuropress_amd import kernels
+
+    w = kernels.vq_dequant(cfg3["packed"], cfg3["cb"], 16, cfg3["n"], cfg3["k"], dtype)
+    idx = cfg3["idx16"].to(torch.int64) & 0xFFFF
+    assert torch.equal(w, cfg3["cb"][idx].reshape(cfg3["n"], cfg3["k"]).to(dtype))
+
+
+@pytest.mark.parametrize("m", [1, 2, 16])
+def test_cfg3_gemv_properties(gpu, cfg3, m):
+    from neuropress_amd import kernels
+
+    n, k = cfg3["n"], cfg3["k"]
+    x = torch.randn(m, k, generator=cases.gen(m)).bfloat16().to(gpu)
+    bias = torch.randn(n, generator=cases.gen(9)).to(gpu)
+    y = kernels.vq_linear(x, cfg3["packed"], cfg3["cb"], 16, 8, bias, n)
+    # against the dense product of the decoded weight (torch matmul = library routine)
+    w = kernels.vq_dequant(cfg3["packed"], cfg3["cb"], 16, n, k, torch.bfloat16)
+    ref = x.float() @ w.float().T + bias
+    _close(y, ref)
+    # codebook row permutation + index remap leaves the result bit-identical
+    perm = torch.randperm(65536, generator=cases.gen(2)).to(gpu)
+    inv = torch.argsort(perm)
+    idx = cfg3["idx16"].to(torch.int64) & 0xFFFF
+    remapped = inv[idx].to(torch.int16).view(torch.uint8)
+    y2 = kernels.vq_linear(x, remapped, cfg3["cb"][perm].contiguous(), 16, 8, bias, n)
+    assert torch.equal(y, y2)
+    # all-zero codebook -> exactly the bias (rounded once)
+    y0 = kernels.vq_linear(x, cfg3["packed"], torch.zeros_like(cfg3["cb"]), 16, 8, bias, n)
+    assert torch.equal(y0, bias.bfloat16().expand(m, n))
+    # rows of the batch are independent: each row alone gives the same bits
+    y_row = kernels.vq_linear(x[:1].contiguous(), cfg3["packed"], cfg3["cb"], 16, 8, bias, n)
+    assert torch.equal(y_row, y[:1])
+
+
+@pytest.mark.parametrize("m", [64, 384])
+def test_cfg3_tile_gemm_properties(gpu, cfg3, m):
+    from neuropress_amd import kernels
+
+    n, k = cfg3["n"], cfg3["k"]
+    x = torch.randn(m, k, generator=cases.gen(m)).bfloat16().to(gpu)
+    y = kernels.vq_gemm_tile(x, cfg3["packed"], cfg3["cb"], 16, n)
+    w = kernels.vq_dequant(cfg3["packed"], cfg3["cb"], 16, n, k, torch.bfloat16)
+    _close(y, x.float() @ w.float().T)
+    # splitting M across calls changes nothing (each output row depends on its own x row only)
+    y_a = kernels.vq_gemm_tile(x[: m // 2].contiguous(), cfg3["packed"], cfg3["cb"], 16, n)
+    assert torch.equal(y_a, y[: m // 2])
+    y0 = kernels.vq_gemm_tile(x, cfg3["packed"], torch.zeros_like(cfg3["cb"]), 16, n)
+    assert not y0.any()
+
+
+def test_cfg3_down_proj_shape(gpu):
+    """4096 x 14336: K = 224 chunks = 56 steps, exercises the many-waves-per-row split."""
+    from neuropress_amd import kernels
+
+    g = cases.gen(1003)
+    cb = (torch.randn(65536, 8, generator=g) * 0.02).half().to(gpu)
+    packed = torch.randint(0, 65536, (4096 * 1792,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8).to(gpu)
+    x = torch.randn(2, 14336, generator=g).bfloat16().to(gpu)
+    w = kernels.vq_dequant(packed, cb, 16, 4096, 14336, torch.bfloat16)
+    ref = x.float() @ w.float().T
+    _close(kernels.vq_linear(x, packed, cb, 16, 8, None, 4096), ref)
+    _close(kernels.vq_gemm_tile(x, packed, cb, 16, 4096), ref)
+
+
+def test_cfg5_q4_full_size(gpu):
+    from neuropress_amd import kernels
+
+    Q = cases.q4_layer(1005, 14336, 4096)
+    blob, sc = Q["blob"].to(gpu), Q["scale"].to(gpu)
+    w = kernels.q_dequant(blob, sc, 4, 32, None, torch.float16)
+    w_ref = ((Q["codes"].to(gpu).float() - 8).reshape(14336, 128, 32) * sc.float().reshape(14336, 128, 1))
+    assert torch.equal(w, w_ref.reshape(14336, 4096).half())
+    for m in (1, 16, 256):
+        x = torch.randn(m, 4096, generator=cases.gen(m)).half().to(gpu)
+        _close(kernels.q_linear(x, blob, sc, 4, 32), x.float() @ w.float().T)
+
+
+def test_cfg4_residual_full_size(gpu):
+    from neuropress_amd import kernels
+
+    L = cases.rvq_layer(1004, 1024, 4096)  # the k/v shape of config 4, Zipf(1.1) indices
+    dev = {k: (v.to(gpu) if isinstance(v, torch.Tensor) else v) for k, v in L.items()}
+    w = kernels.rvq_dequant(dev["pm"], L["bm"], dev["pr"], L["br"], dev["cbm"], dev["cbr"], dev["scale"],
+                            dev["wbias"], 1024, 4096, torch.float16)
+    w_ref = (dev["cbm"][dev["im"]] + dev["cbr"][dev["ir"]]).reshape(1024, 4096)
+    w_ref = (w_ref * dev["scale"][:, None]) + dev["wbias"][:, None]  # torch fp16 ops round one at a time
+    assert torch.equal(w, w_ref)
+    for m, tile in ((1, False), (384, True)):
+        x = torch.randn(m, 4096, generator=cases.gen(m)).half().to(gpu)
+        y = kernels.rvq_linear(x, dev["pm"], L["bm"], dev["pr"], L["br"], dev["cbm"], dev["cbr"], dev["scale"],
+                               dev["wbias"], 1024, None, tile=tile)
+        _close(y, x.float() @ w.float().T)
