@@ -241,6 +241,11 @@ class NPLinear(nn.Module):
             self._derived["bias_f32"] = b
         return b
 
+    def _bias_as(self, dtype: torch.dtype) -> torch.Tensor | None:
+        if self.bias is None or self.bias.dtype == dtype:
+            return self.bias
+        return self.bias.to(dtype)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.backend == LinearBackend.CUDA:
             return self._forward_cuda(x)
@@ -249,7 +254,8 @@ class NPLinear(nn.Module):
 
     def _forward_compile(self, x: torch.Tensor) -> torch.Tensor:
         return _q_dequant_linear(
-            x, self.u8_blob, self.scale, self.nbits, self.group_size, self.zero_point, self.bias
+            x, self.u8_blob, self.scale, self.nbits, self.group_size, self.zero_point,
+            self._bias_as(x.dtype),
         )
 
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:
@@ -278,7 +284,7 @@ class NPLinear(nn.Module):
                 raise
             kernels.warn_kernel_fallback("q_linear", "torch dequant + matmul", exc)
             return self._forward_compile(x)
-        return F.linear(x, w, self.bias)
+        return F.linear(x, w, self._bias_as(x.dtype))
 
     def extra_repr(self) -> str:
         return (

@@ -412,6 +412,12 @@ class NPVQLinear(nn.Module):
             self._derived["bias_f32"] = b
         return b
 
+    def _bias_as(self, dtype: torch.dtype) -> torch.Tensor | None:
+        """Bias in the activation dtype for the torch GEMM (``F.linear`` wants one dtype)."""
+        if self.bias is None or self.bias.dtype == dtype:
+            return self.bias
+        return self.bias.to(dtype)
+
     def _kernel_stream(self) -> tuple[torch.Tensor, int]:
         """Index stream and width the fused kernels read.
 
@@ -474,10 +480,10 @@ class NPVQLinear(nn.Module):
     def _forward_default(self, x: torch.Tensor) -> torch.Tensor:
         """Follows neuropress/nn/np_vq_linear.py:1091-1095."""
         if self.is_residual:
-            return F.linear(x, self._dense_weight_torch(x.dtype), self.bias)
+            return F.linear(x, self._dense_weight_torch(x.dtype), self._bias_as(x.dtype))
         return _vq_dequant_linear(
             x, self.packed_indices, self.proxy.centroids, self.bits, self.n_vectors,
-            self.out_features, self.in_features, self.bias,
+            self.out_features, self.in_features, self._bias_as(x.dtype),
         )  # fmt: skip
 
     def _forward_compile(self, x: torch.Tensor) -> torch.Tensor:
@@ -518,7 +524,7 @@ class NPVQLinear(nn.Module):
         except RuntimeError as exc:
             self._fallback("vq_dequant", "the gather path", exc)
             return self._forward_compile(x)
-        return F.linear(x, w, self.bias)
+        return F.linear(x, w, self._bias_as(x.dtype))
 
     def _forward_tile_gemm(self, x: torch.Tensor) -> torch.Tensor:
         """Band (b): MFMA GEMM decoding weight tiles in-kernel.
