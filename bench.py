@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain device copy of 256 MiB (10 launches): the known-size kernel "
+                         "the FETCH_SIZE / WRITE_SIZE counters are scaled against")
     return ap.parse_args()
 
 
@@ -117,6 +120,17 @@ def main():
     _lib.load()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy:
+        nbytes = 256 << 20
+        src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize(dev)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize(dev)
+        print(json.dumps({"calibration": "device copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": 10}))
+        return
 
     # ---------------- headline: config 3 up/gate, M = 1, fused GEMV -------------
     n, k = 14336, 4096
