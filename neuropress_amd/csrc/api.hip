@@ -76,25 +76,11 @@ GemvPlan plan_gemv(int N, int chunks) {
   return p;
 }
 
-// NPAMD_TILE_MT overrides the choice (tuning aid).
-int plan_tile_mt(int M, int N) {
-  const int mt_env = env_int("NPAMD_TILE_MT", 0);
-  if (mt_env >= 1 && mt_env <= 4) return mt_env;
-  const int cus = device_cu_count();
-  const int n_blocks = (N + kTileCols - 1) / kTileCols;
-  int best = 1;
-  double best_cost = 1e30;
-  for (int mt = 1; mt <= 4; ++mt) {
-    const int m_blocks = (M + 32 * mt - 1) / (32 * mt);
-    const int64_t blocks = (int64_t)m_blocks * n_blocks;
-    const int64_t passes = (blocks + cus - 1) / cus;
-    const double cost = (double)passes * (mt + 1.0);
-    if (cost < best_cost - 1e-9) {
-      best_cost = cost;
-      best = mt;
-    }
-  }
-  return best;
+int plan_tile_mw(int M) {
+  const int mw_env = env_int("NPAMD_TILE_MW", 0);
+  if (mw_env >= 1 && mw_env <= 3) return mw_env;
+  const int mw = (M + 127) / 128;
+  return mw < 1 ? 1 : (mw > 3 ? 3 : mw);
 }
 
 }  // namespace npamd

@@ -54,42 +54,51 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
 
   const int step_begin = wave * s.steps_per_wave;
   const int step_end = min(step_begin + s.steps_per_wave, s.steps);
-  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(s.x) + (int64_t)c * s.ldx;
+  // Loads are branch-free: out-of-range lanes read a clamped (valid) address and
+  // their operand is zeroed afterwards, so all gathers of a step are in flight
+  // together instead of each sitting behind its own branch and wait.
+  const int x_row = min(c, s.M - 1);
+  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(s.x) + (int64_t)x_row * s.ldx;
   const bool x_lane = c < s.M;
+  const u32x4 zero4{0, 0, 0, 0};
 
   for (int step = step_begin; step < step_end; ++step) {
-    const int kc = step * 4 + q;
-    const bool kvalid = kc < s.chunks;
+    const int kc_raw = step * 4 + q;
+    const bool kvalid = kc_raw < s.chunks;
+    const int kc = min(kc_raw, s.chunks - 1);
 
     typename Provider::Raw raw[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int n = row0 + 16 * r + c;
-      prov.load(raw[r], n, kc, kvalid && n < s.N);
-    }
+    for (int r = 0; r < R; ++r) prov.load(raw[r], min(row0 + 16 * r + c, s.N - 1), kc);
 
     u32x4 xa[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      xa[j] = u32x4{0, 0, 0, 0};
-      if (x_lane && kvalid) {
-        xa[j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)kc * 64 + j * 8);
-        if constexpr (Provider::kPermuteA) xa[j] = permute_a_0415(xa[j]);
-      }
+      xa[j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)kc * 64 + j * 8);
+      if constexpr (Provider::kPermuteA) xa[j] = permute_a_0415(xa[j]);
+      xa[j] = (x_lane && kvalid) ? xa[j] : zero4;
     }
 
+    // Rows past N are computed on a clamped row and never stored; a k-slot past
+    // K must contribute exactly zero, so its operands are zeroed (x is zero
+    // there too, but 0 * inf would not be).
     u32x4 b[R][8];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const bool valid = kvalid && (row0 + 16 * r + c) < s.N;
-      b[r][0] = prov.template operand<0>(raw[r], valid);
-      b[r][1] = prov.template operand<1>(raw[r], valid);
-      b[r][2] = prov.template operand<2>(raw[r], valid);
-      b[r][3] = prov.template operand<3>(raw[r], valid);
-      b[r][4] = prov.template operand<4>(raw[r], valid);
-      b[r][5] = prov.template operand<5>(raw[r], valid);
-      b[r][6] = prov.template operand<6>(raw[r], valid);
-      b[r][7] = prov.template operand<7>(raw[r], valid);
+      b[r][0] = prov.template operand<0>(raw[r]);
+      b[r][1] = prov.template operand<1>(raw[r]);
+      b[r][2] = prov.template operand<2>(raw[r]);
+      b[r][3] = prov.template operand<3>(raw[r]);
+      b[r][4] = prov.template operand<4>(raw[r]);
+      b[r][5] = prov.template operand<5>(raw[r]);
+      b[r][6] = prov.template operand<6>(raw[r]);
+      b[r][7] = prov.template operand<7>(raw[r]);
+    }
+    if (s.chunks & 3) {  // uniform: only shapes with a ragged last step pay for the select
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) b[r][j] = kvalid ? b[r][j] : zero4;
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j)

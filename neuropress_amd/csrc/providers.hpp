@@ -5,9 +5,12 @@
 // eight 16-bit values.  A provider turns the packed bytes of that chunk into
 // those operands:
 //
-//   load(raw, n, kc, valid)   -- global loads of the packed chunk kc of row n
-//   operand<j>(raw, valid)    -- B-operand j (k = 64*kc + 8*j .. +7) in the
-//                                activation dtype, zero when !valid
+//   load(raw, n, kc)   -- global loads of the packed chunk kc of row n
+//   operand<j>(raw)    -- B-operand j (k = 64*kc + 8*j .. +7) in the activation dtype
+//
+// Both are branch-free: the caller passes in-range (clamped) coordinates and
+// discards or zeroes what it does not need.  A predicated load would put every
+// gather behind its own branch and its own wait, serialising them.
 //
 // A B-operand of a VQ weight with VL = 8 is exactly one codebook row, so the
 // 16-byte gather lands in MFMA layout with no shuffling.  For int4 the eight
@@ -38,18 +41,13 @@ struct VqProvider {
   const Args& a;
   __device__ explicit VqProvider(const Args& args) : a(args) {}
 
-  __device__ __forceinline__ void load(Raw& r, int n, int kc, bool valid) const {
-    r.idx = u32x4{0, 0, 0, 0};
-    if (valid) r.idx = load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8);
+  __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
+    r.idx = load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8);
   }
   template <int J>
-  __device__ __forceinline__ u32x4 operand(const Raw& r, bool valid) const {
-    u32x4 c{0, 0, 0, 0};
-    if (valid) {
-      const uint32_t idx = min(idx8_get(r.idx, J), a.nc_minus_1);
-      c = a.cb[idx];
-      if constexpr (CONV) c = cb_to_act<ACT>(c);
-    }
+  __device__ __forceinline__ u32x4 operand(const Raw& r) const {
+    u32x4 c = a.cb[min(idx8_get(r.idx, J), a.nc_minus_1)];
+    if constexpr (CONV) c = cb_to_act<ACT>(c);
     return c;
   }
 };
@@ -78,42 +76,34 @@ struct RvqProvider {
   const Args& a;
   __device__ explicit RvqProvider(const Args& args) : a(args) {}
 
-  __device__ __forceinline__ void load(Raw& r, int n, int kc, bool valid) const {
-    r.im = u32x4{0, 0, 0, 0};
-    r.ir = u32x4{0, 0, 0, 0};
+  __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
+    const int64_t i0 = ((int64_t)n * a.chunks + kc) * 8;
+    r.im = load_idx8<BITS_M>(a.packed_m, i0);
+    r.ir = load_idx8<BITS_R>(a.packed_r, i0);
     r.s2 = 0x3C003C00u;  // 1.0, 1.0
     r.b2 = 0u;
-    if (valid) {
-      const int64_t i0 = ((int64_t)n * a.chunks + kc) * 8;
-      r.im = load_idx8<BITS_M>(a.packed_m, i0);
-      r.ir = load_idx8<BITS_R>(a.packed_r, i0);
-      if (a.row_scale) r.s2 = (uint32_t)a.row_scale[n] * 0x10001u;
-      if (a.row_bias) r.b2 = (uint32_t)a.row_bias[n] * 0x10001u;
-    }
+    if (a.row_scale) r.s2 = (uint32_t)a.row_scale[n] * 0x10001u;  // uniform branches
+    if (a.row_bias) r.b2 = (uint32_t)a.row_bias[n] * 0x10001u;
   }
   template <int J>
-  __device__ __forceinline__ u32x4 operand(const Raw& r, bool valid) const {
+  __device__ __forceinline__ u32x4 operand(const Raw& r) const {
 #pragma clang fp contract(off)
-    u32x4 c{0, 0, 0, 0};
-    if (valid) {
-      const u32x4 cm = a.cb_m[min(idx8_get(r.im, J), a.ncm_minus_1)];
-      const u32x4 cr = a.cb_r[min(idx8_get(r.ir, J), a.ncr_minus_1)];
-      const f16x2 s = __builtin_bit_cast(f16x2, r.s2);
-      const f16x2 b = __builtin_bit_cast(f16x2, r.b2);
-      const bool has_s = a.row_scale != nullptr, has_b = a.row_bias != nullptr;
-      uint32_t o[4];
-      const uint32_t m4[4] = {cm.x, cm.y, cm.z, cm.w};
-      const uint32_t r4[4] = {cr.x, cr.y, cr.z, cr.w};
+    const u32x4 cm = a.cb_m[min(idx8_get(r.im, J), a.ncm_minus_1)];
+    const u32x4 cr = a.cb_r[min(idx8_get(r.ir, J), a.ncr_minus_1)];
+    const f16x2 s = __builtin_bit_cast(f16x2, r.s2);
+    const f16x2 b = __builtin_bit_cast(f16x2, r.b2);
+    const bool has_s = a.row_scale != nullptr, has_b = a.row_bias != nullptr;
+    uint32_t o[4];
+    const uint32_t m4[4] = {cm.x, cm.y, cm.z, cm.w};
+    const uint32_t r4[4] = {cr.x, cr.y, cr.z, cr.w};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        f16x2 h = __builtin_bit_cast(f16x2, m4[i]) + __builtin_bit_cast(f16x2, r4[i]);
-        if (has_s) h = h * s;
-        if (has_b) h = h + b;
-        o[i] = __builtin_bit_cast(uint32_t, h);
-      }
-      c = cb_to_act<ACT>(u32x4{o[0], o[1], o[2], o[3]});
+    for (int i = 0; i < 4; ++i) {
+      f16x2 h = __builtin_bit_cast(f16x2, m4[i]) + __builtin_bit_cast(f16x2, r4[i]);
+      if (has_s) h = h * s;
+      if (has_b) h = h + b;
+      o[i] = __builtin_bit_cast(uint32_t, h);
     }
-    return c;
+    return cb_to_act<ACT>(u32x4{o[0], o[1], o[2], o[3]});
   }
 };
 
@@ -140,23 +130,17 @@ struct Q4Provider {
   const Args& a;
   __device__ explicit Q4Provider(const Args& args) : a(args) {}
 
-  __device__ __forceinline__ void load(Raw& r, int n, int kc, bool valid) const {
-    r.w0 = u32x4{0, 0, 0, 0};
-    r.w1 = u32x4{0, 0, 0, 0};
-    r.s_lo = r.s_hi = 0;
-    if (valid) {
-      const u32x4* p = reinterpret_cast<const u32x4*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 32);
-      r.w0 = p[0];
-      r.w1 = p[1];
-      const uint16_t* s = a.scale + (int64_t)n * a.groups_per_row;
-      r.s_lo = (uint32_t)s[(2 * kc) >> a.gs_shift_chunks] * 0x10001u;
-      r.s_hi = (uint32_t)s[(2 * kc + 1) >> a.gs_shift_chunks] * 0x10001u;
-    }
+  __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
+    const u32x4* p = reinterpret_cast<const u32x4*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 32);
+    r.w0 = p[0];
+    r.w1 = p[1];
+    const uint16_t* s = a.scale + (int64_t)n * a.groups_per_row;
+    r.s_lo = (uint32_t)s[(2 * kc) >> a.gs_shift_chunks] * 0x10001u;
+    r.s_hi = (uint32_t)s[(2 * kc + 1) >> a.gs_shift_chunks] * 0x10001u;
   }
   template <int J>
-  __device__ __forceinline__ u32x4 operand(const Raw& r, bool valid) const {
+  __device__ __forceinline__ u32x4 operand(const Raw& r) const {
 #pragma clang fp contract(off)
-    (void)valid;  // raw words and scales are zero when invalid -> (0-8)*0 = -0: harmless, x is 0 there
     const u32x4& ww = (J < 4) ? r.w0 : r.w1;
     const uint32_t w = (J % 4 == 0) ? ww.x : (J % 4 == 1) ? ww.y : (J % 4 == 2) ? ww.z : ww.w;
     const uint32_t s2 = (J < 4) ? r.s_lo : r.s_hi;

@@ -62,8 +62,13 @@ _LUT_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_LUT_MAX_TOKENS",), 0)
 # Upper end of the tile-decode GEMM band.  NEUROPRESS_VQ_TRITON_MAX_TOKENS is the
 # reference's name for the same knob and is honoured too.  0 disables the band.
 _TILE_MAX_TOKENS: int = _env_int(
-    ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 1024
+    ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 384
 )
+
+# The tile GEMM gives each workgroup 64 output columns (and up to 384 rows), so a
+# layer with few output features leaves most of the GPU idle; below this fraction
+# of the compute units the decode + GEMM band is used instead.
+_TILE_MIN_GRID_FRACTION: float = 0.7
 
 # Opt-in: when a HIP kernel call fails, warn once and run torch ops instead (the
 # reference's behaviour).  Off by default so a missing or broken kernel library
@@ -448,7 +453,11 @@ class NPVQLinear(nn.Module):
                 return self._forward_dequant_gemm(x)  # fp32 activations: decode + GEMM
             m = x.numel() // self.in_features
             if m > _fused_max_tokens(self.backend):
-                if self.backend != VQBackend.CUDA_LUT and m <= _TILE_MAX_TOKENS:
+                if (
+                    self.backend != VQBackend.CUDA_LUT
+                    and m <= _TILE_MAX_TOKENS
+                    and self._tile_grid_fills_gpu(x, m)
+                ):
                     return self._forward_tile_gemm(x)
                 return self._forward_dequant_gemm(x)
         if self.backend == VQBackend.CUDA_LUT:
@@ -460,6 +469,18 @@ class NPVQLinear(nn.Module):
         if self.backend == VQBackend.COMPILE:
             return self._forward_compile(x)
         return self._forward_default(x)
+
+    def _tile_grid_fills_gpu(self, x: torch.Tensor, m: int) -> bool:
+        """True when the tile GEMM's grid (64 columns x up to 384 rows per workgroup)
+        covers at least ``_TILE_MIN_GRID_FRACTION`` of the device's compute units."""
+        if not x.is_cuda:
+            return True
+        cus = self._derived.get("cus")
+        if cus is None:
+            cus = torch.cuda.get_device_properties(x.device).multi_processor_count
+            self._derived["cus"] = cus
+        blocks = -(-self.out_features // 64) * -(-m // 384)
+        return blocks >= _TILE_MIN_GRID_FRACTION * cus
 
     # -- torch-op paths ---------------------------------------------------
 

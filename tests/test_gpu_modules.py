@@ -31,6 +31,7 @@ def _close(y_gpu, y_ref):
 def test_npvqlinear_all_bands_match_default(gpu, act, bits, nc, monkeypatch):
     monkeypatch.setattr(vqmod, "_FUSED_MAX_TOKENS", 16)
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)  # small layers: force the tile band
     L = cases.vq_layer(40 + bits, 96, 256, nc, bits=bits, bias=True, std=0.05)
     ref_layer = NPVQLinear(VQProxy(L["cb"]), L["packed"], bits, 96, 256, 8, "default", bias=L["bias"].float())
     proxy = VQProxy(L["cb"]).to(gpu)
@@ -73,7 +74,7 @@ def test_lowering_auto_runs_hip_backends_on_gpu(gpu):
     m = m.to(gpu)
     assert m.fc.backend.value == "cuda_wmma" and m.q.backend.value == "cuda"
     _close(m(x.to(gpu)), ref)
-    _close(m(torch.cat([x] * 8).to(gpu))[:5], ref)  # 40 tokens: tile bands
+    _close(m(torch.cat([x] * 8).to(gpu))[:5], ref)  # 40 tokens: past the fused band
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
@@ -91,6 +92,7 @@ def test_nplinear_bands(gpu, act, monkeypatch):
 
 def test_residual_module_bands(gpu, monkeypatch):
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)  # small layers: force the tile band
     L = cases.rvq_layer(12, 48, 256, nc_main=65536, nc_res=256)
     mk = lambda backend: NPVQLinear(VQProxy(L["cbm"]), L["pm"], L["bm"], 48, 256, 8, backend,
                                     residual_proxy=VQProxy(L["cbr"]), packed_residual=L["pr"],

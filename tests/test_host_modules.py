@@ -113,6 +113,7 @@ def _fused_layer_with_spies(monkeypatch, backend, lut_max_tokens=16, tile_max_to
     monkeypatch.setattr(vqmod, "_FUSED_MAX_TOKENS", 16)
     monkeypatch.setattr(vqmod, "_LUT_MAX_TOKENS", lut_max_tokens)
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", tile_max_tokens)
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
     lin = _make_linear_with_vq(16, 32)
     layer = NPVQLinear.from_qtensor_linear(lin, VQProxy(lin.weight.qscheme.centroids), backend=backend)
     calls = []
@@ -177,6 +178,7 @@ def test_opt_in_fallback_warns_once_and_latches(monkeypatch, caplog):
     monkeypatch.setattr(vqmod, "_ALLOW_FALLBACK", True)
     monkeypatch.setattr(vqmod, "_tile_failed", False)
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
     monkeypatch.setattr(K, "_warned_fallbacks", set())
     lin = _make_linear_with_vq(16, 32)
     layer = NPVQLinear.from_qtensor_linear(lin, VQProxy(lin.weight.qscheme.centroids), backend="cuda_wmma")
