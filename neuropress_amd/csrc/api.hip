@@ -55,15 +55,20 @@ static int device_cu_count() {
 // HBM round trip, so the plan aims at every job's packed bytes being requested
 // as soon as the grid starts: jobs per wave is kept near jobs / (16 waves * CUs).
 // NPAMD_GEMV_R / NPAMD_GEMV_SPW override the choice (tuning aid).
+bool gemv_lds_codebook_enabled() { return env_int("NPAMD_GEMV_LDS_CB", 1) != 0; }
+
 GemvPlan plan_gemv(int N, int chunks) {
   const int steps = (chunks + 3) / 4;
   const int tiles = (N + 15) / 16;
   const int64_t jobs = (int64_t)tiles * steps;
-  const int64_t target_waves = (int64_t)device_cu_count() * 16;
+  const int cus = device_cu_count();
+  const int64_t target_waves = (int64_t)cus * 16;
   int jpw = (int)((jobs + target_waves - 1) / target_waves);
   if (jpw < 1) jpw = 1;
   GemvPlan p;
-  p.R = (jpw >= 2 && tiles >= 2) ? 2 : 1;
+  // Two row tiles per block share the x operands, but only while that still
+  // leaves at least one block per compute unit.
+  p.R = (jpw >= 2 && tiles >= 2 * cus) ? 2 : 1;
   int spw = (jpw + p.R - 1) / p.R;
   const int r_env = env_int("NPAMD_GEMV_R", 0);
   if (r_env == 1 || r_env == 2 || r_env == 4) p.R = r_env;

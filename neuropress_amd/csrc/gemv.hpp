@@ -36,14 +36,26 @@ struct GemvShape {
 template <int R>
 constexpr int kGemvMaxWaves = (R >= 4) ? 8 : 16;
 
-template <int ACT, class Provider, int R>
+// CB_LDS: the block first copies the whole codebook into LDS and gathers from
+// there (ds_read_b128) instead of from L1/L2.  Pays off when the table is too
+// big for L1 (> 32 KiB) yet fits LDS, or is so small that the copy is free.
+template <int ACT, class Provider, int R, bool CB_LDS>
 __global__ void __launch_bounds__(kGemvMaxWaves<R> * 64)
 fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
-  extern __shared__ float red[];  // [waves][M][16*R]
-  const Provider prov(pargs);
+  extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][M][16*R] (+ codebook copy)
+  Provider prov(pargs);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int n_waves = blockDim.x >> 6;
+  if constexpr (CB_LDS) {
+    // codebook copy lives after the reduction buffer, 16-byte aligned
+    const int red_floats = (n_waves * s.M * 16 * R + 3) & ~3;
+    u32x4* cb_lds = reinterpret_cast<u32x4*>(red + red_floats);
+    const u32x4* src = prov.global_codebook();
+    for (int i = threadIdx.x; i < prov.codebook_rows(); i += blockDim.x) cb_lds[i] = src[i];
+    __syncthreads();
+    prov.use_codebook(cb_lds);
+  }
   const int c = lane & 15;
   const int q = lane >> 4;
   const int row0 = blockIdx.x * (16 * R);
@@ -140,24 +152,48 @@ struct GemvPlan {
 
 GemvPlan plan_gemv(int N, int chunks);
 
-template <int ACT, class Provider, int R>
+// Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
+constexpr int kGemvLdsCodebookMax = 64 * 1024;
+bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
+
+template <int ACT, class Provider, int R, bool CB_LDS>
 int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const GemvPlan& plan,
-                        hipStream_t st, const char* what) {
+                        int cb_bytes, hipStream_t st, const char* what) {
   s.steps_per_wave = plan.steps_per_wave;
   const int blocks = (s.N + 16 * R - 1) / (16 * R);
-  const size_t lds = (size_t)plan.waves * s.M * 16 * R * sizeof(float);
-  fused_gemv_kernel<ACT, Provider, R><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
+  const int red_floats = (plan.waves * s.M * 16 * R + 3) & ~3;
+  const int lds = red_floats * (int)sizeof(float) + (CB_LDS ? cb_bytes : 0);
+  if (lds > 64 * 1024) {
+    static int reserved = 0;  // per instantiation: largest dynamic-LDS size enabled so far
+    if (lds > reserved) {
+      const hipError_t e = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess)
+        return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
+      reserved = lds;
+    }
+  }
+  fused_gemv_kernel<ACT, Provider, R, CB_LDS><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);
 }
 
+// cb_bytes: size of the (single) codebook for providers that can stage it in LDS, else 0.
 template <int ACT, class Provider>
 int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStream_t st,
-                      const char* what) {
+                      const char* what, int cb_bytes = 0) {
   s.steps = (s.chunks + 3) / 4;
   const GemvPlan plan = plan_gemv(s.N, s.chunks);
-  if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4>(s, pargs, plan, st, what);
-  if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2>(s, pargs, plan, st, what);
-  return launch_fused_gemv_r<ACT, Provider, 1>(s, pargs, plan, st, what);
+  if constexpr (Provider::kLdsCodebook) {
+    if (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) {
+      if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true>(s, pargs, plan, cb_bytes, st, what);
+      if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true>(s, pargs, plan, cb_bytes, st, what);
+      return launch_fused_gemv_r<ACT, Provider, 1, true>(s, pargs, plan, cb_bytes, st, what);
+    }
+  }
+  if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, false>(s, pargs, plan, 0, st, what);
+  if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, false>(s, pargs, plan, 0, st, what);
+  return launch_fused_gemv_r<ACT, Provider, 1, false>(s, pargs, plan, 0, st, what);
 }
 
 // ---------------------------------------------------------------------------

@@ -38,15 +38,20 @@ struct VqProvider {
   struct Raw {
     u32x4 idx;
   };
+  static constexpr bool kLdsCodebook = true;  // the codebook may be staged in LDS (use_codebook)
   const Args& a;
-  __device__ explicit VqProvider(const Args& args) : a(args) {}
+  const u32x4* cb;  // where operands are gathered from: global memory, or an LDS copy
+  __device__ explicit VqProvider(const Args& args) : a(args), cb(args.cb) {}
+  __device__ __forceinline__ void use_codebook(const u32x4* p) { cb = p; }
+  __device__ __forceinline__ const u32x4* global_codebook() const { return a.cb; }
+  __device__ __forceinline__ int codebook_rows() const { return (int)a.nc_minus_1 + 1; }
 
   __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
     r.idx = load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8);
   }
   template <int J>
   __device__ __forceinline__ u32x4 operand(const Raw& r) const {
-    u32x4 c = a.cb[min(idx8_get(r.idx, J), a.nc_minus_1)];
+    u32x4 c = cb[min(idx8_get(r.idx, J), a.nc_minus_1)];
     if constexpr (CONV) c = cb_to_act<ACT>(c);
     return c;
   }
@@ -73,6 +78,7 @@ struct RvqProvider {
     u32x4 im, ir;
     uint32_t s2, b2;  // scale / bias replicated in both halves
   };
+  static constexpr bool kLdsCodebook = false;
   const Args& a;
   __device__ explicit RvqProvider(const Args& args) : a(args) {}
 
@@ -127,6 +133,7 @@ struct Q4Provider {
     u32x4 w0, w1;
     uint32_t s_lo, s_hi;  // scale (replicated pair) for operands 0-3 and 4-7
   };
+  static constexpr bool kLdsCodebook = false;
   const Args& a;
   __device__ explicit Q4Provider(const Args& args) : a(args) {}
 

@@ -11,12 +11,12 @@ int run_vq(const VqCall& c, const GemvShape& s) {
     if (c.cb_dtype == NPAMD_F16) {
       using P = VqProvider<ACT, BITS, true>;
       typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-      return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+      return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, c.nc * 16);
     }
   }
   using P = VqProvider<ACT, BITS, false>;
   typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, c.nc * 16);
 }
 
 template <int ACT>
