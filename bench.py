@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="measure only the memory-system ceilings for config 3's access pattern: plain read of "
+                         "the index stream, and one 16-byte table lookup per index for several table sizes")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain device copy of 256 MiB (10 launches): the known-size kernel "
                          "the FETCH_SIZE / WRITE_SIZE counters are scaled against")
@@ -130,6 +133,30 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize(dev)
         print(json.dumps({"calibration": "device copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": 10}))
+        return
+
+    if args.ceilings:
+        n_idx = 14336 * 512
+        n_rot = max(2, POOL_BYTES // (n_idx * 2))
+        g = gen(1003)
+        base = torch.randint(0, 65536, (n_idx,), generator=g, dtype=torch.int32).to(torch.int16).to(dev)
+        pool = [base] + [base.clone() for _ in range(n_rot - 1)]
+        table = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+        st = lambda: torch.cuda.current_stream(dev).cuda_stream
+        out = {"ceilings": "config 3 access pattern, 7 340 032 16-bit indices (14.7 MB), rotating pool",
+               "stream_read_us": round(time_graph(lambda i: _lib.call(
+                   "npamd_diag_stream_read", pool[i].data_ptr(), n_idx * 2, sink.data_ptr(), st()),
+                   n_rot, args.steps, args.warmup, dev), 2)}
+        for entries in (256, 2048, 4096, 16384, 65536):
+            out[f"gather_global_{entries}_rows_us"] = round(time_graph(lambda i: _lib.call(
+                "npamd_diag_gather", pool[i].data_ptr(), n_idx, table.data_ptr(), entries, 0, sink.data_ptr(), st()),
+                n_rot, args.steps, args.warmup, dev), 2)
+        for entries in (256, 4096, 8192):
+            out[f"gather_lds_{entries}_rows_us"] = round(time_graph(lambda i: _lib.call(
+                "npamd_diag_gather", pool[i].data_ptr(), n_idx, table.data_ptr(), entries, 1, sink.data_ptr(), st()),
+                n_rot, args.steps, args.warmup, dev), 2)
+        print(json.dumps(out))
         return
 
     # ---------------- headline: config 3 up/gate, M = 1, fused GEMV -------------

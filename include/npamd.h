@@ -153,6 +153,22 @@ int npamd_q_gemm_tile(const void* x, int64_t ldx, const uint8_t* w_pack, const v
                       int M, int N, int K, int nbits, int group_size, int act_dtype,
                       void* stream);
 
+/* ------------------------------------------------------ diagnostics ---- */
+/*
+ * Memory-system ceilings for the access patterns of the kernels above (no
+ * counterpart in the reference; used by the benchmark to state what bounds the
+ * decode kernels).  Results are discarded; `sink16` is a 16-byte device buffer.
+ *
+ * npamd_diag_stream_read: read `n_bytes` (multiple of 16) once.
+ * npamd_diag_gather: stream `n_indices` uint16 indices (multiple of 8) and fetch
+ *   one 16-byte row of `table16` per index (index masked to `table_entries`, a
+ *   power of two), from global memory or, with from_lds != 0, from an LDS copy
+ *   of the table (at most 8192 rows).
+ */
+int npamd_diag_stream_read(const void* src, int64_t n_bytes, void* sink16, void* stream);
+int npamd_diag_gather(const void* idx_u16, int64_t n_indices, const void* table16,
+                      int table_entries, int from_lds, void* sink16, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

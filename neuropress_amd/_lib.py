@@ -39,6 +39,8 @@ SIGNATURES: dict[str, list] = {
     "npamd_q_dequant": [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _int, _vp],
     "npamd_q_gemv": _Q_LINEAR,
     "npamd_q_gemm_tile": _Q_LINEAR,
+    "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
+    "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],
 }
 
 _lib: ctypes.CDLL | None = None
