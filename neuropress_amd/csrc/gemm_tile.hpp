@@ -20,10 +20,10 @@
 // 32 consecutive rows are bank-conflict free:
 //   x tile  [BM][64 k], double buffered, loaded coalesced by the consumers one
 //           step ahead through registers;
-//   W tile  [64][64 k], double buffered.  Producer q decodes the steps
-//           p == q (mod 4), lane = column.  It keeps kDepth decodes in flight
-//           in registers (issued 4*kDepth iterations before they are consumed)
-//           and writes a finished one to LDS one iteration before its step.
+//   W tile  [64][64 k], double buffered.  Every producer decodes a quarter of
+//           every step's tile (16 columns x 8 operands; lane = column x
+//           operand pair), keeps kDepth steps in flight in registers and
+//           writes a finished pair to LDS one iteration before its step.
 // One block barrier per macro-step, executed by all eight waves.
 #pragma once
 
@@ -47,7 +47,7 @@ struct GemmShape {
   int steps;   // == chunks
 };
 
-constexpr int kDepth = 4;  // decodes in flight per producer wave
+constexpr int kDepth = 8;  // steps in flight per producer wave (2 operands each)
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains
 // every outstanding global load (vmcnt(0)), which would serialise the
@@ -74,10 +74,6 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   const int m0 = blockIdx.y * BM;
   const int n0 = blockIdx.x * kTileCols;
 
-  // Every wave executes the same number of barriers: one after the prologue and
-  // one per iteration t = 0 .. total-1, where the last three iterations are
-  // padding that lets the producers' four-iteration rounds end cleanly.
-  const int total = s.steps + 3;
   // Column blocks walk k in rotated order (iteration t contracts chunk
   // (t + rot) mod steps): at any instant different blocks read different parts
   // of the index rows and of x, which spreads the traffic over the L2 channels
@@ -88,101 +84,68 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     return kc >= s.steps ? kc - s.steps : kc;
   };
 
+  // Both software pipelines are unrolled by their depth with no branches inside
+  // (a branch would make the compiler drain every outstanding load at the join),
+  // so all waves run `total` iterations: steps rounded up to a multiple of kDepth.
+  // The padding iterations decode clamped addresses into buffers nobody reads.
+  const int total = (s.steps + kDepth - 1) / kDepth * kDepth;
+
   if (wave >= 4) {
-    // ====================== producer wave q: steps p == q (mod 4) ==========
-    // Production k of this wave is step q + 4k.  Its "slot" is iteration
-    // q + 4k - 1, the one before the step is consumed.  In slot k the wave
-    //   1. writes production k (gathered kDepth slots ago) to the W buffer,
-    //   2. issues the gathers of production k + kDepth from the packed chunk it
-    //      loaded kDepth slots ago,
-    //   3. loads the packed chunk of production k + 2*kDepth.
-    // Loads are consumed in the order they were issued, so the in-order VMEM
-    // counter never has to drain younger gathers to release an older one.
+    // ====================== producer wave q ================================
+    // Every producer works every iteration on a quarter of the W tile: lane
+    // (col = 16q + l % 16, jp = l / 16) owns operands 2jp and 2jp+1 of its
+    // column, so the decode work (gathers, or int4 dequant VALU) is spread over
+    // all four producers instead of falling on one wave per step.
+    //
+    // Software pipeline, kDepth steps deep, all in registers.  In iteration t
+    // the wave
+    //   1. writes the operands of step t+1 (issued kDepth iterations ago) to LDS,
+    //   2. issues the gathers of step t+1+kDepth from packed bytes loaded kDepth
+    //      iterations ago,
+    //   3. loads the packed bytes of step t+1+2*kDepth.
+    // Loads are consumed in the order they were issued, so waiting for the
+    // oldest never drains the younger ones.
     const Provider prov(pargs);
     const int q = wave - 4;
-    // Branch-free decode: columns past N and productions past the last step
-    // read clamped (valid) addresses; their results land in columns / buffers
-    // nobody consumes.
-    const int ncol = min(n0 + lane, s.N - 1);
-    typename Provider::Raw raws[kDepth];
-    u32x4 ops[kDepth][8];
-    auto load_raw = [&](typename Provider::Raw& raw, int k) {
-      prov.load(raw, ncol, chunk_of(min(q + 4 * k, s.steps - 1)));
+    const int col = 16 * q + (lane & 15);
+    const int jp = lane >> 4;
+    // Branch-free decode: columns past N and steps past the last one read
+    // clamped (valid) addresses; their results land where nobody looks.
+    const int ncol = min(n0 + col, s.N - 1);
+    typename Provider::PairRaw raws[kDepth];
+    u32x4 ops[kDepth][2];
+    auto load_raw = [&](typename Provider::PairRaw& raw, int step) {
+      prov.load_pair(raw, ncol, chunk_of(min(step, s.steps - 1)), jp);
     };
-    auto produce = [&](u32x4 (&b)[8], const typename Provider::Raw& raw) {
-      b[0] = prov.template operand<0>(raw);
-      b[1] = prov.template operand<1>(raw);
-      b[2] = prov.template operand<2>(raw);
-      b[3] = prov.template operand<3>(raw);
-      b[4] = prov.template operand<4>(raw);
-      b[5] = prov.template operand<5>(raw);
-      b[6] = prov.template operand<6>(raw);
-      b[7] = prov.template operand<7>(raw);
+    auto store_w = [&](const u32x4 (&b)[2], int step) {
+      uint8_t* dst = ws + (step & 1) * kWBufBytes + col * kRowBytes + jp * 32;
+      *reinterpret_cast<u32x4*>(dst) = b[0];
+      *reinterpret_cast<u32x4*>(dst + 16) = b[1];
     };
-    auto store_w = [&](const u32x4 (&b)[8], int k) {
-      uint8_t* dst = ws + ((q + 4 * k) & 1) * kWBufBytes + lane * kRowBytes;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(dst + j * 16) = b[j];
-    };
-    int t = 0;  // next iteration whose barrier this wave has not passed yet
-    auto slot = [&](u32x4 (&b)[8], typename Provider::Raw& raw, int k) {
-      store_w(b, k);
-      produce(b, raw);
-      load_raw(raw, k + 2 * kDepth);
-    };
-    auto round = [&](u32x4 (&b)[8], typename Provider::Raw& raw, int k) {  // slot + 3 idle iterations
-      slot(b, raw, k);
-      block_sync_lds();
-      block_sync_lds();
-      block_sync_lds();
-      block_sync_lds();
-      t += 4;
+    auto advance = [&](u32x4 (&b)[2], typename Provider::PairRaw& raw, int t) {
+      store_w(b, t + 1);
+      prov.operand_pair(raw, b[0], b[1]);
+      load_raw(raw, t + 1 + 2 * kDepth);
     };
 
-    // Prologue: productions 0..kDepth-1 in flight, chunks kDepth..2*kDepth-1 loaded.
+    // Prologue: steps 0..kDepth-1 in flight, packed bytes of kDepth..2*kDepth-1
+    // loaded; then "iteration -1": store step 0 and refill its registers.
 #pragma unroll
-    for (int k = 0; k < kDepth; ++k) load_raw(raws[k], k);
+    for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p);
 #pragma unroll
-    for (int k = 0; k < kDepth; ++k) produce(ops[k], raws[k]);
+    for (int p = 0; p < kDepth; ++p) prov.operand_pair(raws[p], ops[p][0], ops[p][1]);
 #pragma unroll
-    for (int k = 0; k < kDepth; ++k) load_raw(raws[k], k + kDepth);
-    // Step 0 is consumed in iteration 0: producer 0 runs its slot 0 now.
-    if (q == 0) slot(ops[0], raws[0], 0);
+    for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p + kDepth);
+    advance(ops[0], raws[0], -1);
     block_sync_lds();
 
-    // Idle until the first slot after the prologue: iteration q - 1 (q >= 1),
-    // or iteration 3 (q == 0, production 1).
-    const int first = (q == 0) ? 3 : q - 1;
-    while (t < first) {
-      block_sync_lds();
-      ++t;
-    }
-    // Rounds of four iterations, unrolled by kDepth so the register sets rotate
-    // statically.  Producer 0 starts at production 1, the others at production 0.
-    if (q == 0) {
-      for (int k = 1; t + 4 <= total; k += 4) {
-        round(ops[1], raws[1], k);
-        if (t + 4 > total) break;
-        round(ops[2], raws[2], k + 1);
-        if (t + 4 > total) break;
-        round(ops[3], raws[3], k + 2);
-        if (t + 4 > total) break;
-        round(ops[0], raws[0], k + 3);
+    // Iteration t handles step t+1, which lives in register set (t+1) % kDepth.
+    for (int t0 = 0; t0 < total; t0 += kDepth) {
+#pragma unroll
+      for (int d = 0; d < kDepth; ++d) {
+        advance(ops[(d + 1) % kDepth], raws[(d + 1) % kDepth], t0 + d);
+        block_sync_lds();
       }
-    } else {
-      for (int k = 0; t + 4 <= total; k += 4) {
-        round(ops[0], raws[0], k);
-        if (t + 4 > total) break;
-        round(ops[1], raws[1], k + 1);
-        if (t + 4 > total) break;
-        round(ops[2], raws[2], k + 2);
-        if (t + 4 > total) break;
-        round(ops[3], raws[3], k + 3);
-      }
-    }
-    while (t < total) {
-      block_sync_lds();
-      ++t;
     }
     return;
   }
@@ -236,20 +199,27 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     }
   };
 
-  // x tile pipeline: the registers loaded during iteration s-1 hold tile s+1;
-  // they are written to LDS at the top of iteration s and immediately reloaded
-  // with tile s+2, so every global load has a full iteration to land.
-  u32x4 xr[kPieces];
-  load_x(xr, 0);
-  store_x(xr, 0);
-  if (s.steps > 1) load_x(xr, 1);
+  // x tile pipeline: kXDepth register sets hold the tiles of the next steps in
+  // flight (a global load takes longer than one iteration).  Step p lives in
+  // set p % kXDepth; iteration t writes tile t+1 to LDS and reloads its set
+  // with tile t+1+kXDepth.
+  constexpr int kXDepth = (MW == 1) ? 4 : 2;  // divides kDepth, so `total` suits both loops
+  u32x4 xr[kXDepth][kPieces];
+  load_x(xr[0], 0);
+  store_x(xr[0], 0);
+#pragma unroll
+  for (int p = 1; p <= kXDepth; ++p) load_x(xr[p % kXDepth], min(p, s.steps - 1));
   block_sync_lds();
 
-  for (int step = 0; step < total; ++step) {
-    if (step + 1 < s.steps) store_x(xr, (step + 1) & 1);
-    if (step + 2 < s.steps) load_x(xr, step + 2);
-    if (wave_active && step < s.steps) mma(step);
-    block_sync_lds();
+  for (int t0 = 0; t0 < total; t0 += kXDepth) {
+#pragma unroll
+    for (int d = 0; d < kXDepth; ++d) {
+      const int step = t0 + d;
+      store_x(xr[(d + 1) % kXDepth], (step + 1) & 1);
+      load_x(xr[(d + 1) % kXDepth], min(step + 1 + kXDepth, s.steps - 1));
+      if (wave_active && step < s.steps) mma(step);
+      block_sync_lds();
+    }
   }
 
   // ---- epilogue: D[m = 8*(i/4) + 4h + i%4][n = c] --------------------------

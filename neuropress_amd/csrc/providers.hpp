@@ -12,6 +12,12 @@
 // discards or zeroes what it does not need.  A predicated load would put every
 // gather behind its own branch and its own wait, serialising them.
 //
+// The tile GEMM splits a chunk four ways: lane-group jp (0..3) of a producer
+// wave owns operands 2*jp and 2*jp+1 of its column:
+//
+//   load_pair(raw, n, kc, jp)     -- packed bytes for that operand pair
+//   operand_pair(raw, b0, b1)     -- the two operands
+//
 // A B-operand of a VQ weight with VL = 8 is exactly one codebook row, so the
 // 16-byte gather lands in MFMA layout with no shuffling.  For int4 the eight
 // nibbles of one dword are one operand, produced in the k-order
@@ -21,6 +27,13 @@
 #include "common.hpp"
 
 namespace npamd {
+
+// Dword jp (lane-varying, 0..3) of a four-dword vector.
+__device__ __forceinline__ uint32_t select_dword(const u32x4& v, int jp) {
+  const uint32_t lo = (jp & 1) ? v.y : v.x;
+  const uint32_t hi = (jp & 1) ? v.w : v.z;
+  return (jp & 2) ? hi : lo;
+}
 
 // ---------------------------------------------------------------------------
 // Single-codebook VQ, VL = 8, fast index widths.
@@ -54,6 +67,22 @@ struct VqProvider {
     u32x4 c = cb[min(idx8_get(r.idx, J), a.nc_minus_1)];
     if constexpr (CONV) c = cb_to_act<ACT>(c);
     return c;
+  }
+
+  struct PairRaw {
+    uint32_t pair;  // indices of operands 2*jp (low half) and 2*jp+1 (high half)
+  };
+  __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
+    // the four lane-groups of a column read the same 8-index group: one request
+    r.pair = select_dword(load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8), jp);
+  }
+  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
+    b0 = cb[min(r.pair & 0xFFFFu, a.nc_minus_1)];
+    b1 = cb[min(r.pair >> 16, a.nc_minus_1)];
+    if constexpr (CONV) {
+      b0 = cb_to_act<ACT>(b0);
+      b1 = cb_to_act<ACT>(b1);
+    }
   }
 };
 
@@ -93,11 +122,32 @@ struct RvqProvider {
   }
   template <int J>
   __device__ __forceinline__ u32x4 operand(const Raw& r) const {
+    return combine(idx8_get(r.im, J), idx8_get(r.ir, J), r.s2, r.b2);
+  }
+
+  struct PairRaw {
+    uint32_t pm, pr, s2, b2;
+  };
+  __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
+    const int64_t i0 = ((int64_t)n * a.chunks + kc) * 8;
+    r.pm = select_dword(load_idx8<BITS_M>(a.packed_m, i0), jp);
+    r.pr = select_dword(load_idx8<BITS_R>(a.packed_r, i0), jp);
+    r.s2 = 0x3C003C00u;
+    r.b2 = 0u;
+    if (a.row_scale) r.s2 = (uint32_t)a.row_scale[n] * 0x10001u;
+    if (a.row_bias) r.b2 = (uint32_t)a.row_bias[n] * 0x10001u;
+  }
+  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
+    b0 = combine(r.pm & 0xFFFFu, r.pr & 0xFFFFu, r.s2, r.b2);
+    b1 = combine(r.pm >> 16, r.pr >> 16, r.s2, r.b2);
+  }
+
+  __device__ __forceinline__ u32x4 combine(uint32_t im, uint32_t ir, uint32_t s2, uint32_t b2) const {
 #pragma clang fp contract(off)
-    const u32x4 cm = a.cb_m[min(idx8_get(r.im, J), a.ncm_minus_1)];
-    const u32x4 cr = a.cb_r[min(idx8_get(r.ir, J), a.ncr_minus_1)];
-    const f16x2 s = __builtin_bit_cast(f16x2, r.s2);
-    const f16x2 b = __builtin_bit_cast(f16x2, r.b2);
+    const u32x4 cm = a.cb_m[min(im, a.ncm_minus_1)];
+    const u32x4 cr = a.cb_r[min(ir, a.ncr_minus_1)];
+    const f16x2 s = __builtin_bit_cast(f16x2, s2);
+    const f16x2 b = __builtin_bit_cast(f16x2, b2);
     const bool has_s = a.row_scale != nullptr, has_b = a.row_bias != nullptr;
     uint32_t o[4];
     const uint32_t m4[4] = {cm.x, cm.y, cm.z, cm.w};
@@ -147,10 +197,28 @@ struct Q4Provider {
   }
   template <int J>
   __device__ __forceinline__ u32x4 operand(const Raw& r) const {
-#pragma clang fp contract(off)
     const u32x4& ww = (J < 4) ? r.w0 : r.w1;
     const uint32_t w = (J % 4 == 0) ? ww.x : (J % 4 == 1) ? ww.y : (J % 4 == 2) ? ww.z : ww.w;
-    const uint32_t s2 = (J < 4) ? r.s_lo : r.s_hi;
+    return dequant8(w, (J < 4) ? r.s_lo : r.s_hi);
+  }
+
+  struct PairRaw {
+    u32x2 w;      // 16 nibbles = operands 2*jp, 2*jp+1
+    uint32_t s2;  // their scale (one 32-k group), replicated
+  };
+  __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
+    r.w = *reinterpret_cast<const u32x2*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 32 + jp * 8);
+    const uint16_t* s = a.scale + (int64_t)n * a.groups_per_row;
+    r.s2 = (uint32_t)s[(2 * kc + (jp >> 1)) >> a.gs_shift_chunks] * 0x10001u;
+  }
+  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
+    b0 = dequant8(r.w.x, r.s2);
+    b1 = dequant8(r.w.y, r.s2);
+  }
+
+  // Eight nibbles of one dword -> one operand, k-order (0,4,1,5,2,6,3,7).
+  __device__ __forceinline__ u32x4 dequant8(uint32_t w, uint32_t s2) const {
+#pragma clang fp contract(off)
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

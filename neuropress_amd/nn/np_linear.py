@@ -34,7 +34,11 @@ from .backends import Backend, LinearBackend, is_hip_backend_available
 log = logging.getLogger(__name__)
 
 # Upper end of the fused-GEMM band for the int4 path; above it decode + GEMM.
-_Q_TILE_MAX_TOKENS: int = int(os.environ.get("NEUROPRESS_Q_TILE_MAX_TOKENS", "1024"))
+# Measured on one MI355X (14336 x 4096, group 32): fused GEMM 38-42 us up to 128
+# tokens and 72 us at 256 against 56-62 / 78 us for decode + GEMM; 104 vs 84 us at 384.
+_Q_TILE_MAX_TOKENS: int = int(os.environ.get("NEUROPRESS_Q_TILE_MAX_TOKENS", "256"))
+# As for the VQ path: narrow layers leave most compute units idle in the fused GEMM.
+_Q_TILE_MIN_GRID_FRACTION: float = 0.7
 _Q_FUSED_MAX_TOKENS: int = 16
 
 _ALLOW_FALLBACK: bool = os.environ.get("NEUROPRESS_ALLOW_KERNEL_FALLBACK", "").strip() in (
@@ -258,6 +262,14 @@ class NPLinear(nn.Module):
             self._bias_as(x.dtype),
         )
 
+    def _tile_grid_fills_gpu(self, x: torch.Tensor, m: int) -> bool:
+        cus = self._derived.get("cus")
+        if cus is None:
+            cus = torch.cuda.get_device_properties(x.device).multi_processor_count
+            self._derived["cus"] = cus
+        blocks = -(-self.out_features // 64) * -(-m // 384)
+        return blocks >= _Q_TILE_MIN_GRID_FRACTION * cus
+
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:
         """HIP path by token count; takes the place of np_linear.py:731-761."""
         if not x.is_cuda:
@@ -266,7 +278,10 @@ class NPLinear(nn.Module):
 
         m = x.numel() // self.in_features
         try:
-            if x.dtype in (torch.float16, torch.bfloat16) and m <= _Q_TILE_MAX_TOKENS:
+            fused_ok = x.dtype in (torch.float16, torch.bfloat16)
+            if fused_ok and m > _Q_FUSED_MAX_TOKENS:
+                fused_ok = m <= _Q_TILE_MAX_TOKENS and self._tile_grid_fills_gpu(x, m)
+            if fused_ok:
                 if m <= _Q_FUSED_MAX_TOKENS:
                     return kernels.q_linear(
                         x, self.u8_blob, self.scale, self.nbits, self.group_size,

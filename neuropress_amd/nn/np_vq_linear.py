@@ -61,8 +61,11 @@ _LUT_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_LUT_MAX_TOKENS",), 0)
 
 # Upper end of the tile-decode GEMM band.  NEUROPRESS_VQ_TRITON_MAX_TOKENS is the
 # reference's name for the same knob and is honoured too.  0 disables the band.
+# Measured on one MI355X (14336 x 4096 layer): the tile GEMM beats decode + GEMM
+# from 17 to about 320 tokens (58 vs 67 us at 64, 74 vs 86 us at 256, 100 vs 96 us
+# at 384, 190 vs 101 us at 512, where a second row block re-decodes the weight).
 _TILE_MAX_TOKENS: int = _env_int(
-    ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 384
+    ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 256
 )
 
 # The tile GEMM gives each workgroup 64 output columns (and up to 384 rows), so a

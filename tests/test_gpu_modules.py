@@ -82,6 +82,7 @@ def test_nplinear_bands(gpu, act, monkeypatch):
     import neuropress_amd.nn.np_linear as qmod
 
     monkeypatch.setattr(qmod, "_Q_TILE_MAX_TOKENS", 64)
+    monkeypatch.setattr(qmod, "_Q_TILE_MIN_GRID_FRACTION", 0.0)  # small layer: force the fused GEMM band
     Q = cases.q4_layer(8, 80, 256, bias=True)
     layer = NPLinear(Q["blob"], Q["scale"], 80, 256, 32, 4, "sym", "cuda", bias=Q["bias"].float()).to(gpu)
     w = ((Q["codes"].float() - 8).reshape(80, 8, 32) * Q["scale"].float().reshape(80, 8, 1)).reshape(80, 256)
