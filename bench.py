@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
+    ap.add_argument("--case", default="", choices=["", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "dequant", "q4_gemv_m1", "q4_tile_m128"],
+                    help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
+                         "on the config-3 / config-5 shape and print a one-line JSON with its HIP-event time")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure only the memory-system ceilings for config 3's access pattern: plain read of "
                          "the index stream, and one 16-byte table lookup per index for several table sizes")
@@ -133,6 +136,54 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize(dev)
         print(json.dumps({"calibration": "device copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": 10}))
+        return
+
+    if args.case:
+        from neuropress_amd.t2n.packing import BitPacking4
+        from neuropress_amd.transforms.vq_packing import IndexPacking
+
+        n, k = 14336, 4096
+        g = gen(1003)
+        n_rot = 8
+        if args.case.startswith("q4"):
+            blob = BitPacking4.compress(torch.randint(0, 16, (n, k), generator=g, dtype=torch.int64).to(torch.uint8))
+            sc = (torch.rand(n * k // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
+            pool = [blob.to(dev).clone() for _ in range(n_rot)]
+            m = 1 if args.case == "q4_gemv_m1" else 128
+            x = torch.randn(m, k, generator=g).to(torch.float16).to(dev)
+            fn = lambda i: kernels.q_linear(x, pool[i], sc, 4, 32)
+            alg, flops = n * k // 2 + n * k // 32 * 2 + m * k * 2 + m * n * 2, 2.0 * m * n * k
+        else:
+            nc, bits = (4096, 12) if args.case == "gemv_nc4096_m1" else (65536, 16)
+            cb = (torch.randn(nc, 8, generator=g) * 0.02).to(torch.float16)
+            if bits == 16:
+                base = torch.randint(0, 65536, (n * k // 8,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8)
+            else:
+                base = IndexPacking.pack(torch.randint(0, nc, (n * k // 8,), generator=g), bits)
+            pool = [base.to(dev).clone() for _ in range(n_rot)]
+            cb16, cbb = cb.to(dev), cb.to(torch.bfloat16).to(dev)
+            m = 256 if args.case == "tile_m256" else 1
+            x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
+            if args.case == "tile_m256":
+                fn = lambda i: kernels.vq_gemm_tile(x, pool[i], cbb, bits, n, None)
+            elif args.case == "dequant":
+                fn = lambda i: kernels.vq_dequant(pool[i], cb16, bits, n, k, torch.bfloat16)
+            else:
+                fn = lambda i: kernels.vq_linear(x, pool[i], cbb, bits, 8, None, n)
+            alg = base.numel() + nc * 16 + m * k * 2 + m * n * 2 + (n * k * 2 if args.case == "dequant" else 0)
+            flops = 2.0 * m * n * k
+        for i in range(args.warmup):
+            fn(i % n_rot)
+        torch.cuda.synchronize(dev)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            fn(i % n_rot)
+        e1.record()
+        torch.cuda.synchronize(dev)
+        us = e0.elapsed_time(e1) * 1e3 / args.steps
+        print(json.dumps({"case": args.case, "steps": args.steps, "us_per_launch_incl_python": round(us, 2),
+                          "algorithmic_bytes": alg, "flops": flops}))
         return
 
     if args.ceilings:
