@@ -91,6 +91,74 @@ int npamd_vq_gemm_tile(const void* x, int64_t ldx, const uint8_t* packed, int64_
 int npamd_vq_widen_u16(const uint8_t* packed, int64_t n_bytes, int bits,
                        int64_t n_indices, uint16_t* out, void* stream);
 
+/* ------------------------------------- slice-list form of the indices ---- */
+/*
+ * For codebooks too large for a compute unit's LDS (more than 4096 rows) the
+ * decode GEMV is bound by random 16-byte codebook lookups in L2.  The slice-list
+ * form files every index under the 8192-row codebook slice it points into, so a
+ * workgroup that holds one slice in LDS only sees the lookups that hit it; every
+ * lane sums the entries of one output row in a register.  It is
+ * built once per layer from the packed stream (a construction-time re-layout,
+ * as the reference pre-unpacks embedding indices to an int16 table,
+ * neuropress/nn/np_vq_embedding.py:244-246) and used by npamd_vq_gemv_sliced.
+ * The format itself has no counterpart in the reference.
+ *
+ * The blob starts with this header; the rest is described in
+ * neuropress_amd/csrc/sliced_format.hpp.  All offsets are bytes from the start.
+ */
+typedef struct npamd_sliced_header {
+  uint32_t magic;         /* "NPSL" */
+  uint32_t version;
+  int32_t n, k, vl, nc;   /* the layer the blob was built for */
+  int32_t slice_rows;     /* codebook rows per slice */
+  int32_t n_slices;
+  int32_t n_workgroups;   /* grid size of the GEMV */
+  int32_t n_partials;     /* partial-sum vectors per output row */
+  int32_t groups_max;     /* largest group range of a workgroup */
+  int32_t reserved32;
+  int64_t n_quads;        /* 768-byte entry quads */
+  int64_t n_entries;      /* real (non-padding) entries = N * K / VL */
+  int64_t off_workgroups, off_rowmap, off_entries;
+  int64_t total_bytes;
+  int64_t reserved[4];
+} npamd_sliced_header;
+
+/*
+ * HOST function: build the slice-list blob from a packed index stream in host
+ * memory.  `target_workgroups` = compute units to fill (0 = 256).  Writes the
+ * size to *blob_bytes; if `blob` is NULL or `capacity` is too small nothing else
+ * is written and NPAMD_ERR_INVALID is returned when blob != NULL.
+ * Call once with blob = NULL for the size, then with a buffer.  VL must be 8.
+ */
+int npamd_vq_sliced_build(const uint8_t* packed_host, int64_t n_bytes, int bits,
+                          int N, int K, int vl, int nc, int target_workgroups,
+                          void* blob_host, int64_t capacity, int64_t* blob_bytes);
+
+/*
+ * HOST function: structural check of a blob in host memory (offsets inside
+ * total_bytes, every row / group / slice field in range, every index filed
+ * exactly once).  A blob that passes cannot make
+ * npamd_vq_gemv_sliced read outside the blob, the codebook or its LDS arrays.
+ */
+int npamd_vq_sliced_check(const void* blob_host, int64_t blob_bytes);
+
+/* Bytes of f32 workspace npamd_vq_gemv_sliced needs for M tokens. */
+int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, int M);
+
+/*
+ * Decode GEMV over the slice-list form, M <= NPAMD_GEMV_MAX_M (tokens are
+ * processed one after the other):
+ *   y[m, n] = sum_k x[m, k] * codebook[idx(n, k/VL), k%VL] (+ bias[n]).
+ * `header_host` is a host copy of the blob's header, `blob` the whole blob in
+ * device memory.  The codebook must be in the activation dtype.  `workspace`
+ * is device memory of npamd_vq_sliced_workspace_bytes() bytes, 16-byte aligned,
+ * contents irrelevant before and after.
+ */
+int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_sliced_header* header_host,
+                         const void* blob, const void* codebook, int codebook_dtype,
+                         const float* bias, void* y, int64_t ldy, int M, int act_dtype,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------- residual VQ (RVQ) ---- */
 /*
  * Two codebooks + per-output-row fp16 scale and bias (no counterpart in the

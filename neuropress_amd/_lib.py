@@ -32,6 +32,11 @@ SIGNATURES: dict[str, list] = {
     "npamd_vq_gemv": _VQ_LINEAR,
     "npamd_vq_gemm_tile": _VQ_LINEAR,
     "npamd_vq_widen_u16": [_vp, _i64, _int, _i64, _vp, _vp],
+    "npamd_vq_sliced_build": [_vp, _i64, _int, _int, _int, _int, _int, _int, _vp, _i64,
+                              ctypes.POINTER(_i64)],  # fmt: skip
+    "npamd_vq_sliced_check": [_vp, _i64],
+    "npamd_vq_sliced_workspace_bytes": [_vp, _int],
+    "npamd_vq_gemv_sliced": [_vp, _i64, _vp, _vp, _vp, _int, _vp, _vp, _i64, _int, _int, _vp, _i64, _vp],
     "npamd_rvq_dequant": [_vp, _i64, _int, _vp, _i64, _int, _vp, _int, _vp, _int, _vp, _vp, _int,
                           _int, _int, _vp, _int, _vp],  # fmt: skip
     "npamd_rvq_gemv": _RVQ_LINEAR,
@@ -42,6 +47,9 @@ SIGNATURES: dict[str, list] = {
     "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
     "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],
 }
+
+_RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64}
+SLICED_HEADER_BYTES = 128
 
 _lib: ctypes.CDLL | None = None
 _load_error: str | None = None
@@ -63,7 +71,7 @@ def load() -> ctypes.CDLL:
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
-            fn.restype = _int
+            fn.restype = _RESTYPES.get(name, _int)
         if lib.npamd_version() != ABI_VERSION:
             raise OSError(f"libnpamd ABI version {lib.npamd_version()} != expected {ABI_VERSION}")
     except (OSError, AttributeError) as exc:

@@ -1,0 +1,307 @@
+// Host-side builder and checker of the slice-list form (see sliced_format.hpp).
+// Nothing in this file touches the GPU.
+#include <string.h>
+
+#include <algorithm>
+#include <numeric>
+#include <vector>
+
+#include "common.hpp"
+#include "sliced_format.hpp"
+
+using namespace npamd;
+
+namespace {
+
+inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+inline uint32_t host_read_index(const uint8_t* packed, int64_t n_bytes, int64_t i, int bits) {
+  const int64_t bit = i * (int64_t)bits;
+  const int64_t b0 = bit >> 3;
+  const int off = (int)(bit & 7);
+  uint64_t w = 0;
+  for (int j = 0; j < 4; ++j)
+    if (b0 + j < n_bytes) w |= (uint64_t)packed[b0 + j] << (8 * j);
+  return (uint32_t)((w >> off) & ((1u << bits) - 1u));
+}
+
+inline void put_entry24(uint8_t* quad_lane, int j, uint32_t e) {
+  quad_lane[3 * j + 0] = (uint8_t)(e & 0xFF);
+  quad_lane[3 * j + 1] = (uint8_t)((e >> 8) & 0xFF);
+  quad_lane[3 * j + 2] = (uint8_t)((e >> 16) & 0xFF);
+}
+
+inline uint32_t get_entry24(const uint8_t* quad_lane, int j) {
+  return (uint32_t)quad_lane[3 * j] | ((uint32_t)quad_lane[3 * j + 1] << 8) |
+         ((uint32_t)quad_lane[3 * j + 2] << 16);
+}
+
+inline int lds_bytes_needed(int slice_rows, int groups_max) { return slice_rows * 16 + (groups_max + 1) * 16; }
+
+// How the layer is cut: `row_blocks` row ranges of `rows_per_block` rows, and per
+// slice `parts[s]` group ranges.  One workgroup per (slice, group range, row block).
+struct Geometry {
+  int row_blocks = 1, rows_per_block = 1;
+  std::vector<int> parts;
+  int64_t workgroups = 0;
+};
+
+Geometry plan_geometry(int N, int G, const std::vector<int64_t>& slice_count, int64_t n_idx, int target) {
+  const int S = (int)slice_count.size();
+  const int rb_min = (N + kSlicedTasks - 1) / kSlicedTasks;
+  const int kp_min = (G + kSlicedMaxGroups - 1) / kSlicedMaxGroups;
+  Geometry best;
+  double best_cost = 0;
+  for (int rb = rb_min; rb <= 2 * rb_min + 1; ++rb) {
+    Geometry geo;
+    geo.row_blocks = rb;
+    geo.rows_per_block = (N + rb - 1) / rb;
+    geo.parts.resize((size_t)S);
+    double heaviest = 0;
+    for (int s = 0; s < S; ++s) {
+      const double share = (double)slice_count[s] / (double)n_idx;
+      // Group ranges in proportion to the slice's load, but no finer than about
+      // 16 entries per row and range: a workgroup pays for loading its slice.
+      const int kp_max = std::max(kp_min, (int)((double)G * share / 16.0));
+      int kp = (int)((double)target * share / rb + 0.5);
+      kp = std::max(kp_min, std::min(kp, kp_max));
+      geo.parts[s] = kp;
+      geo.workgroups += (int64_t)kp * rb;
+      heaviest = std::max(heaviest, share / ((double)kp * rb));
+    }
+    // Rounds of workgroups over the compute units times the heaviest workgroup,
+    // plus a charge per round for loading a slice.
+    const double rounds = (double)((geo.workgroups + target - 1) / target);
+    const double cost = rounds * (heaviest + 0.25 / (double)target);
+    if (best.workgroups == 0 || cost < best_cost - 1e-12) {
+      best = geo;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+}  // namespace
+
+extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int bits, int N, int K,
+                                     int vl, int nc, int target_workgroups, void* blob,
+                                     int64_t capacity, int64_t* blob_bytes) {
+  const char* what = "npamd_vq_sliced_build";
+  NPAMD_REQUIRE(blob_bytes != nullptr, "%s: blob_bytes is null", what);
+  NPAMD_REQUIRE(vl == 8, "%s: the slice-list form needs VL = 8 (got %d)", what, vl);
+  NPAMD_REQUIRE(bits >= 4 && bits <= 20, "%s: bits must be in [4, 20], got %d", what, bits);
+  NPAMD_REQUIRE(N > 0 && K > 0 && nc >= 1, "%s: bad shape N=%d K=%d NC=%d", what, N, K, nc);
+  NPAMD_REQUIRE(K % vl == 0, "%s: K=%d not divisible by VL=%d", what, K, vl);
+  const int G = K / vl;
+  const int64_t n_idx = (int64_t)N * G;
+  NPAMD_REQUIRE(packed != nullptr && (n_idx * bits + 7) / 8 <= n_bytes, "%s: packed buffer too short", what);
+  if (target_workgroups <= 0) target_workgroups = 256;
+
+  const int slice_rows = kSlicedMaxSliceRows;
+  const int S = (nc + slice_rows - 1) / slice_rows;
+
+  // Indices transposed to [G][N] so a (group, row range) scan is contiguous.
+  std::vector<uint32_t> idx_t((size_t)n_idx);
+  std::vector<int64_t> slice_count((size_t)S, 0);
+  for (int n = 0; n < N; ++n)
+    for (int g = 0; g < G; ++g) {
+      uint32_t v = host_read_index(packed, n_bytes, (int64_t)n * G + g, bits);
+      if (v > (uint32_t)nc - 1u) v = (uint32_t)nc - 1u;  // same clamp as the decode kernels
+      idx_t[(size_t)g * N + n] = v;
+      slice_count[v / slice_rows]++;
+    }
+
+  const Geometry geo = plan_geometry(N, G, slice_count, n_idx, target_workgroups);
+  std::vector<int> partial_base((size_t)S);
+  int n_partials = 0;
+  for (int s = 0; s < S; ++s) {
+    partial_base[s] = n_partials;
+    n_partials += geo.parts[s];
+  }
+
+  // Workgroups, dealt round-robin over the slices so that workgroup id mod 8
+  // (the XCD it lands on) tends to see one slice only.
+  struct Job { int slice, part, block; };
+  std::vector<Job> jobs;
+  {
+    std::vector<std::vector<Job>> per_slice((size_t)S);
+    for (int s = 0; s < S; ++s)
+      for (int kp = 0; kp < geo.parts[s]; ++kp)
+        for (int rb = 0; rb < geo.row_blocks; ++rb) per_slice[s].push_back(Job{s, kp, rb});
+    size_t remaining = 0;
+    for (auto& v : per_slice) remaining += v.size();
+    for (size_t j = 0; remaining > 0; ++j)
+      for (int s = 0; s < S; ++s)
+        if (j < per_slice[s].size()) {
+          jobs.push_back(per_slice[s][j]);
+          --remaining;
+        }
+  }
+  const int n_wg = (int)jobs.size();
+
+  std::vector<SlicedWorkgroup> wgs((size_t)n_wg);
+  std::vector<uint32_t> rowmap((size_t)n_wg * kSlicedTasks, kSlicedNoRow);
+  std::vector<uint8_t> quads;
+  std::vector<std::vector<uint32_t>> task((size_t)geo.rows_per_block);
+  std::vector<int> order;
+  int64_t real_entries = 0;
+  int groups_max = 1;
+
+  for (int w = 0; w < n_wg; ++w) {
+    const Job& job = jobs[w];
+    SlicedWorkgroup& wg = wgs[w];
+    memset(&wg, 0, sizeof(wg));
+    const int g_begin = (int)((int64_t)G * job.part / geo.parts[job.slice]);
+    const int g_end = (int)((int64_t)G * (job.part + 1) / geo.parts[job.slice]);
+    const int row0 = job.block * geo.rows_per_block;
+    const int rows = std::max(0, std::min(geo.rows_per_block, N - row0));
+    wg.slice = (uint32_t)job.slice;
+    wg.partial = (uint32_t)(partial_base[job.slice] + job.part);
+    wg.g_begin = (uint32_t)g_begin;
+    wg.g_count = (uint32_t)(g_end - g_begin);
+    groups_max = std::max(groups_max, g_end - g_begin);
+
+    for (int r = 0; r < rows; ++r) task[(size_t)r].clear();
+    for (int g = g_begin; g < g_end; ++g) {
+      const uint32_t* col = &idx_t[(size_t)g * N + row0];
+      for (int r = 0; r < rows; ++r) {
+        const uint32_t v = col[r];
+        if ((int)(v / slice_rows) == job.slice)
+          task[(size_t)r].push_back((uint32_t)(g - g_begin) | ((v % slice_rows) << 11));
+      }
+    }
+    // Longest tasks first; 64 neighbours in that order share a strip.
+    order.resize((size_t)rows);
+    std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int a, int b) { return task[(size_t)a].size() > task[(size_t)b].size(); });
+    const uint32_t pad = wg.g_count;  // zero activation vector, slice row 0
+    for (int s = 0; s * 64 < rows; ++s) {
+      const int first = s * 64;
+      const int lanes = std::min(64, rows - first);
+      const int64_t steps = (int64_t)task[(size_t)order[(size_t)first]].size();
+      const int64_t nq = (steps + 3) / 4;
+      wg.wave[s].quad_begin = nq ? (uint32_t)(quads.size() / kSlicedQuadBytes) : 0u;
+      wg.wave[s].steps = (uint32_t)steps;
+      const size_t base = quads.size();
+      quads.resize(base + (size_t)nq * kSlicedQuadBytes);
+      for (int lane = 0; lane < 64; ++lane) {
+        const std::vector<uint32_t>* t = nullptr;
+        if (lane < lanes) {
+          const int r = order[(size_t)(first + lane)];
+          t = &task[(size_t)r];
+          rowmap[(size_t)w * kSlicedTasks + (size_t)s * 64 + lane] = (uint32_t)(row0 + r);
+          real_entries += (int64_t)t->size();
+        }
+        for (int64_t i = 0; i < nq * 4; ++i) {
+          const uint32_t e = (t && i < (int64_t)t->size()) ? (*t)[(size_t)i] : pad;
+          put_entry24(&quads[base + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12], (int)(i % 4), e);
+        }
+      }
+    }
+  }
+  if (quads.empty()) quads.resize(kSlicedQuadBytes, 0);  // waves without a strip still load quad 0
+
+  npamd_sliced_header h;
+  memset(&h, 0, sizeof(h));
+  h.magic = kSlicedMagic;
+  h.version = kSlicedVersion;
+  h.n = N; h.k = K; h.vl = vl; h.nc = nc;
+  h.slice_rows = slice_rows;
+  h.n_slices = S;
+  h.n_workgroups = n_wg;
+  h.n_partials = n_partials;
+  h.groups_max = groups_max;
+  h.n_quads = (int64_t)(quads.size() / kSlicedQuadBytes);
+  h.n_entries = real_entries;
+  h.off_workgroups = sizeof(h);
+  h.off_rowmap = align_up(h.off_workgroups + (int64_t)n_wg * (int64_t)sizeof(SlicedWorkgroup), 256);
+  h.off_entries = align_up(h.off_rowmap + (int64_t)rowmap.size() * 4, 256);
+  h.total_bytes = align_up(h.off_entries + (int64_t)quads.size(), 256);
+  *blob_bytes = h.total_bytes;
+  if (blob == nullptr) return NPAMD_OK;
+  NPAMD_REQUIRE(capacity >= h.total_bytes, "%s: buffer of %lld bytes, %lld needed", what,
+                (long long)capacity, (long long)h.total_bytes);
+  uint8_t* out = (uint8_t*)blob;
+  memset(out, 0, (size_t)h.total_bytes);
+  memcpy(out, &h, sizeof(h));
+  memcpy(out + h.off_workgroups, wgs.data(), wgs.size() * sizeof(SlicedWorkgroup));
+  memcpy(out + h.off_rowmap, rowmap.data(), rowmap.size() * 4);
+  memcpy(out + h.off_entries, quads.data(), quads.size());
+  return NPAMD_OK;
+}
+
+extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
+  const char* what = "npamd_vq_sliced_check";
+  NPAMD_REQUIRE(blob != nullptr && blob_bytes >= (int64_t)sizeof(npamd_sliced_header), "%s: blob too short", what);
+  npamd_sliced_header h;
+  memcpy(&h, blob, sizeof(h));
+  NPAMD_REQUIRE(h.magic == kSlicedMagic && h.version == kSlicedVersion, "%s: not a slice-list blob (magic/version)", what);
+  NPAMD_REQUIRE(h.total_bytes <= blob_bytes, "%s: blob holds %lld bytes, header says %lld", what,
+                (long long)blob_bytes, (long long)h.total_bytes);
+  NPAMD_REQUIRE(h.n > 0 && h.k > 0 && h.vl == 8 && h.nc >= 1 && h.k % 8 == 0, "%s: bad layer shape", what);
+  NPAMD_REQUIRE(h.slice_rows >= 1 && h.slice_rows <= kSlicedMaxSliceRows &&
+                    h.n_slices == (h.nc + h.slice_rows - 1) / h.slice_rows,
+                "%s: bad slice geometry", what);
+  NPAMD_REQUIRE(h.groups_max >= 1 && h.groups_max <= kSlicedMaxGroups &&
+                    lds_bytes_needed(h.slice_rows, h.groups_max) <= kSlicedLdsBytes,
+                "%s: group range %d does not fit in LDS", what, h.groups_max);
+  NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1 && h.n_quads >= 1, "%s: bad counts", what);
+  const int64_t end_wg = h.off_workgroups + (int64_t)h.n_workgroups * (int64_t)sizeof(SlicedWorkgroup);
+  const int64_t end_rm = h.off_rowmap + (int64_t)h.n_workgroups * kSlicedTasks * 4;
+  const int64_t end_en = h.off_entries + h.n_quads * kSlicedQuadBytes;
+  NPAMD_REQUIRE(h.off_workgroups >= (int64_t)sizeof(h) && end_wg <= h.off_rowmap && end_rm <= h.off_entries &&
+                    end_en <= h.total_bytes && h.off_entries % 16 == 0 && h.off_rowmap % 4 == 0 &&
+                    h.off_workgroups % 4 == 0,
+                "%s: section offsets out of order or outside the blob", what);
+  const uint8_t* base = (const uint8_t*)blob;
+  const SlicedWorkgroup* wgs = (const SlicedWorkgroup*)(base + h.off_workgroups);
+  const uint32_t* rowmap = (const uint32_t*)(base + h.off_rowmap);
+  const uint8_t* quads = base + h.off_entries;
+  const int G = h.k / 8;
+  std::vector<uint8_t> covered((size_t)h.n_partials * (size_t)h.n, 0);
+  std::vector<uint8_t> filed((size_t)h.n * (size_t)G, 0);
+  for (int w = 0; w < h.n_workgroups; ++w) {
+    const SlicedWorkgroup& wg = wgs[w];
+    NPAMD_REQUIRE(wg.slice < (uint32_t)h.n_slices && wg.partial < (uint32_t)h.n_partials,
+                  "%s: workgroup %d: slice/partial out of range", what, w);
+    NPAMD_REQUIRE(wg.g_count >= 1 && wg.g_count <= (uint32_t)h.groups_max && (int64_t)wg.g_begin + wg.g_count <= G,
+                  "%s: workgroup %d: group range out of bounds", what, w);
+    const uint32_t slice_len = (uint32_t)std::min(h.slice_rows, h.nc - (int)wg.slice * h.slice_rows);
+    for (int s = 0; s < kSlicedWaves; ++s) {
+      const SlicedWave& wave = wg.wave[s];
+      const int64_t nq = ((int64_t)wave.steps + 3) / 4;
+      NPAMD_REQUIRE((int64_t)wave.quad_begin + std::max<int64_t>(nq, 1) <= h.n_quads,
+                    "%s: workgroup %d wave %d: entries out of bounds", what, w, s);
+      for (int lane = 0; lane < 64; ++lane) {
+        const uint32_t row = rowmap[(size_t)w * kSlicedTasks + (size_t)s * 64 + lane];
+        NPAMD_REQUIRE(row == kSlicedNoRow || row < (uint32_t)h.n, "%s: workgroup %d: row out of range", what, w);
+        if (row != kSlicedNoRow) {
+          uint8_t& c = covered[(size_t)wg.partial * h.n + row];
+          NPAMD_REQUIRE(c == 0, "%s: partial %u row %u written twice", what, wg.partial, row);
+          c = 1;
+        }
+        for (int64_t i = 0; i < nq * 4; ++i) {
+          const uint32_t e = get_entry24(quads + ((size_t)wave.quad_begin + (size_t)(i / 4)) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4));
+          const uint32_t g_local = e & 0x7FFu, local = e >> 11;
+          NPAMD_REQUIRE(g_local <= wg.g_count && local < slice_len, "%s: workgroup %d: entry field out of range", what, w);
+          if (g_local < wg.g_count) {
+            NPAMD_REQUIRE(row != kSlicedNoRow && i < (int64_t)wave.steps, "%s: workgroup %d: live entry in a lane without a row", what, w);
+            uint8_t& f = filed[(size_t)row * G + wg.g_begin + g_local];
+            NPAMD_REQUIRE(f == 0, "%s: index (%u, %u) filed twice", what, row, wg.g_begin + g_local);
+            f = 1;
+          }
+        }
+      }
+    }
+  }
+  for (uint8_t c : covered) NPAMD_REQUIRE(c == 1, "%s: some (partial, row) pair is never written", what);
+  for (uint8_t f : filed) NPAMD_REQUIRE(f == 1, "%s: some index is not filed", what);
+  NPAMD_REQUIRE(h.n_entries == (int64_t)h.n * G, "%s: entry count in the header is wrong", what);
+  return NPAMD_OK;
+}
+
+extern "C" int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* h, int M) {
+  if (h == nullptr || M < 1) return 0;
+  return (int64_t)h->n_partials * (int64_t)h->n * 4 * (int64_t)M;
+}

@@ -1,0 +1,220 @@
+// Decode GEMV over the slice-list form of the indices (see sliced_format.hpp).
+//
+// One workgroup of 16 waves holds one 8192-row codebook slice (128 KiB) and the
+// activations of its group range in LDS.  Every lane owns one output row and
+// walks the entries filed under (slice, group range, row): two 16-byte LDS reads
+// (codebook row, activation vector) and four packed dot products per entry, the
+// sum kept in registers.  Each lane then writes one float into the partial-sum
+// vector of its (slice, group range); a second kernel adds the partial vectors
+// of a row in a fixed order, adds the bias and rounds once.  No atomics: the
+// result does not depend on timing.
+#include "common.hpp"
+#include "sliced_format.hpp"
+
+namespace npamd {
+
+struct SlicedArgs {
+  const u32x4* x;  // one token: K/8 vectors of eight 16-bit values
+  const u32x4* codebook;
+  const SlicedWorkgroup* wgs;
+  const uint32_t* rowmap;
+  const uint8_t* entries;
+  float* partials;  // [n_partials][n]
+  int n, nc, slice_rows;
+};
+
+// Operands are taken by value: __builtin_bit_cast applied directly to a vector
+// element expression (v.y) reads element 0 with this compiler.
+template <int ACT>
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  if constexpr (ACT == NPAMD_BF16)
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+  else
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+
+template <int ACT>
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float c) {
+  c = dot2<ACT>(a.x, b.x, c);
+  c = dot2<ACT>(a.y, b.y, c);
+  c = dot2<ACT>(a.z, b.z, c);
+  return dot2<ACT>(a.w, b.w, c);
+}
+
+struct Quad {
+  uint32_t d0, d1, d2;
+};
+
+constexpr int kQuadsInFlight = 8;
+constexpr int kSliceBytes = kSlicedMaxSliceRows * 16;  // the activations follow the slice in LDS
+
+// Loads of quads q0 .. q0+7 of one strip (indices past the strip's last quad
+// re-read the last one, so the loads carry no branch).
+__device__ __forceinline__ void load_quads(Quad (&q)[kQuadsInFlight], const uint8_t* strip_lane, int q0, int nq) {
+#pragma unroll
+  for (int i = 0; i < kQuadsInFlight; ++i) {
+    const int qi = max(min(q0 + i, nq - 1), 0);
+    __builtin_memcpy(&q[i], __builtin_assume_aligned(strip_lane + (size_t)qi * kSlicedQuadBytes, 4), 12);
+  }
+}
+
+// The four entries of one quad: all eight LDS reads first, then the dot products.
+template <int ACT>
+__device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, float& acc0, float& acc1) {
+  uint32_t e[4];
+  e[0] = q.d0 & 0xFFFFFFu;
+  e[1] = (q.d0 >> 24) | ((q.d1 & 0xFFFFu) << 8);
+  e[2] = (q.d1 >> 16) | ((q.d2 & 0xFFu) << 16);
+  e[3] = q.d2 >> 8;
+  u32x4 c[4], xv[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    c[j] = *reinterpret_cast<const u32x4*>(lds + ((e[j] >> 11) << 4));
+    xv[j] = *reinterpret_cast<const u32x4*>(lds + kSliceBytes + ((e[j] & 0x7FFu) << 4));
+  }
+  acc0 = dot8<ACT>(c[0], xv[0], acc0);
+  acc1 = dot8<ACT>(c[1], xv[1], acc1);
+  acc0 = dot8<ACT>(c[2], xv[2], acc0);
+  acc1 = dot8<ACT>(c[3], xv[3], acc1);
+}
+
+template <int ACT>
+__global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  u32x4* cb = reinterpret_cast<u32x4*>(lds);
+  u32x4* xl = reinterpret_cast<u32x4*>(lds + kSliceBytes);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const SlicedWorkgroup& wg = a.wgs[blockIdx.x];
+  const int steps = (int)wg.wave[wave].steps;
+  const int nq = (steps + 3) >> 2;  // a strip is padded to whole quads, so padded steps are run too
+  const uint8_t* strip_lane = a.entries + (size_t)wg.wave[wave].quad_begin * kSlicedQuadBytes + (size_t)lane * 12;
+
+  // Requests in the order they are needed last-to-first: entries, slice, activations.
+  Quad q[kQuadsInFlight];
+  load_quads(q, strip_lane, 0, nq);
+  const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
+  {
+    const int slice_len = min(a.slice_rows, a.nc - (int)wg.slice * a.slice_rows);
+    const u32x4* src = a.codebook + (int64_t)wg.slice * a.slice_rows;
+    const int g_count = (int)wg.g_count;
+    u32x4 t[8], xt[2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) xt[i] = a.x[wg.g_begin + min(tid + i * kSlicedTasks, g_count - 1)];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int g = tid + i * kSlicedTasks;
+      if (g < g_count) xl[g] = xt[i];
+      else if (g == g_count) xl[g] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
+    }
+  }
+  __syncthreads();
+
+  float acc0 = 0.f, acc1 = 0.f;
+  for (int q0 = 0; q0 < nq; q0 += kQuadsInFlight) {
+    if (q0 > 0) load_quads(q, strip_lane, q0, nq);
+#pragma unroll
+    for (int i = 0; i < kQuadsInFlight; ++i) {
+      if (q0 + i >= nq) break;
+      run_quad<ACT>(q[i], lds, acc0, acc1);
+    }
+  }
+  if (row != kSlicedNoRow) a.partials[(size_t)wg.partial * a.n + row] = acc0 + acc1;
+}
+
+// y[row] = round(sum over the partial vectors + bias).  16 rows per block; the
+// partial vectors are dealt over 16 threads per row, whose sums are then added
+// in a fixed order.
+template <int ACT>
+__global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restrict__ partials, int n_partials,
+                                                             int n, const float* __restrict__ bias,
+                                                             void* __restrict__ y) {
+  __shared__ float red[16][17];
+  const int r = threadIdx.x & 15, j = threadIdx.x >> 4;
+  const int row = blockIdx.x * 16 + r;
+  float sum = 0.f;
+  if (row < n)
+    for (int p = j; p < n_partials; p += 16) sum += partials[(size_t)p * n + row];
+  red[j][r] = sum;
+  __syncthreads();
+  if (j == 0 && row < n) {
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) total += red[i][r];
+    if (bias) total += bias[row];
+    store_from_f32<ACT>(y, row, total);
+  }
+}
+
+template <int ACT>
+int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void* x, int64_t ldx,
+                  const void* codebook, const float* bias, void* y, int64_t ldy, int M, float* workspace,
+                  hipStream_t st, const char* what) {
+  const int lds = kSliceBytes + (h.groups_max + 1) * 16;
+  static int reserved = 0;
+  if (lds > 64 * 1024 && lds > reserved) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess)
+      return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
+    reserved = lds;
+  }
+  SlicedArgs a;
+  a.codebook = (const u32x4*)codebook;
+  a.wgs = (const SlicedWorkgroup*)(blob + h.off_workgroups);
+  a.rowmap = (const uint32_t*)(blob + h.off_rowmap);
+  a.entries = blob + h.off_entries;
+  a.n = h.n; a.nc = h.nc; a.slice_rows = h.slice_rows;
+  const size_t per_token = (size_t)h.n_partials * (size_t)h.n;
+  for (int m = 0; m < M; ++m) {
+    a.x = (const u32x4*)((const uint16_t*)x + (size_t)m * ldx);
+    a.partials = workspace + (size_t)m * per_token;
+    sliced_gemv_kernel<ACT><<<h.n_workgroups, kSlicedWaves * 64, lds, st>>>(a);
+    sliced_reduce_kernel<ACT><<<(h.n + 15) / 16, 256, 0, st>>>(a.partials, h.n_partials, h.n, bias,
+                                                                  (uint16_t*)y + (size_t)m * ldy);
+  }
+  return check_launch(what);
+}
+
+}  // namespace npamd
+
+using namespace npamd;
+
+extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_sliced_header* hp,
+                                    const void* blob, const void* codebook, int codebook_dtype,
+                                    const float* bias, void* y, int64_t ldy, int M, int act_dtype,
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
+  const char* what = "npamd_vq_gemv_sliced";
+  NPAMD_REQUIRE(hp != nullptr, "%s: header is null", what);
+  const npamd_sliced_header h = *hp;
+  NPAMD_REQUIRE(h.magic == kSlicedMagic && h.version == kSlicedVersion, "%s: not a slice-list header", what);
+  NPAMD_REQUIRE(act_dtype == NPAMD_F16 || act_dtype == NPAMD_BF16,
+                "%s: activations must be f16 or bf16 (got dtype code %d)", what, act_dtype);
+  NPAMD_REQUIRE(codebook_dtype == act_dtype, "%s: the codebook must be in the activation dtype", what);
+  NPAMD_REQUIRE(M >= 0 && M <= NPAMD_GEMV_MAX_M, "%s: M=%d exceeds the fused limit %d", what, M, NPAMD_GEMV_MAX_M);
+  NPAMD_REQUIRE(h.n > 0 && h.k > 0 && h.vl == 8 && h.k % 8 == 0 && h.nc >= 1, "%s: bad layer shape in header", what);
+  NPAMD_REQUIRE(h.slice_rows >= 1 && h.slice_rows <= kSlicedMaxSliceRows && h.groups_max >= 1 &&
+                    h.groups_max <= kSlicedMaxGroups,
+                "%s: slice geometry does not fit in LDS", what);
+  NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1, "%s: bad counts in header", what);
+  NPAMD_REQUIRE(ldx >= h.k && ldy >= h.n, "%s: row stride smaller than the row", what);
+  if (M == 0) return NPAMD_OK;
+  NPAMD_REQUIRE(x && blob && codebook && y && workspace, "%s: null pointer", what);
+  NPAMD_REQUIRE(ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0 &&
+                    (reinterpret_cast<uintptr_t>(codebook) % 16) == 0 &&
+                    (reinterpret_cast<uintptr_t>(blob) % 16) == 0 &&
+                    (reinterpret_cast<uintptr_t>(workspace) % 16) == 0,
+                "%s: x, codebook, blob and workspace must be 16-byte aligned (ldx a multiple of 8)", what);
+  NPAMD_REQUIRE(workspace_bytes >= npamd_vq_sliced_workspace_bytes(&h, M), "%s: workspace of %lld bytes, %lld needed",
+                what, (long long)workspace_bytes, (long long)npamd_vq_sliced_workspace_bytes(&h, M));
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == NPAMD_BF16)
+    return launch_sliced<NPAMD_BF16>(h, (const uint8_t*)blob, x, ldx, codebook, bias, y, ldy, M, (float*)workspace, st, what);
+  return launch_sliced<NPAMD_F16>(h, (const uint8_t*)blob, x, ldx, codebook, bias, y, ldy, M, (float*)workspace, st, what);
+}

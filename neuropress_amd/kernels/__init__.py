@@ -204,6 +204,116 @@ def vq_linear(
     return _vq_fused("npamd_vq_gemv", x, packed_indices, centroids, bits, out_features, bias)
 
 
+class SlicedIndices:
+    """Slice-list form of one layer's indices: the blob on the GPU plus a host copy of its header.
+
+    Built by :func:`vq_slice_indices`, consumed by :func:`vq_linear_sliced`.
+    """
+
+    _FIELDS = ("magic", "version", "n", "k", "vl", "nc", "slice_rows", "n_slices", "n_workgroups",
+               "n_partials", "groups_max", "reserved32", "n_quads", "n_entries", "off_workgroups",
+               "off_rowmap", "off_entries", "total_bytes")  # fmt: skip
+
+    def __init__(self, blob: torch.Tensor, header: bytes):
+        import ctypes
+        import struct
+
+        if len(header) != _lib.SLICED_HEADER_BYTES:
+            raise RuntimeError("SlicedIndices: header must be 128 bytes")
+        self.blob = blob
+        self.header = header
+        self._header_buf = ctypes.create_string_buffer(header, len(header))
+        values = struct.unpack("<2I10i6q", header[:96])
+        for name, value in zip(self._FIELDS, values):
+            setattr(self, name, value)
+
+    @property
+    def header_ptr(self) -> int:
+        import ctypes
+
+        return ctypes.addressof(self._header_buf)
+
+    def workspace_bytes(self, m: int) -> int:
+        return int(_lib.load().npamd_vq_sliced_workspace_bytes(self.header_ptr, int(m)))
+
+    def to(self, device) -> "SlicedIndices":
+        return SlicedIndices(self.blob.to(device), self.header)
+
+
+def vq_slice_indices(
+    packed_indices: torch.Tensor,
+    bits: int,
+    out_features: int,
+    in_features: int,
+    vector_len: int,
+    num_centroids: int,
+    device: torch.device | str | None = None,
+    target_workgroups: int = 0,
+) -> SlicedIndices:
+    """Re-lay a packed index stream into the slice-list form (host work, once per layer).
+
+    The stream is copied to the host, filed by codebook slice there
+    (``npamd_vq_sliced_build``), checked (``npamd_vq_sliced_check``) and uploaded to
+    *device* (default: where *packed_indices* lives).  No reference counterpart.
+    """
+    import ctypes
+
+    what = "vq_slice_indices"
+    if packed_indices.dtype != torch.uint8:
+        raise RuntimeError(f"{what}: packed indices must be uint8, got {packed_indices.dtype}")
+    dev = torch.device(device) if device is not None else packed_indices.device
+    host = packed_indices.detach().to("cpu").contiguous().reshape(-1)
+    if target_workgroups <= 0 and dev.type == "cuda":
+        target_workgroups = torch.cuda.get_device_properties(dev).multi_processor_count
+    size = ctypes.c_int64(0)
+    args = (host.data_ptr(), host.numel(), int(bits), int(out_features), int(in_features),
+            int(vector_len), int(num_centroids), int(target_workgroups))  # fmt: skip
+    _lib.call("npamd_vq_sliced_build", *args, None, 0, ctypes.byref(size))
+    blob = torch.empty(size.value, dtype=torch.uint8, pin_memory=dev.type == "cuda")
+    _lib.call("npamd_vq_sliced_build", *args, blob.data_ptr(), blob.numel(), ctypes.byref(size))
+    _lib.call("npamd_vq_sliced_check", blob.data_ptr(), blob.numel())
+    header = bytes(blob[: _lib.SLICED_HEADER_BYTES].numpy().tobytes())
+    return SlicedIndices(blob.to(dev), header)
+
+
+def vq_linear_sliced(
+    x: torch.Tensor,
+    sliced: SlicedIndices,
+    centroids: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Decode GEMV over the slice-list form, ``M <= 16`` (``npamd_vq_gemv_sliced``).
+
+    *centroids* must already be in ``x.dtype`` (the modules cache that copy).
+    *workspace*: optional float32 scratch of ``sliced.workspace_bytes(M) / 4`` elements.
+    """
+    what = "vq_linear_sliced"
+    _check_device(what, x, sliced.blob, centroids, bias, workspace)
+    x = _x2d(x, what)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"{what}: x must be float16 or bfloat16, got {x.dtype}")
+    cb = _centroids_f16(centroids, what)
+    if cb.dtype != x.dtype:
+        raise RuntimeError(f"{what}: centroids must be in x's dtype ({x.dtype}), got {cb.dtype}")
+    m, k = x.shape
+    if k != sliced.k or cb.shape[0] != sliced.nc or cb.shape[1] != sliced.vl:
+        raise RuntimeError(f"{what}: slice lists were built for K={sliced.k}, codebook [{sliced.nc}, {sliced.vl}]")
+    need = sliced.workspace_bytes(max(m, 1))
+    if workspace is None:
+        workspace = torch.empty(need // 4, device=x.device, dtype=torch.float32)
+    elif workspace.dtype != torch.float32 or not workspace.is_contiguous():
+        raise RuntimeError(f"{what}: workspace must be a contiguous float32 tensor")
+    y = torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
+    b32 = _bias_f32(bias)
+    _lib.call(
+        "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), sliced.header_ptr, sliced.blob.data_ptr(),
+        cb.data_ptr(), _DT[cb.dtype], _ptr(b32), y.data_ptr(), y.stride(0), m, _DT[x.dtype],
+        workspace.data_ptr(), workspace.numel() * 4, _stream(x),
+    )  # fmt: skip
+    return y
+
+
 def vq_linear_wmma(
     x: torch.Tensor,
     packed_indices: torch.Tensor,

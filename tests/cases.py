@@ -62,3 +62,50 @@ def within_tol(y: np.ndarray, ref: np.ndarray, atol=1e-2, rtol=1e-2):
     err = np.abs(y.astype(np.float64) - ref)
     bound = atol + rtol * np.abs(ref)
     return bool((err <= bound).all()), float(err.max(initial=0.0)), float((err / bound).max(initial=0.0))
+
+
+def decode_sliced_blob(blob: np.ndarray) -> tuple[np.ndarray, dict]:
+    """Read a slice-list blob back into the ``[N, K/8]`` index matrix it was built from.
+
+    An independent reader of the layout (header, workgroup records with their
+    16 wave records, per-lane row map, 24-bit entries four to a 12-byte lane
+    record).  ``hits`` counts how often each (row, group) pair was filed and
+    ``writes`` how often each (partial, row) cell is written; both must be 1
+    everywhere.
+    """
+    import struct
+
+    names = ("magic", "version", "n", "k", "vl", "nc", "slice_rows", "n_slices", "n_workgroups",
+             "n_partials", "groups_max", "reserved32", "n_quads", "n_entries", "off_workgroups",
+             "off_rowmap", "off_entries", "total_bytes")  # fmt: skip
+    h = dict(zip(names, struct.unpack("<2I10i6q", blob[:96].tobytes())))
+    assert h["magic"] == 0x4C53504E and h["vl"] == 8
+    n, groups, n_wg = h["n"], h["k"] // 8, h["n_workgroups"]
+    wgs = np.frombuffer(blob, dtype="<u4", count=n_wg * 40, offset=h["off_workgroups"]).reshape(n_wg, 40).astype(np.int64)
+    rowmap = np.frombuffer(blob, dtype="<u4", count=n_wg * 1024, offset=h["off_rowmap"]).reshape(n_wg, 16, 64).astype(np.int64)
+    quads = np.frombuffer(blob, dtype=np.uint8, count=h["n_quads"] * 768, offset=h["off_entries"]).reshape(-1, 64, 4, 3)
+    idx = np.full((n, groups), -1, dtype=np.int64)
+    hits = np.zeros((n, groups), dtype=np.int32)
+    writes = np.zeros((h["n_partials"], n), dtype=np.int32)
+    for w in range(n_wg):
+        sl, partial, g_begin, g_count = wgs[w, :4]
+        for s in range(16):
+            quad_begin, steps = wgs[w, 8 + 2 * s], wgs[w, 9 + 2 * s]
+            rows = rowmap[w, s]
+            has_row = rows != 0xFFFFFFFF
+            np.add.at(writes, (np.full(int(has_row.sum()), partial), rows[has_row]), 1)
+            nq = (steps + 3) // 4
+            if nq == 0:
+                continue
+            q = quads[quad_begin : quad_begin + nq].astype(np.int64)  # [nq, lane, 4, 3]
+            e = q[..., 0] | (q[..., 1] << 8) | (q[..., 2] << 16)  # [nq, lane, 4]
+            e = e.transpose(1, 0, 2).reshape(64, nq * 4)  # [lane, step]
+            g_local, local = e & 0x7FF, e >> 11
+            live = g_local < g_count
+            assert not live[:, steps:].any(), "live entry beyond the strip's step count"
+            assert not live[~has_row].any(), "live entry in a lane without a row"
+            rr = np.broadcast_to(rows[:, None], e.shape)[live]
+            gg = (g_begin + g_local)[live]
+            idx[rr, gg] = (sl * h["slice_rows"] + local)[live]
+            np.add.at(hits, (rr, gg), 1)
+    return idx, {"header": h, "hits": hits, "writes": writes}
