@@ -48,14 +48,8 @@ struct Quad {
 constexpr int kQuadsInFlight = 8;
 constexpr int kSliceBytes = kSlicedMaxSliceRows * 16;  // the activations follow the slice in LDS
 
-// Loads of quads q0 .. q0+7 of one strip (indices past the strip's last quad
-// re-read the last one, so the loads carry no branch).
-__device__ __forceinline__ void load_quads(Quad (&q)[kQuadsInFlight], const uint8_t* strip_lane, int q0, int nq) {
-#pragma unroll
-  for (int i = 0; i < kQuadsInFlight; ++i) {
-    const int qi = max(min(q0 + i, nq - 1), 0);
-    __builtin_memcpy(&q[i], __builtin_assume_aligned(strip_lane + (size_t)qi * kSlicedQuadBytes, 4), 12);
-  }
+__device__ __forceinline__ void load_quad(Quad& q, const uint8_t* strip_lane, int qi) {
+  __builtin_memcpy(&q, __builtin_assume_aligned(strip_lane + (size_t)qi * kSlicedQuadBytes, 4), 12);
 }
 
 // The four entries of one quad: all eight LDS reads first, then the dot products.
@@ -91,10 +85,10 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
   const int nq = (steps + 3) >> 2;  // a strip is padded to whole quads, so padded steps are run too
   const uint8_t* strip_lane = a.entries + (size_t)wg.wave[wave].quad_begin * kSlicedQuadBytes + (size_t)lane * 12;
 
-  // Requests in the order they are needed last-to-first: entries, slice, activations.
+  // Requests in the order they are needed: the slice and the activations (mostly
+  // L2 hits) first, then the entries, which stream from HBM while the slice is
+  // being stored and the first quads are worked on.
   Quad q[kQuadsInFlight];
-  load_quads(q, strip_lane, 0, nq);
-  const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
   {
     const int slice_len = min(a.slice_rows, a.nc - (int)wg.slice * a.slice_rows);
     const u32x4* src = a.codebook + (int64_t)wg.slice * a.slice_rows;
@@ -104,6 +98,12 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
 #pragma unroll
     for (int i = 0; i < 2; ++i) xt[i] = a.x[wg.g_begin + min(tid + i * kSlicedTasks, g_count - 1)];
+    __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
+    // The first eight quads (past the strip's end: its last quad again, or quad 0
+    // of the blob for a wave without a strip; no branch around a load).
+#pragma unroll
+    for (int i = 0; i < kQuadsInFlight; ++i) load_quad(q[i], strip_lane, max(min(i, nq - 1), 0));
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
@@ -114,16 +114,33 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
       else if (g == g_count) xl[g] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
     }
   }
+  const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
   __syncthreads();
 
+  // Eight quads stay in flight: each one is replaced by the quad eight further on
+  // as soon as it has been read.
   float acc0 = 0.f, acc1 = 0.f;
-  for (int q0 = 0; q0 < nq; q0 += kQuadsInFlight) {
-    if (q0 > 0) load_quads(q, strip_lane, q0, nq);
+  int q0 = 0;
+  for (; q0 + 2 * kQuadsInFlight <= nq; q0 += kQuadsInFlight) {
 #pragma unroll
     for (int i = 0; i < kQuadsInFlight; ++i) {
-      if (q0 + i >= nq) break;
-      run_quad<ACT>(q[i], lds, acc0, acc1);
+      const Quad cur = q[i];
+      load_quad(q[i], strip_lane, q0 + i + kQuadsInFlight);
+      run_quad<ACT>(cur, lds, acc0, acc1);
     }
+  }
+#pragma unroll
+  for (int i = 0; i < kQuadsInFlight; ++i) {
+    if (q0 + i >= nq) break;
+    const Quad cur = q[i];
+    if (q0 + i + kQuadsInFlight < nq) load_quad(q[i], strip_lane, q0 + i + kQuadsInFlight);
+    run_quad<ACT>(cur, lds, acc0, acc1);
+  }
+  q0 += kQuadsInFlight;
+#pragma unroll
+  for (int i = 0; i < kQuadsInFlight; ++i) {
+    if (q0 + i >= nq) break;
+    run_quad<ACT>(q[i], lds, acc0, acc1);
   }
   if (row != kSlicedNoRow) a.partials[(size_t)wg.partial * a.n + row] = acc0 + acc1;
 }
