@@ -152,7 +152,9 @@ int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, 
  * `header_host` is a host copy of the blob's header, `blob` the whole blob in
  * device memory.  The codebook must be in the activation dtype.  `workspace`
  * is device memory of npamd_vq_sliced_workspace_bytes() bytes, 16-byte aligned,
- * contents irrelevant before and after.
+ * contents irrelevant before the call; afterwards it holds, per token, the
+ * n_partials partial-sum vectors [n_partials][N] (f32) whose sum over the first
+ * axis is the un-biased result.  With y == NULL only those are produced.
  */
 int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_sliced_header* header_host,
                          const void* blob, const void* codebook, int codebook_dtype,

@@ -62,7 +62,7 @@ Geometry plan_geometry(int N, int G, const std::vector<int64_t>& slice_count, in
       const double share = (double)slice_count[s] / (double)n_idx;
       // Group ranges in proportion to the slice's load, but no finer than about
       // 16 entries per row and range: a workgroup pays for loading its slice.
-      const int kp_max = std::max(kp_min, (int)((double)G * share / 16.0));
+      const int kp_max = std::max(kp_min, (int)((double)G * share / 16.0 + 0.5));
       int kp = (int)((double)target * share / rb + 0.5);
       kp = std::max(kp_min, std::min(kp, kp_max));
       geo.parts[s] = kp;

@@ -193,8 +193,9 @@ int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void*
     a.x = (const u32x4*)((const uint16_t*)x + (size_t)m * ldx);
     a.partials = workspace + (size_t)m * per_token;
     sliced_gemv_kernel<ACT><<<h.n_workgroups, kSlicedWaves * 64, lds, st>>>(a);
-    sliced_reduce_kernel<ACT><<<(h.n + 15) / 16, 256, 0, st>>>(a.partials, h.n_partials, h.n, bias,
-                                                                  (uint16_t*)y + (size_t)m * ldy);
+    if (y)
+      sliced_reduce_kernel<ACT><<<(h.n + 15) / 16, 256, 0, st>>>(a.partials, h.n_partials, h.n, bias,
+                                                                    (uint16_t*)y + (size_t)m * ldy);
   }
   return check_launch(what);
 }
@@ -222,7 +223,7 @@ extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_slic
   NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1, "%s: bad counts in header", what);
   NPAMD_REQUIRE(ldx >= h.k && ldy >= h.n, "%s: row stride smaller than the row", what);
   if (M == 0) return NPAMD_OK;
-  NPAMD_REQUIRE(x && blob && codebook && y && workspace, "%s: null pointer", what);
+  NPAMD_REQUIRE(x && blob && codebook && workspace, "%s: null pointer", what);
   NPAMD_REQUIRE(ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(codebook) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(blob) % 16) == 0 &&

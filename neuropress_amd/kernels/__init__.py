@@ -282,11 +282,14 @@ def vq_linear_sliced(
     centroids: torch.Tensor,
     bias: torch.Tensor | None = None,
     workspace: torch.Tensor | None = None,
-) -> torch.Tensor:
+    partials_only: bool = False,
+) -> torch.Tensor | None:
     """Decode GEMV over the slice-list form, ``M <= 16`` (``npamd_vq_gemv_sliced``).
 
     *centroids* must already be in ``x.dtype`` (the modules cache that copy).
-    *workspace*: optional float32 scratch of ``sliced.workspace_bytes(M) / 4`` elements.
+    *workspace*: optional float32 scratch of ``sliced.workspace_bytes(M) / 4`` elements;
+    after the call it holds the ``[M, n_partials, N]`` partial sums.  With
+    *partials_only* nothing else is computed and None is returned.
     """
     what = "vq_linear_sliced"
     _check_device(what, x, sliced.blob, centroids, bias, workspace)
@@ -304,11 +307,11 @@ def vq_linear_sliced(
         workspace = torch.empty(need // 4, device=x.device, dtype=torch.float32)
     elif workspace.dtype != torch.float32 or not workspace.is_contiguous():
         raise RuntimeError(f"{what}: workspace must be a contiguous float32 tensor")
-    y = torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
+    y = None if partials_only else torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
     b32 = _bias_f32(bias)
     _lib.call(
         "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), sliced.header_ptr, sliced.blob.data_ptr(),
-        cb.data_ptr(), _DT[cb.dtype], _ptr(b32), y.data_ptr(), y.stride(0), m, _DT[x.dtype],
+        cb.data_ptr(), _DT[cb.dtype], _ptr(b32), _ptr(y), sliced.n, m, _DT[x.dtype],
         workspace.data_ptr(), workspace.numel() * 4, _stream(x),
     )  # fmt: skip
     return y

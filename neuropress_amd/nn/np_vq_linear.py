@@ -56,6 +56,17 @@ def _env_int(names: tuple[str, ...], default: int) -> int:
 # band ends at 16 here (2 in the reference, whose GEMV re-reads the weight per token).
 _FUSED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_FUSED_MAX_TOKENS",), 16)
 
+# Decode steps (1-2 tokens) of layers whose codebook is too large to sit in a
+# compute unit's LDS next to the GEMV's buffers (more than 4096 rows): the fused
+# GEMV then pays one L2 lookup per index (34 us on a 14336 x 4096 layer with a
+# 65536-row codebook), while the slice-list GEMV (kernels.vq_linear_sliced) keeps
+# 8192-row codebook slices in LDS and takes 14.5 us per token.  The slice lists
+# are built on the host at first use (about 25 MB per such layer, on top of the
+# packed stream the other bands keep reading).  0 disables the path.
+_SLICED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_SLICED_MAX_TOKENS",), 2)
+_SLICED_MIN_CENTROIDS: int = 4097
+_SLICED_MIN_INDICES: int = _env_int(("NEUROPRESS_VQ_SLICED_MIN_INDICES",), 1 << 20)
+
 # cuda_lut layers: 0 = always decode + GEMM, the reference's default routing.
 _LUT_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_LUT_MAX_TOKENS",), 0)
 
@@ -455,6 +466,8 @@ class NPVQLinear(nn.Module):
             if x.dtype not in (torch.float16, torch.bfloat16):
                 return self._forward_dequant_gemm(x)  # fp32 activations: decode + GEMM
             m = x.numel() // self.in_features
+            if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and self._sliced_ready(x):
+                return self._forward_sliced(x)
             if m > _fused_max_tokens(self.backend):
                 if (
                     self.backend != VQBackend.CUDA_LUT
@@ -472,6 +485,60 @@ class NPVQLinear(nn.Module):
         if self.backend == VQBackend.COMPILE:
             return self._forward_compile(x)
         return self._forward_default(x)
+
+    # -- slice-list GEMV ---------------------------------------------------
+
+    def _sliced_eligible(self) -> bool:
+        return (
+            _SLICED_MAX_TOKENS > 0
+            and not self.is_residual
+            and self.vector_len == 8
+            and self.proxy.num_centroids >= _SLICED_MIN_CENTROIDS
+            and self.n_vectors >= _SLICED_MIN_INDICES
+        )
+
+    def prepare_sliced(self) -> bool:
+        """Build the slice-list form of the indices for the module's current device.
+
+        Called lazily by the first 1-2 token forward; call it yourself before
+        capturing a HIP graph (the build copies the stream to the host and back).
+        Returns False when the layer does not use the path.
+        """
+        if not (self._sliced_eligible() and self.packed_indices.is_cuda):
+            return False
+        sl = self._derived.get("sliced")
+        if sl is None or sl.blob.device != self.packed_indices.device:
+            from .. import kernels
+
+            self._derived["sliced"] = kernels.vq_slice_indices(
+                self.packed_indices, self.bits, self.out_features, self.in_features,
+                self.vector_len, self.proxy.num_centroids,
+            )  # fmt: skip
+        return True
+
+    def _sliced_ready(self, x: torch.Tensor) -> bool:
+        if not (x.is_cuda and self._sliced_eligible()):
+            return False
+        sl = self._derived.get("sliced")
+        if sl is not None and sl.blob.device == x.device:
+            return True
+        if torch.cuda.is_current_stream_capturing():
+            return False  # no host work inside a capture: the fused GEMV runs instead
+        return self.prepare_sliced()
+
+    def _forward_sliced(self, x: torch.Tensor) -> torch.Tensor:
+        from .. import kernels
+
+        *leading, _ = x.shape
+        try:
+            y = kernels.vq_linear_sliced(
+                x.reshape(-1, self.in_features), self._derived["sliced"],
+                self.proxy.centroids_as(x.dtype), self._bias_f32(),
+            )  # fmt: skip
+        except RuntimeError as exc:
+            self._fallback("vq_linear_sliced", "decode + GEMM", exc)
+            return self._forward_dequant_gemm(x)
+        return y.reshape(*leading, self.out_features)
 
     def _tile_grid_fills_gpu(self, x: torch.Tensor, m: int) -> bool:
         """True when the tile GEMM's grid (64 columns x up to 384 rows per workgroup)

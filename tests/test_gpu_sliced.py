@@ -1,0 +1,187 @@
+"""Parity of the slice-list decode GEMV against the CPU oracle, through the C ABI.
+
+Bar: outputs within 1e-2 abs + 1e-2 rel of the oracle's double-accumulated
+contraction of the oracle-decoded weight; results identical from run to run.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def _vq_ref(oracle_lib, L, act):
+    code = orc.torch_dtype_code(act)
+    w = oracle_lib.vq_decode(L["packed"].numpy(), L["bits"], orc.to_bits(L["cb"]), L["n"], L["k"], code)
+    bias = None if L["bias"] is None else orc.to_bits(L["bias"])
+    return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
+
+
+def _check(y: torch.Tensor, ref: np.ndarray):
+    ok, max_abs, excess = cases.within_tol(y.float().cpu().numpy(), ref)
+    assert ok, f"max abs err {max_abs:.3e}, {excess:.2f}x the 1e-2 bound"
+
+
+def _run(gpu, L, act, **kw):
+    from neuropress_amd import kernels
+
+    sl = kernels.vq_slice_indices(L["packed"], L["bits"], L["n"], L["k"], 8, L["nc"], device=gpu)
+    bias = None if L["bias"] is None else L["bias"].to(gpu)
+    return kernels.vq_linear_sliced(L["x"].to(gpu), sl, L["cb"].to(act).to(gpu), bias, **kw), sl
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize(
+    "n,k,nc,bits",
+    [
+        (72, 96, 300, None),  # one slice
+        (130, 8, 9000, None),  # a single group, two slices
+        (1000, 64, 20000, None),  # short last slice
+        (1100, 256, 65536, 16),  # two row blocks
+        (300, 128, 4096, 12),
+        (96, 12296, 65536, 16),  # K / 8 = 1537 groups: two group ranges are forced
+    ],
+)
+@pytest.mark.parametrize("m", [1, 3])
+def test_sliced_gemv_matches_oracle(gpu, oracle_lib, act, n, k, nc, bits, m):
+    L = cases.vq_layer(900 + n + m, n, k, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
+    y, _ = _run(gpu, L, act)
+    assert y.shape == (m, n) and y.dtype == act
+    _check(y, _vq_ref(oracle_lib, L, act))
+
+
+def test_sliced_gemv_zipf_indices(gpu, oracle_lib):
+    """Config-4-like index statistics: slice 0 receives most entries and gets more group ranges."""
+    from neuropress_amd.transforms.vq_packing import IndexPacking
+
+    n, k, nc, act = 517, 1024, 65536, torch.float16
+    L = cases.vq_layer(77, n, k, nc, bits=16, act=act, m=2, bias=False, std=0.05)
+    idx = cases.zipf_indices(cases.gen(78), nc, n * (k // 8))
+    L["idx"], L["packed"] = idx, IndexPacking.pack(idx, 16)
+    y, sl = _run(gpu, L, act)
+    assert sl.n_partials > sl.n_slices  # the hot slice was split over several group ranges
+    _check(y, _vq_ref(oracle_lib, L, act))
+
+
+def test_sliced_gemv_full_size_and_fused_gemv_agree(gpu, oracle_lib):
+    """BASELINE config 3 shape (14336 x 4096, 65536 x 8 codebook, bf16), one token: against the
+    oracle, against the fused GEMV (same f32-accumulated sum in another order), run to run,
+    and through the partial sums left in the workspace."""
+    from neuropress_amd import kernels
+
+    act = torch.bfloat16
+    L = cases.vq_layer(1003, 14336, 4096, 65536, bits=16, act=act, m=1, bias=True, std=0.02)
+    ws = torch.empty(64 * 14336, device=gpu, dtype=torch.float32)
+    y, sl = _run(gpu, L, act, workspace=ws)
+    assert sl.n_workgroups <= 2 * torch.cuda.get_device_properties(gpu).multi_processor_count
+    _check(y, _vq_ref(oracle_lib, L, act))
+    cb = L["cb"].to(act).to(gpu)
+    y_fused = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), cb, 16, 8, L["bias"].to(gpu), 14336)
+    assert (y.float() - y_fused.float()).abs().max().item() <= 2 ** -6  # one bf16 ulp at |y| < 4
+    for _ in range(3):
+        again = kernels.vq_linear_sliced(L["x"].to(gpu), sl, cb, L["bias"].to(gpu), workspace=ws)
+        assert torch.equal(again, y)
+    partials = ws[: sl.n_partials * 14336].reshape(sl.n_partials, 14336)
+    total = partials.sum(0, dtype=torch.float64) + L["bias"].to(gpu).double()
+    assert (total - y.double()).abs().max().item() <= 2 ** -6
+
+
+def test_sliced_gemv_partials_only(gpu):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(5, 200, 128, 20000, act=torch.float16, m=1, std=0.05)
+    sl = kernels.vq_slice_indices(L["packed"], L["bits"], 200, 128, 8, 20000, device=gpu)
+    cb, x = L["cb"].to(gpu), L["x"].to(gpu)
+    ws = torch.full((sl.workspace_bytes(1) // 4,), float("nan"), device=gpu)
+    assert kernels.vq_linear_sliced(x, sl, cb, workspace=ws, partials_only=True) is None
+    y = kernels.vq_linear_sliced(x, sl, cb)
+    total = ws.reshape(sl.n_partials, 200).sum(0)
+    assert torch.isfinite(total).all()
+    assert (total - y.float()).abs().max().item() < 1e-2
+
+
+def test_sliced_wrapper_errors(gpu):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(6, 64, 64, 20000, act=torch.float16, m=1)
+    sl = kernels.vq_slice_indices(L["packed"], L["bits"], 64, 64, 8, 20000, device=gpu)
+    x, cb = L["x"].to(gpu), L["cb"].to(gpu)
+    with pytest.raises(RuntimeError, match="x's dtype"):
+        kernels.vq_linear_sliced(x.to(torch.bfloat16), sl, cb)
+    with pytest.raises(RuntimeError, match="built for"):
+        kernels.vq_linear_sliced(x[:, :32].contiguous(), sl, cb)
+    with pytest.raises(RuntimeError, match="must be float16 or bfloat16"):
+        kernels.vq_linear_sliced(x.float(), sl, cb.float())
+    with pytest.raises(RuntimeError, match="workspace of"):
+        kernels.vq_linear_sliced(x, sl, cb, workspace=torch.empty(4, device=gpu))
+    with pytest.raises(RuntimeError, match="VL = 8"):
+        kernels.vq_slice_indices(L["packed"], L["bits"], 64, 64, 4, 20000, device=gpu)
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act, monkeypatch):
+    """NPVQLinear: 1-2 tokens on a layer with a large codebook use the slice lists, more
+    tokens the fused GEMV; both match the oracle; a HIP graph captured after
+    prepare_sliced() replays to the same bits."""
+    from neuropress_amd import kernels
+    from neuropress_amd.nn import np_vq_linear as mod
+
+    monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    n, k, nc = 384, 512, 20000
+    L = cases.vq_layer(41, n, k, nc, act=act, m=4, bias=True, std=0.05)
+    proxy = mod.VQProxy(L["cb"]).to(gpu)
+    layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], n, k, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
+    calls = []
+    real = kernels.vq_linear_sliced
+    monkeypatch.setattr(kernels, "vq_linear_sliced", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
+    x = L["x"].to(gpu)
+    ref = _vq_ref(oracle_lib, L, act)
+    y1 = layer(x[:1])
+    y2 = layer(x[:2].reshape(1, 2, k))
+    y4 = layer(x)
+    assert calls == [1, 2] and y2.shape == (1, 2, n)
+    _check(y1, ref[:1])
+    _check(y2.reshape(2, n), ref[:2])
+    _check(y4, ref)
+    # Graph capture: no host work may happen inside; the lists already exist.
+    assert layer.prepare_sliced()
+    static_x = x[:1].clone()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        layer(static_x)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            static_y = layer(static_x)
+    for i in range(3):
+        static_x.copy_(x[i : i + 1])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, layer(x[i : i + 1]))
+
+
+def test_module_without_prepared_lists_inside_capture_uses_fused_gemv(gpu, monkeypatch):
+    from neuropress_amd.nn import np_vq_linear as mod
+
+    monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    L = cases.vq_layer(42, 128, 256, 20000, act=torch.float16, m=1, std=0.05)
+    proxy = mod.VQProxy(L["cb"]).to(gpu)
+    layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], 128, 256, 8, "cuda_wmma").to(gpu)
+    x = L["x"].to(gpu)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 0)
+        layer(x)  # warm the fused path outside the capture
+        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 2)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            y = layer(x)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert "sliced" not in layer._derived
+    assert torch.equal(y, layer(x)) or (y.float() - layer(x).float()).abs().max().item() < 1e-2
