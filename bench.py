@@ -3,10 +3,11 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-sweep]
 
-One "step" = one call of the fused decode GEMV on BASELINE config 3's up/gate
+One "step" = one decode-step call (M=1 token) of BASELINE config 3's up/gate
 layer (Llama-3-8B MLP, N=14336, K=4096, vector length 8, 65536-entry fp16
-codebook, 16-bit indices, bf16 activations, M=1 token) on synthetic seeded
-data already resident in HBM.  K steps are recorded into one HIP graph over a
+codebook, 16-bit indices, bf16 activations) on synthetic seeded data already
+resident in HBM, through the kernels NPVQLinear uses for it: the slice-list
+decode GEMV and its partial-sum reduction.  K steps are recorded into one HIP graph over a
 rotating pool of weight/activation buffers larger than L2 + Infinity Cache and
 timed with HIP events on the launch stream, so `value` is kernel throughput,
 not Python launch overhead, and the index stream really comes from HBM.
@@ -43,7 +44,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
-    ap.add_argument("--case", default="", choices=["", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "dequant", "q4_gemv_m1", "q4_tile_m128"],
+    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "dequant", "q4_gemv_m1", "q4_tile_m128"],
                     help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
                          "on the config-3 / config-5 shape and print a one-line JSON with its HIP-event time")
     ap.add_argument("--ceilings", action="store_true",
@@ -164,7 +165,12 @@ def main():
             cb16, cbb = cb.to(dev), cb.to(torch.bfloat16).to(dev)
             m = 256 if args.case == "tile_m256" else 1
             x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
-            if args.case == "tile_m256":
+            if args.case == "sliced_m1":
+                sl0 = kernels.vq_slice_indices(base, bits, n, k, 8, nc, device=dev)
+                spool = [sl0] + [kernels.SlicedIndices(sl0.blob.clone(), sl0.header) for _ in range(n_rot - 1)]
+                ws = torch.empty(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
+                fn = lambda i: kernels.vq_linear_sliced(x, spool[i], cbb, None, workspace=ws)
+            elif args.case == "tile_m256":
                 fn = lambda i: kernels.vq_gemm_tile(x, pool[i], cbb, bits, n, None)
             elif args.case == "dequant":
                 fn = lambda i: kernels.vq_dequant(pool[i], cb16, bits, n, k, torch.bfloat16)
@@ -210,19 +216,28 @@ def main():
         print(json.dumps(out))
         return
 
-    # ---------------- headline: config 3 up/gate, M = 1, fused GEMV -------------
+    # ---------------- headline: config 3 up/gate, M = 1 --------------------------
     n, k = 14336, 4096
     n_rot = max(2, POOL_BYTES // (n * k // 8 * 2))
     c3 = vq_case(dev, 1003, n, k, 65536, 16, torch.bfloat16, n_rot)
     xs = [torch.randn(1, k, generator=gen(7 + i)).to(torch.bfloat16).to(dev) for i in range(n_rot)]
     ys = [None] * n_rot
+    sl0 = kernels.vq_slice_indices(c3["packed"], 16, n, k, 8, 65536, device=dev)
+    s_rot = max(2, POOL_BYTES // sl0.total_bytes)
+    spool = [sl0] + [kernels.SlicedIndices(sl0.blob.clone(), sl0.header) for _ in range(s_rot - 1)]
+    ws = torch.empty(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
 
     def step(i):
-        ys[i] = kernels.vq_linear(xs[i], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n)
+        ys[i % n_rot] = kernels.vq_linear_sliced(xs[i % n_rot], spool[i], c3["d_cb_act"], None, workspace=ws)
 
-    us = time_graph(step, n_rot, args.steps, args.warmup, dev)
+    us = time_graph(step, s_rot, args.steps, args.warmup, dev)
+    # The dominant kernel alone (sliced_gemv_kernel, partial sums only), for the roofline line.
+    us_main = time_graph(lambda i: kernels.vq_linear_sliced(xs[i % n_rot], spool[i], c3["d_cb_act"], None,
+                                                            workspace=ws, partials_only=True),
+                         s_rot, args.steps, args.warmup, dev)
     alg = vq_alg_bytes(c3, 1)
     gbs = alg / us / 1e3
+    gbs_main = alg / us_main / 1e3
 
     # correctness gate on the timed configuration (decode bit-exact, output within 1e-2)
     w_gpu = kernels.vq_dequant(c3["pool"][0], c3["d_cb"], 16, n, k, torch.bfloat16)
@@ -247,14 +262,18 @@ def main():
         "data": "synthetic (seed 1003; uniform 16-bit indices, N(0,0.02) fp16 codebook, N(0,1) bf16 activations)",
         "config": {
             "workload": "BASELINE config 3: Llama-3-8B MLP up/gate 14336x4096, VL=8, 65536-entry fp16 codebook, "
-                        "16-bit indices, bf16, M=1 (fused decode GEMV, band a)",
-            "N": n, "K": k, "M": 1, "rotating_pool_MB": round(n_rot * c3["idx_bytes"] / 2**20),
+                        "16-bit indices, bf16, M=1 (band a: slice-list decode GEMV + partial-sum reduction)",
+            "N": n, "K": k, "M": 1, "rotating_pool_MB": round(s_rot * sl0.total_bytes / 2**20),
         },
         "roofline": {
-            "bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-            "kernel": "fused_gemv_kernel (vq, 16-bit)", "algorithmic_bytes_per_launch": alg,
-            "avg_launch_us": round(us, 3),
+            "bound": "hbm", "achieved": round(gbs_main, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs_main / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "sliced_gemv_kernel<bf16>", "algorithmic_bytes_per_launch": alg,
+            "avg_launch_us": round(us_main, 3),
+            "streamed_bytes_per_launch": sl0.total_bytes + sl0.n_workgroups * (8192 * 16) + sl0.n_partials * n * 4,
+            "note": "achieved = bytes of the reference's format (16-bit index stream + codebook + x + y) / duration of "
+                    "sliced_gemv_kernel alone; `value` divides the same bytes by the whole call (that kernel + the "
+                    "partial-sum reduction kernel)",
         },
         "checks": {"decode_bit_exact": decode_exact, "output_within_1e-2": ok, "max_abs_err": max_abs},
     }
@@ -268,11 +287,18 @@ def main():
                           "TFLOPs": round(flops / us_ / 1e6, 1), "mfma_frac": round(flops / us_ / 1e6 / MFMA_PEAK_TFLOPS, 4)})
 
         steps_s = max(10, args.steps // 10)
-        for m in (2, 16):
+        xm2 = [torch.randn(2, k, generator=gen(52)).to(torch.bfloat16).to(dev) for _ in range(2)]
+        ws2 = torch.empty(sl0.workspace_bytes(2) // 4, device=dev, dtype=torch.float32)
+        t = time_graph(lambda i: kernels.vq_linear_sliced(xm2[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2),
+                       s_rot, steps_s * 2, 3, dev)
+        add("cfg3 14336x4096 bf16", "a:sliced-gemv", 2, t, vq_alg_bytes(c3, 2), 2.0 * 2 * n * k)
+        del spool[1:]
+        torch.cuda.empty_cache()
+        for m in (1, 2, 16):
             xm = [torch.randn(m, k, generator=gen(50 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
             t = time_graph(lambda i: kernels.vq_linear(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n),
                            n_rot, steps_s * 2, 3, dev)
-            add("cfg3 14336x4096 bf16", "a:gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+            add("cfg3 14336x4096 bf16", "a:fused-gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
         for m in (64, 384, 1024):
             xm = [torch.randn(m, k, generator=gen(60 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
             t = time_graph(lambda i: kernels.vq_gemm_tile(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, n, None),
@@ -286,7 +312,16 @@ def main():
         torch.cuda.empty_cache()
         # config 3 down-proj shape
         c3d = vq_case(dev, 1003, 4096, 14336, 65536, 16, torch.bfloat16, n_rot)
-        for m, fn, band in ((1, kernels.vq_linear, "a:gemv"), (384, None, "b:tile-gemm")):
+        sld = kernels.vq_slice_indices(c3d["packed"], 16, 4096, 14336, 8, 65536, device=dev)
+        sdpool = [sld] + [kernels.SlicedIndices(sld.blob.clone(), sld.header) for _ in range(s_rot - 1)]
+        wsd = torch.empty(sld.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
+        xd = torch.randn(1, 14336, generator=gen(71)).to(torch.bfloat16).to(dev)
+        t = time_graph(lambda i: kernels.vq_linear_sliced(xd, sdpool[i], c3d["d_cb_act"], None, workspace=wsd),
+                       s_rot, steps_s * 2, 3, dev)
+        add("cfg3 4096x14336 bf16", "a:sliced-gemv", 1, t, vq_alg_bytes(c3d, 1), 2.0 * 4096 * 14336)
+        del sdpool, sld
+        torch.cuda.empty_cache()
+        for m, fn, band in ((1, kernels.vq_linear, "a:fused-gemv"), (384, None, "b:tile-gemm")):
             xm = [torch.randn(m, 14336, generator=gen(70 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
             if fn is not None:
                 f = lambda i: kernels.vq_linear(xm[i % 2], c3d["pool"][i], c3d["d_cb_act"], 16, 8, None, 4096)
