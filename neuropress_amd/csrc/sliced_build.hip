@@ -25,18 +25,17 @@ inline uint32_t host_read_index(const uint8_t* packed, int64_t n_bytes, int64_t 
   return (uint32_t)((w >> off) & ((1u << bits) - 1u));
 }
 
-inline void put_entry24(uint8_t* quad_lane, int j, uint32_t e) {
-  quad_lane[3 * j + 0] = (uint8_t)(e & 0xFF);
-  quad_lane[3 * j + 1] = (uint8_t)((e >> 8) & 0xFF);
-  quad_lane[3 * j + 2] = (uint8_t)((e >> 16) & 0xFF);
+// Entry j of a lane's 12-byte quad record: row = bytes 2j, 2j+1 (little endian), group = byte 8 + j.
+// In memory an entry is handled as row | group << 16.
+inline void put_entry(uint8_t* quad_lane, int j, uint32_t e) {
+  quad_lane[2 * j + 0] = (uint8_t)(e & 0xFF);
+  quad_lane[2 * j + 1] = (uint8_t)((e >> 8) & 0xFF);
+  quad_lane[8 + j] = (uint8_t)((e >> 16) & 0xFF);
 }
 
-inline uint32_t get_entry24(const uint8_t* quad_lane, int j) {
-  return (uint32_t)quad_lane[3 * j] | ((uint32_t)quad_lane[3 * j + 1] << 8) |
-         ((uint32_t)quad_lane[3 * j + 2] << 16);
+inline uint32_t get_entry(const uint8_t* quad_lane, int j) {
+  return (uint32_t)quad_lane[2 * j] | ((uint32_t)quad_lane[2 * j + 1] << 8) | ((uint32_t)quad_lane[8 + j] << 16);
 }
-
-inline int lds_bytes_needed(int slice_rows, int groups_max) { return slice_rows * 16 + (groups_max + 1) * 16; }
 
 // How the layer is cut: `row_blocks` row ranges of `rows_per_block` rows, and per
 // slice `parts[s]` group ranges.  One workgroup per (slice, group range, row block).
@@ -167,7 +166,7 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
       for (int r = 0; r < rows; ++r) {
         const uint32_t v = col[r];
         if ((int)(v / slice_rows) == job.slice)
-          task[(size_t)r].push_back((uint32_t)(g - g_begin) | ((v % slice_rows) << 11));
+          task[(size_t)r].push_back((v % slice_rows) | ((uint32_t)(g - g_begin) << 16));
       }
     }
     // Longest tasks first; 64 neighbours in that order share a strip.
@@ -175,7 +174,7 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
     std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(),
                      [&](int a, int b) { return task[(size_t)a].size() > task[(size_t)b].size(); });
-    const uint32_t pad = wg.g_count;  // zero activation vector, slice row 0
+    const uint32_t pad = (uint32_t)kSlicedPadRow;  // the zero row, group 0
     for (int s = 0; s * 64 < rows; ++s) {
       const int first = s * 64;
       const int lanes = std::min(64, rows - first);
@@ -195,7 +194,7 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
         }
         for (int64_t i = 0; i < nq * 4; ++i) {
           const uint32_t e = (t && i < (int64_t)t->size()) ? (*t)[(size_t)i] : pad;
-          put_entry24(&quads[base + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12], (int)(i % 4), e);
+          put_entry(&quads[base + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12], (int)(i % 4), e);
         }
       }
     }
@@ -243,9 +242,7 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
   NPAMD_REQUIRE(h.slice_rows >= 1 && h.slice_rows <= kSlicedMaxSliceRows &&
                     h.n_slices == (h.nc + h.slice_rows - 1) / h.slice_rows,
                 "%s: bad slice geometry", what);
-  NPAMD_REQUIRE(h.groups_max >= 1 && h.groups_max <= kSlicedMaxGroups &&
-                    lds_bytes_needed(h.slice_rows, h.groups_max) <= kSlicedLdsBytes,
-                "%s: group range %d does not fit in LDS", what, h.groups_max);
+  NPAMD_REQUIRE(h.groups_max >= 1 && h.groups_max <= kSlicedMaxGroups, "%s: group range %d too long", what, h.groups_max);
   NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1 && h.n_quads >= 1, "%s: bad counts", what);
   const int64_t end_wg = h.off_workgroups + (int64_t)h.n_workgroups * (int64_t)sizeof(SlicedWorkgroup);
   const int64_t end_rm = h.off_rowmap + (int64_t)h.n_workgroups * kSlicedTasks * 4;
@@ -282,10 +279,11 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
           c = 1;
         }
         for (int64_t i = 0; i < nq * 4; ++i) {
-          const uint32_t e = get_entry24(quads + ((size_t)wave.quad_begin + (size_t)(i / 4)) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4));
-          const uint32_t g_local = e & 0x7FFu, local = e >> 11;
-          NPAMD_REQUIRE(g_local <= wg.g_count && local < slice_len, "%s: workgroup %d: entry field out of range", what, w);
-          if (g_local < wg.g_count) {
+          const uint32_t e = get_entry(quads + ((size_t)wave.quad_begin + (size_t)(i / 4)) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4));
+          const uint32_t local = e & 0xFFFFu, g_local = e >> 16;
+          NPAMD_REQUIRE(g_local < wg.g_count && (local < slice_len || local == (uint32_t)kSlicedPadRow),
+                        "%s: workgroup %d: entry field out of range", what, w);
+          if (local != (uint32_t)kSlicedPadRow) {
             NPAMD_REQUIRE(row != kSlicedNoRow && i < (int64_t)wave.steps, "%s: workgroup %d: live entry in a lane without a row", what, w);
             uint8_t& f = filed[(size_t)row * G + wg.g_begin + g_local];
             NPAMD_REQUIRE(f == 0, "%s: index (%u, %u) filed twice", what, row, wg.g_begin + g_local);

@@ -15,12 +15,15 @@
 // A workgroup covers one (slice, group range) and up to 1024 rows.  Its tasks
 // are sorted by length and cut into strips of 64 (one strip per wave, at most
 // 16); a strip is padded to its longest task with entries that select an
-// all-zero activation vector.  The row each lane works for is stored per lane.
+// all-zero codebook row.  The row each lane works for is stored per lane.
 //
-// Entry (24 bits): bits 0..10 group inside the workgroup's range (the value
-// `g_count` selects the zero vector), bits 11..23 codebook row inside the slice.
-// Entries are stored four to a lane: quad q of a strip is 64 lanes x 12 bytes,
-// lane-major, so one 12-byte load per lane fetches steps 4q .. 4q + 3.
+// Entry (24 bits): a 16-bit codebook row inside the slice (kSlicedPadRow = the
+// zero row) and an 8-bit group inside the workgroup's range.  Entries are stored
+// four to a lane: quad q of a strip is 64 lanes x 12 bytes, lane-major, so one
+// 12-byte load per lane fetches steps 4q .. 4q + 3.  Inside the 12 bytes the
+// four rows come first (uint16 each), then the four groups (uint8 each): every
+// field sits on a 16- or 8-bit boundary and becomes an LDS address in one
+// shift.
 #pragma once
 
 #include <stdint.h>
@@ -30,11 +33,12 @@
 namespace npamd {
 
 constexpr uint32_t kSlicedMagic = 0x4C53504Eu;  // "NPSL"
-constexpr uint32_t kSlicedVersion = 1;
+constexpr uint32_t kSlicedVersion = 2;
 constexpr int kSlicedWaves = 16;             // waves (= strips) per workgroup
 constexpr int kSlicedTasks = kSlicedWaves * 64;
-constexpr int kSlicedMaxSliceRows = 8192;    // 13-bit in-slice row
-constexpr int kSlicedMaxGroups = 1536;       // groups per range; 11-bit field, and (1536 + 1) * 16 B beside a slice
+constexpr int kSlicedMaxSliceRows = 8192;    // rows of a slice (128 KiB of LDS)
+constexpr int kSlicedPadRow = 8192;          // row field of a padding entry: the zero row behind the slice
+constexpr int kSlicedMaxGroups = 256;        // groups per range (8-bit field; 4 KiB of activations in LDS)
 constexpr int kSlicedLdsBytes = 160 * 1024;
 constexpr int kSlicedQuadBytes = 64 * 12;
 constexpr uint32_t kSlicedNoRow = 0xFFFFFFFFu;

@@ -1,7 +1,7 @@
 // Decode GEMV over the slice-list form of the indices (see sliced_format.hpp).
 //
-// One workgroup of 16 waves holds one 8192-row codebook slice (128 KiB) and the
-// activations of its group range in LDS.  Every lane owns one output row and
+// One workgroup of 16 waves holds the activations of its group range (up to 4 KiB),
+// one 8192-row codebook slice (128 KiB) and a zero row in LDS.  Every lane owns one output row and
 // walks the entries filed under (slice, group range, row): two 16-byte LDS reads
 // (codebook row, activation vector) and four packed dot products per entry, the
 // sum kept in registers.  Each lane then writes one float into the partial-sum
@@ -49,25 +49,37 @@ struct Quad {
 // 8 in flight 12.1 us (the entries then arrive wave by wave instead of interleaved, and the
 // last waves start working late).
 constexpr int kQuadsInFlight = 3;
-constexpr int kSliceBytes = kSlicedMaxSliceRows * 16;  // the activations follow the slice in LDS
+// LDS map: activations of the group range, then the slice, then the zero row that
+// padding entries select.  Both bases fit the 16-bit offset field of an LDS read.
+constexpr int kLdsX = 0;
+constexpr int kLdsSlice = kSlicedMaxGroups * 16;
+constexpr int kLdsBytes = kLdsSlice + (kSlicedMaxSliceRows + 1) * 16;
 
 __device__ __forceinline__ void load_quad(Quad& q, const uint8_t* strip_lane, int qi) {
   __builtin_memcpy(&q, __builtin_assume_aligned(strip_lane + (size_t)qi * kSlicedQuadBytes, 4), 12);
 }
 
+template <uint32_t MASK>
+__device__ __forceinline__ uint32_t low_field(uint32_t v) {
+  uint32_t r;
+  asm("v_and_b32 %0, %1, %2" : "=v"(r) : "s"(MASK), "v"(v));
+  return r;
+}
+
 // The four entries of one quad: all eight LDS reads first, then the dot products.
+// A lane's record is four 16-bit rows followed by four 8-bit groups, so each LDS
+// address is one field shifted left by four.
 template <int ACT>
 __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, float& acc0, float& acc1) {
-  uint32_t e[4];
-  e[0] = q.d0 & 0xFFFFFFu;
-  e[1] = (q.d0 >> 24) | ((q.d1 & 0xFFFFu) << 8);
-  e[2] = (q.d1 >> 16) | ((q.d2 & 0xFFu) << 16);
-  e[3] = q.d2 >> 8;
+  // Each address is two instructions: extract the field, then shift-and-add the LDS
+  // base.  (Written as a plain mask, the low fields become shift + mask + add.)
+  const uint32_t row[4] = {low_field<0xFFFFu>(q.d0), q.d0 >> 16, low_field<0xFFFFu>(q.d1), q.d1 >> 16};
+  const uint32_t grp[4] = {low_field<0xFFu>(q.d2), (q.d2 >> 8) & 0xFFu, (q.d2 >> 16) & 0xFFu, q.d2 >> 24};
   u32x4 c[4], xv[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    c[j] = *reinterpret_cast<const u32x4*>(lds + ((e[j] >> 11) << 4));
-    xv[j] = *reinterpret_cast<const u32x4*>(lds + kSliceBytes + ((e[j] & 0x7FFu) << 4));
+    c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + (row[j] << 4));
+    xv[j] = *reinterpret_cast<const u32x4*>(lds + kLdsX + (grp[j] << 4));
   }
   acc0 = dot8<ACT>(c[0], xv[0], acc0);
   acc1 = dot8<ACT>(c[1], xv[1], acc1);
@@ -78,8 +90,8 @@ __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, floa
 template <int ACT>
 __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  u32x4* cb = reinterpret_cast<u32x4*>(lds);
-  u32x4* xl = reinterpret_cast<u32x4*>(lds + kSliceBytes);
+  u32x4* xl = reinterpret_cast<u32x4*>(lds + kLdsX);
+  u32x4* cb = reinterpret_cast<u32x4*>(lds + kLdsSlice);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -96,11 +108,10 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     const int slice_len = min(a.slice_rows, a.nc - (int)wg.slice * a.slice_rows);
     const u32x4* src = a.codebook + (int64_t)wg.slice * a.slice_rows;
     const int g_count = (int)wg.g_count;
-    u32x4 t[8], xt[2];
+    u32x4 t[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) xt[i] = a.x[wg.g_begin + min(tid + i * kSlicedTasks, g_count - 1)];
+    const u32x4 xt = a.x[wg.g_begin + min(tid, g_count - 1)];
     __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
     // The first quads (past the strip's end: its last quad again, or quad 0
     // of the blob for a wave without a strip; no branch around a load).
@@ -110,12 +121,8 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int g = tid + i * kSlicedTasks;
-      if (g < g_count) xl[g] = xt[i];
-      else if (g == g_count) xl[g] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
-    }
+    if (tid < g_count) xl[tid] = xt;
+    if (tid == kSlicedTasks - 1) cb[kSlicedPadRow] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
   }
   const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
   __syncthreads();
@@ -176,7 +183,7 @@ template <int ACT>
 int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void* x, int64_t ldx,
                   const void* codebook, const float* bias, void* y, int64_t ldy, int M, float* workspace,
                   hipStream_t st, const char* what) {
-  const int lds = kSliceBytes + (h.groups_max + 1) * 16;
+  const int lds = kLdsBytes;
   static int reserved = 0;
   if (lds > 64 * 1024 && lds > reserved) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT>),
@@ -222,7 +229,7 @@ extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_slic
   NPAMD_REQUIRE(h.n > 0 && h.k > 0 && h.vl == 8 && h.k % 8 == 0 && h.nc >= 1, "%s: bad layer shape in header", what);
   NPAMD_REQUIRE(h.slice_rows >= 1 && h.slice_rows <= kSlicedMaxSliceRows && h.groups_max >= 1 &&
                     h.groups_max <= kSlicedMaxGroups,
-                "%s: slice geometry does not fit in LDS", what);
+                "%s: slice geometry does not fit the kernel's LDS map", what);
   NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1, "%s: bad counts in header", what);
   NPAMD_REQUIRE(ldx >= h.k && ldy >= h.n, "%s: row stride smaller than the row", what);
   if (M == 0) return NPAMD_OK;

@@ -68,8 +68,8 @@ def decode_sliced_blob(blob: np.ndarray) -> tuple[np.ndarray, dict]:
     """Read a slice-list blob back into the ``[N, K/8]`` index matrix it was built from.
 
     An independent reader of the layout (header, workgroup records with their
-    16 wave records, per-lane row map, 24-bit entries four to a 12-byte lane
-    record).  ``hits`` counts how often each (row, group) pair was filed and
+    16 wave records, per-lane row map, and per lane and quad a 12-byte record of
+    four uint16 codebook rows followed by four uint8 groups).  ``hits`` counts how often each (row, group) pair was filed and
     ``writes`` how often each (partial, row) cell is written; both must be 1
     everywhere.
     """
@@ -83,7 +83,7 @@ def decode_sliced_blob(blob: np.ndarray) -> tuple[np.ndarray, dict]:
     n, groups, n_wg = h["n"], h["k"] // 8, h["n_workgroups"]
     wgs = np.frombuffer(blob, dtype="<u4", count=n_wg * 40, offset=h["off_workgroups"]).reshape(n_wg, 40).astype(np.int64)
     rowmap = np.frombuffer(blob, dtype="<u4", count=n_wg * 1024, offset=h["off_rowmap"]).reshape(n_wg, 16, 64).astype(np.int64)
-    quads = np.frombuffer(blob, dtype=np.uint8, count=h["n_quads"] * 768, offset=h["off_entries"]).reshape(-1, 64, 4, 3)
+    quads = np.frombuffer(blob, dtype=np.uint8, count=h["n_quads"] * 768, offset=h["off_entries"]).reshape(-1, 64, 12)
     idx = np.full((n, groups), -1, dtype=np.int64)
     hits = np.zeros((n, groups), dtype=np.int32)
     writes = np.zeros((h["n_partials"], n), dtype=np.int32)
@@ -97,14 +97,14 @@ def decode_sliced_blob(blob: np.ndarray) -> tuple[np.ndarray, dict]:
             nq = (steps + 3) // 4
             if nq == 0:
                 continue
-            q = quads[quad_begin : quad_begin + nq].astype(np.int64)  # [nq, lane, 4, 3]
-            e = q[..., 0] | (q[..., 1] << 8) | (q[..., 2] << 16)  # [nq, lane, 4]
-            e = e.transpose(1, 0, 2).reshape(64, nq * 4)  # [lane, step]
-            g_local, local = e & 0x7FF, e >> 11
-            live = g_local < g_count
+            q = quads[quad_begin : quad_begin + nq].astype(np.int64)  # [nq, lane, 12]
+            local = (q[..., 0:8:2] | (q[..., 1:8:2] << 8)).transpose(1, 0, 2).reshape(64, nq * 4)  # [lane, step]
+            g_local = q[..., 8:12].transpose(1, 0, 2).reshape(64, nq * 4)
+            live = local != 8192  # 8192 = the zero row padding entries select
+            assert (g_local < g_count).all() and (local[live] < h["slice_rows"]).all()
             assert not live[:, steps:].any(), "live entry beyond the strip's step count"
             assert not live[~has_row].any(), "live entry in a lane without a row"
-            rr = np.broadcast_to(rows[:, None], e.shape)[live]
+            rr = np.broadcast_to(rows[:, None], local.shape)[live]
             gg = (g_begin + g_local)[live]
             idx[rr, gg] = (sl * h["slice_rows"] + local)[live]
             np.add.at(hits, (rr, gg), 1)

@@ -59,8 +59,7 @@ def test_build_round_trip(n, k, nc, bits, zipf):
     assert h["n_entries"] == n * (k // 8) and h["total_bytes"] == blob.numel()
     assert np.array_equal(dec, idx.numpy())
     assert (info["hits"] == 1).all() and (info["writes"] == 1).all()
-    # LDS budget of the kernel: one slice + the group range's activations + a zero vector.
-    assert 8192 * 16 + (h["groups_max"] + 1) * 16 <= 160 * 1024
+    assert h["groups_max"] <= 256  # the kernel's LDS map: 4 KiB of activations, a slice, a zero row
 
 
 def test_build_fills_the_requested_workgroups():
@@ -131,12 +130,13 @@ def test_check_rejects_damaged_blobs():
     # and a row outside the layer must all be caught.
     quads = h["off_entries"]
     bad = blob.clone()
-    bad[quads : quads + 3] = torch.tensor([0xFF, 0xFF, 0xFF], dtype=torch.uint8)
-    with pytest.raises(RuntimeError, match="out of range|filed twice|not filed"):
+    bad[quads : quads + 2] = torch.tensor([0xFF, 0xFF], dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="entry field out of range"):
         check(bad)
-    bad = blob.clone()
-    bad[quads + 3 : quads + 6] = bad[quads : quads + 3]
-    with pytest.raises(RuntimeError, match="filed twice|not filed|live entry"):
+    bad = blob.clone()  # entry 1 of lane 0 := entry 0 (row field, then group field)
+    bad[quads + 2 : quads + 4] = bad[quads : quads + 2]
+    bad[quads + 9] = bad[quads + 8]
+    with pytest.raises(RuntimeError, match="filed twice|not filed"):
         check(bad)
     bad = blob.clone()
     row0 = h["off_rowmap"]
