@@ -287,11 +287,12 @@ def main():
                           "TFLOPs": round(flops / us_ / 1e6, 1), "mfma_frac": round(flops / us_ / 1e6 / MFMA_PEAK_TFLOPS, 4)})
 
         steps_s = max(10, args.steps // 10)
-        xm2 = [torch.randn(2, k, generator=gen(52)).to(torch.bfloat16).to(dev) for _ in range(2)]
-        ws2 = torch.empty(sl0.workspace_bytes(2) // 4, device=dev, dtype=torch.float32)
-        t = time_graph(lambda i: kernels.vq_linear_sliced(xm2[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2),
-                       s_rot, steps_s * 2, 3, dev)
-        add("cfg3 14336x4096 bf16", "a:sliced-gemv", 2, t, vq_alg_bytes(c3, 2), 2.0 * 2 * n * k)
+        for m in (2, 4):
+            xm2 = [torch.randn(m, k, generator=gen(50 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
+            ws2 = torch.empty(sl0.workspace_bytes(m) // 4, device=dev, dtype=torch.float32)
+            t = time_graph(lambda i: kernels.vq_linear_sliced(xm2[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2),
+                           s_rot, steps_s * 2, 3, dev)
+            add("cfg3 14336x4096 bf16", "a:sliced-gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
         del spool[1:]
         torch.cuda.empty_cache()
         for m in (1, 2, 16):

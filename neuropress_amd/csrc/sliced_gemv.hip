@@ -1,7 +1,8 @@
 // Decode GEMV over the slice-list form of the indices (see sliced_format.hpp).
 //
-// One workgroup of 16 waves holds the activations of its group range (up to 4 KiB),
-// one 8192-row codebook slice (128 KiB) and a zero row in LDS.  Every lane owns one output row and
+// One workgroup of 16 waves holds the activations of its group range (up to 4 KiB
+// per token, up to four tokens per launch), one 8192-row codebook slice (128 KiB)
+// and a zero row in LDS.  Every lane owns one output row and
 // walks the entries filed under (slice, group range, row): two 16-byte LDS reads
 // (codebook row, activation vector) and four packed dot products per entry, the
 // sum kept in registers.  Each lane then writes one float into the partial-sum
@@ -14,7 +15,9 @@
 namespace npamd {
 
 struct SlicedArgs {
-  const u32x4* x;  // one token: K/8 vectors of eight 16-bit values
+  const uint16_t* x;  // first token of the launch; a token is K/8 vectors of eight 16-bit values
+  int64_t ldx;        // elements between tokens
+  int64_t token_stride;  // floats between the partial sums of consecutive tokens
   const u32x4* codebook;
   const SlicedWorkgroup* wgs;
   const uint32_t* rowmap;
@@ -51,9 +54,11 @@ struct Quad {
 constexpr int kQuadsInFlight = 3;
 // LDS map: activations of the group range, then the slice, then the zero row that
 // padding entries select.  Both bases fit the 16-bit offset field of an LDS read.
-constexpr int kLdsX = 0;
-constexpr int kLdsSlice = kSlicedMaxGroups * 16;
+constexpr int kMaxTokens = 4;  // tokens per launch: one codebook read feeds up to four dot products
+constexpr int kLdsX = 0;       // [group][token] vectors, tokens padded to a power of two
+constexpr int kLdsSlice = kSlicedMaxGroups * 16 * kMaxTokens;
 constexpr int kLdsBytes = kLdsSlice + (kSlicedMaxSliceRows + 1) * 16;
+static_assert(kLdsBytes <= kSlicedLdsBytes && kLdsSlice < 65536, "LDS map");
 
 __device__ __forceinline__ void load_quad(Quad& q, const uint8_t* strip_lane, int qi) {
   __builtin_memcpy(&q, __builtin_assume_aligned(strip_lane + (size_t)qi * kSlicedQuadBytes, 4), 12);
@@ -66,29 +71,36 @@ __device__ __forceinline__ uint32_t low_field(uint32_t v) {
   return r;
 }
 
-// The four entries of one quad: all eight LDS reads first, then the dot products.
-// A lane's record is four 16-bit rows followed by four 8-bit groups, so each LDS
-// address is one field shifted left by four.
-template <int ACT>
-__device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, float& acc0, float& acc1) {
-  // Each address is two instructions: extract the field, then shift-and-add the LDS
-  // base.  (Written as a plain mask, the low fields become shift + mask + add.)
+// The four entries of one quad.  A lane's record is four 16-bit rows followed by
+// four 8-bit groups, so each LDS address is one field extracted and shifted: two
+// instructions.  (Written as a plain mask, the low fields become shift + mask + add.)
+// Per entry: one codebook row and M activation vectors from LDS, 4 M dot products.
+template <int ACT, int M>
+__device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, float (&acc)[M][2]) {
+  constexpr int kShift = 4 + (M > 2 ? 2 : M - 1);  // log2 of the bytes per group in LDS
   const uint32_t row[4] = {low_field<0xFFFFu>(q.d0), q.d0 >> 16, low_field<0xFFFFu>(q.d1), q.d1 >> 16};
   const uint32_t grp[4] = {low_field<0xFFu>(q.d2), (q.d2 >> 8) & 0xFFu, (q.d2 >> 16) & 0xFFu, q.d2 >> 24};
-  u32x4 c[4], xv[4];
+  constexpr int kBatch = M > 2 ? 2 : 4;  // entries whose LDS reads are issued together
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + (row[j] << 4));
-    xv[j] = *reinterpret_cast<const u32x4*>(lds + kLdsX + (grp[j] << 4));
+  for (int j0 = 0; j0 < 4; j0 += kBatch) {
+    u32x4 c[kBatch], xv[kBatch][M];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + (row[j0 + j] << 4));
+      const uint8_t* xg = lds + kLdsX + (grp[j0 + j] << kShift);
+#pragma unroll
+      for (int m = 0; m < M; ++m) xv[j][m] = *reinterpret_cast<const u32x4*>(xg + m * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j)
+#pragma unroll
+      for (int m = 0; m < M; ++m) acc[m][j & 1] = dot8<ACT>(c[j], xv[j][m], acc[m][j & 1]);
   }
-  acc0 = dot8<ACT>(c[0], xv[0], acc0);
-  acc1 = dot8<ACT>(c[1], xv[1], acc1);
-  acc0 = dot8<ACT>(c[2], xv[2], acc0);
-  acc1 = dot8<ACT>(c[3], xv[3], acc1);
 }
 
-template <int ACT>
+template <int ACT, int M>
 __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs a) {
+  constexpr int MP = M > 2 ? 4 : M;  // token slots per group in LDS
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   u32x4* xl = reinterpret_cast<u32x4*>(lds + kLdsX);
   u32x4* cb = reinterpret_cast<u32x4*>(lds + kLdsSlice);
@@ -111,7 +123,9 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     u32x4 t[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
-    const u32x4 xt = a.x[wg.g_begin + min(tid, g_count - 1)];
+    // Thread t stages token t % MP of group t / MP (256 groups x 4 tokens at most).
+    const int xg = tid / MP, xm = tid % MP;
+    const u32x4 xt = reinterpret_cast<const u32x4*>(a.x + (int64_t)min(xm, M - 1) * a.ldx)[wg.g_begin + min(xg, g_count - 1)];
     __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
     // The first quads (past the strip's end: its last quad again, or quad 0
     // of the blob for a wave without a strip; no branch around a load).
@@ -121,7 +135,7 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
-    if (tid < g_count) xl[tid] = xt;
+    if (xg < g_count && xm < M) xl[tid] = xt;
     if (tid == kSlicedTasks - 1) cb[kSlicedPadRow] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
   }
   const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
@@ -129,14 +143,16 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
 
   // kQuadsInFlight quads stay in flight: each one is replaced by the quad that many
   // further on as soon as it has been read.
-  float acc0 = 0.f, acc1 = 0.f;
+  float acc[M][2];
+#pragma unroll
+  for (int m = 0; m < M; ++m) acc[m][0] = acc[m][1] = 0.f;
   int q0 = 0;
   for (; q0 + 2 * kQuadsInFlight <= nq; q0 += kQuadsInFlight) {
 #pragma unroll
     for (int i = 0; i < kQuadsInFlight; ++i) {
       const Quad cur = q[i];
       load_quad(q[i], strip_lane, q0 + i + kQuadsInFlight);
-      run_quad<ACT>(cur, lds, acc0, acc1);
+      run_quad<ACT, M>(cur, lds, acc);
     }
   }
 #pragma unroll
@@ -144,27 +160,33 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     if (q0 + i >= nq) break;
     const Quad cur = q[i];
     if (q0 + i + kQuadsInFlight < nq) load_quad(q[i], strip_lane, q0 + i + kQuadsInFlight);
-    run_quad<ACT>(cur, lds, acc0, acc1);
+    run_quad<ACT, M>(cur, lds, acc);
   }
   q0 += kQuadsInFlight;
 #pragma unroll
   for (int i = 0; i < kQuadsInFlight; ++i) {
     if (q0 + i >= nq) break;
-    run_quad<ACT>(q[i], lds, acc0, acc1);
+    run_quad<ACT, M>(q[i], lds, acc);
   }
-  if (row != kSlicedNoRow) a.partials[(size_t)wg.partial * a.n + row] = acc0 + acc1;
+  if (row != kSlicedNoRow) {
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+      a.partials[(size_t)m * a.token_stride + (size_t)wg.partial * a.n + row] = acc[m][0] + acc[m][1];
+  }
 }
 
-// y[row] = round(sum over the partial vectors + bias).  16 rows per block; the
-// partial vectors are dealt over 16 threads per row, whose sums are then added
-// in a fixed order.
+// y[token][row] = round(sum over the partial vectors + bias).  16 rows per block
+// (blockIdx.y = token); the partial vectors are dealt over 16 threads per row,
+// whose sums are then added in a fixed order.
 template <int ACT>
 __global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restrict__ partials, int n_partials,
                                                              int n, const float* __restrict__ bias,
-                                                             void* __restrict__ y) {
+                                                             void* __restrict__ y, int64_t ldy) {
   __shared__ float red[16][17];
   const int r = threadIdx.x & 15, j = threadIdx.x >> 4;
   const int row = blockIdx.x * 16 + r;
+  partials += (size_t)blockIdx.y * n_partials * n;
+  y = (uint16_t*)y + (size_t)blockIdx.y * ldy;
   float sum = 0.f;
   if (row < n)
     for (int p = j; p < n_partials; p += 16) sum += partials[(size_t)p * n + row];
@@ -179,34 +201,46 @@ __global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restr
   }
 }
 
+template <int ACT, int M>
+int launch_sliced_tokens(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
+  static int reserved = 0;
+  if (reserved == 0) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e != hipSuccess)
+      return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(e));
+    reserved = kLdsBytes;
+  }
+  sliced_gemv_kernel<ACT, M><<<n_workgroups, kSlicedTasks, kLdsBytes, st>>>(a);
+  return NPAMD_OK;
+}
+
 template <int ACT>
 int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void* x, int64_t ldx,
                   const void* codebook, const float* bias, void* y, int64_t ldy, int M, float* workspace,
                   hipStream_t st, const char* what) {
-  const int lds = kLdsBytes;
-  static int reserved = 0;
-  if (lds > 64 * 1024 && lds > reserved) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess)
-      return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
-    reserved = lds;
-  }
   SlicedArgs a;
   a.codebook = (const u32x4*)codebook;
   a.wgs = (const SlicedWorkgroup*)(blob + h.off_workgroups);
   a.rowmap = (const uint32_t*)(blob + h.off_rowmap);
   a.entries = blob + h.off_entries;
   a.n = h.n; a.nc = h.nc; a.slice_rows = h.slice_rows;
-  const size_t per_token = (size_t)h.n_partials * (size_t)h.n;
-  for (int m = 0; m < M; ++m) {
-    a.x = (const u32x4*)((const uint16_t*)x + (size_t)m * ldx);
-    a.partials = workspace + (size_t)m * per_token;
-    sliced_gemv_kernel<ACT><<<h.n_workgroups, kSlicedWaves * 64, lds, st>>>(a);
-    if (y)
-      sliced_reduce_kernel<ACT><<<(h.n + 15) / 16, 256, 0, st>>>(a.partials, h.n_partials, h.n, bias,
-                                                                    (uint16_t*)y + (size_t)m * ldy);
+  a.ldx = ldx;
+  a.token_stride = (int64_t)h.n_partials * (int64_t)h.n;
+  for (int m0 = 0; m0 < M; m0 += kMaxTokens) {
+    a.x = (const uint16_t*)x + (size_t)m0 * ldx;
+    a.partials = workspace + (size_t)m0 * a.token_stride;
+    int rc;
+    switch (M - m0 >= kMaxTokens ? kMaxTokens : M - m0) {
+      case 1: rc = launch_sliced_tokens<ACT, 1>(a, h.n_workgroups, st, what); break;
+      case 2: rc = launch_sliced_tokens<ACT, 2>(a, h.n_workgroups, st, what); break;
+      case 3: rc = launch_sliced_tokens<ACT, 3>(a, h.n_workgroups, st, what); break;
+      default: rc = launch_sliced_tokens<ACT, 4>(a, h.n_workgroups, st, what); break;
+    }
+    if (rc != NPAMD_OK) return rc;
   }
+  if (y)
+    sliced_reduce_kernel<ACT><<<dim3((h.n + 15) / 16, M), 256, 0, st>>>(workspace, h.n_partials, h.n, bias, y, ldy);
   return check_launch(what);
 }
 

@@ -46,7 +46,7 @@ def _run(gpu, L, act, **kw):
         (96, 12296, 65536, 16),  # K / 8 = 1537 groups: two group ranges are forced
     ],
 )
-@pytest.mark.parametrize("m", [1, 3])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7])
 def test_sliced_gemv_matches_oracle(gpu, oracle_lib, act, n, k, nc, bits, m):
     L = cases.vq_layer(900 + n + m, n, k, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
     y, _ = _run(gpu, L, act)
@@ -124,7 +124,7 @@ def test_sliced_wrapper_errors(gpu):
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act, monkeypatch):
-    """NPVQLinear: 1-2 tokens on a layer with a large codebook use the slice lists, more
+    """NPVQLinear: up to 4 tokens on a layer with a large codebook use the slice lists, more
     tokens the fused GEMV; both match the oracle; a HIP graph captured after
     prepare_sliced() replays to the same bits."""
     from neuropress_amd import kernels
@@ -132,7 +132,7 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
 
     monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
     n, k, nc = 384, 512, 20000
-    L = cases.vq_layer(41, n, k, nc, act=act, m=4, bias=True, std=0.05)
+    L = cases.vq_layer(41, n, k, nc, act=act, m=6, bias=True, std=0.05)
     proxy = mod.VQProxy(L["cb"]).to(gpu)
     layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], n, k, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
     calls = []
@@ -142,11 +142,13 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
     ref = _vq_ref(oracle_lib, L, act)
     y1 = layer(x[:1])
     y2 = layer(x[:2].reshape(1, 2, k))
-    y4 = layer(x)
-    assert calls == [1, 2] and y2.shape == (1, 2, n)
+    y4 = layer(x[:4])
+    y6 = layer(x)
+    assert calls == [1, 2, 4] and y2.shape == (1, 2, n)
     _check(y1, ref[:1])
     _check(y2.reshape(2, n), ref[:2])
-    _check(y4, ref)
+    _check(y4, ref[:4])
+    _check(y6, ref)
     # Graph capture: no host work may happen inside; the lists already exist.
     assert layer.prepare_sliced()
     static_x = x[:1].clone()
@@ -176,7 +178,7 @@ def test_module_without_prepared_lists_inside_capture_uses_fused_gemv(gpu, monke
     with torch.cuda.stream(s):
         monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 0)
         layer(x)  # warm the fused path outside the capture
-        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 2)
+        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 4)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=s):
