@@ -5,6 +5,8 @@
 // Fast kernels cover the layout the BASELINE config uses (4 bits, symmetric,
 // group size a power-of-two multiple of 32, K % 64 == 0); every other valid
 // combination (1/2/8 bits, zero points, odd K) runs the element-wise fallback.
+#include <stdlib.h>
+
 #include "gemm_tile.hpp"
 #include "gemv.hpp"
 
@@ -66,6 +68,171 @@ q4_dequant_kernel(const uint32_t* __restrict__ w_pack, const uint16_t* __restric
   }
 }
 
+// ---------------------------------------------------------------------------
+// Row-wise GEMV for 4-bit symmetric weights, fp16 activations, 1 or 2 tokens.
+//
+// A lane takes 16 bytes of one weight row = 32 nibbles = one 32-k group, so the
+// weight stream is read with plain coalesced 16-byte loads and the kernel is
+// meant to run at HBM speed.  Nibbles become fp16 without a subtraction or a
+// multiplication: a nibble in mantissa bits 0..3 of 0x6400 reads as 1024 + q, one
+// in bits 4..7 of 0x5400 as 64 + q, so with b[k] = 1024 for even k and 64 for odd k
+//     sum_k x[k] * (q[k] - 8) * s = s * (sum_k x[k] * (b[k] + q[k]) - sum_k (b[k] + 8) * x[k])
+// with the first sum taken by packed dot products (products exact in f32) and the
+// second, which depends on x only, precomputed per 32-k group.  One shift and four
+// and-or instructions turn eight nibbles into four fp16 pairs (k, k+4); x is staged
+// in LDS once per block in the same pair order and in a lane-major layout, so its
+// reads are conflict-free.  f32 accumulation; a group's sum is up to ~500 times
+// larger than its useful part, i.e. nine of the 24 bits: the result still carries
+// more bits than the fp16 output keeps (measured: error = output rounding).
+// ---------------------------------------------------------------------------
+struct Q4RowArgs {
+  const uint16_t* x; int64_t ldx;
+  const uint8_t* w_pack;   // [N, K/2]
+  const uint16_t* scale;   // [N, K/gs]
+  const float* bias; uint16_t* y; int64_t ldy;
+  int N, K;
+  int groups32;            // K / 32
+  int passes;              // ceil(groups32 / 64)
+  int scales_per_row;      // K / gs
+  int gs_shift;            // log2(gs / 32)
+};
+
+// Operands by value (a bit cast applied directly to a vector element reads element 0).
+__device__ __forceinline__ float fdot2_f16(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+
+// (v & mask) | magic in one instruction; the compiler emits two when both constants are literals.
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic));
+  return r;
+}
+
+constexpr int kQ4RowWaves = 4;   // waves per block; a wave owns R consecutive rows
+
+template <int R>
+struct Q4RowItem {   // one pass (64 groups of 32 k) of R rows
+  u32x4 w[R];
+  uint16_t sc[R];
+};
+
+template <int R>
+__device__ __forceinline__ void q4_row_load(Q4RowItem<R>& it, const Q4RowArgs& a, int r0, int p, int lane) {
+  const int g = min(p * 64 + lane, a.groups32 - 1);
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int n = min(r0 + i, a.N - 1);
+    it.w[i] = *reinterpret_cast<const u32x4*>(a.w_pack + (int64_t)n * (a.K / 2) + (int64_t)g * 16);
+    it.sc[i] = a.scale[(int64_t)n * a.scales_per_row + (g >> a.gs_shift)];
+  }
+}
+
+template <int M, int R>
+__device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4RowArgs& a, const u32x4* xs,
+                                               const float* off, int p, int lane, float (&acc)[R][M]) {
+  const bool live = p * 64 + lane < a.groups32;
+  const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+  u32x4 xv[M][4];
+  float of[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xv[m][j] = xs[((size_t)m * a.passes * 4 + (size_t)p * 4 + j) * 64 + lane];
+    of[m] = off[(m * a.passes + p) * 64 + lane];
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    float g_acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) g_acc[m] = -of[m];
+    const uint32_t wd[4] = {it.w[i].x, it.w[i].y, it.w[i].z, it.w[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t u = wd[j], u8 = u >> 8;
+      const uint32_t p0 = and_or(u, 0x000F000Fu, magic_lo);   // (1024 + q0, 1024 + q4)
+      const uint32_t p1 = and_or(u, 0x00F000F0u, magic_hi);   // (64 + q1, 64 + q5)
+      const uint32_t p2 = and_or(u8, 0x000F000Fu, magic_lo);  // (1024 + q2, 1024 + q6)
+      const uint32_t p3 = and_or(u8, 0x00F000F0u, magic_hi);  // (64 + q3, 64 + q7)
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const u32x4 xx = xv[m][j];
+        float t = g_acc[m];
+        t = fdot2_f16(p0, xx.x, t);
+        t = fdot2_f16(p1, xx.y, t);
+        t = fdot2_f16(p2, xx.z, t);
+        t = fdot2_f16(p3, xx.w, t);
+        g_acc[m] = t;
+      }
+    }
+    const float s_eff = live ? f16_bits_to_f32(it.sc[i]) : 0.f;
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[i][m] = __builtin_fmaf(s_eff, g_acc[m], acc[i][m]);
+  }
+}
+
+template <int M, int R>
+__global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4RowArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // xs[m][pass][piece 0..3][lane] (16-byte vectors), then off[m][pass][lane] (floats).
+  u32x4* xs = reinterpret_cast<u32x4*>(smem);
+  float* off = reinterpret_cast<float*>(smem + (size_t)M * a.passes * 4 * 64 * 16);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r0 = (blockIdx.x * kQ4RowWaves + wave) * R;
+
+  // The first pass of weights is requested before x is staged.
+  Q4RowItem<R> cur, nxt;
+  q4_row_load<R>(cur, a, r0, 0, lane);
+
+  // Stage x: one thread per (token, 32-k group): its four vectors go to the lane-major
+  // layout in (k, k+4) pair order, sum (b[k] + 8) * x[k] to the offset table.
+  for (int i = tid; i < M * a.passes * 64; i += kQ4RowWaves * 64) {
+    const int m = i / (a.passes * 64), g = i % (a.passes * 64);
+    const u32x4* xg = reinterpret_cast<const u32x4*>(a.x + (int64_t)m * a.ldx) + (size_t)g * 4;
+    float sum_even = 0.f, sum_odd = 0.f;  // over even / odd k of the group
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (g < a.groups32) v = permute_a_0415(xg[j]);
+      const uint32_t d[4] = {v.x, v.y, v.z, v.w};  // (k0,k4) (k1,k5) (k2,k6) (k3,k7)
+      sum_even += f16_bits_to_f32(d[0] & 0xFFFFu) + f16_bits_to_f32(d[0] >> 16) +
+                  f16_bits_to_f32(d[2] & 0xFFFFu) + f16_bits_to_f32(d[2] >> 16);
+      sum_odd += f16_bits_to_f32(d[1] & 0xFFFFu) + f16_bits_to_f32(d[1] >> 16) +
+                 f16_bits_to_f32(d[3] & 0xFFFFu) + f16_bits_to_f32(d[3] >> 16);
+      xs[((size_t)m * a.passes * 4 + (size_t)(g >> 6) * 4 + j) * 64 + (g & 63)] = v;
+    }
+    off[i] = 1032.f * sum_even + 72.f * sum_odd;
+  }
+  __syncthreads();
+  if (r0 >= a.N) return;
+
+  float acc[R][M];
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[i][m] = 0.f;
+  // Two passes in flight: the next one is requested before the current one is used.
+  int p = 0;
+  for (; p + 2 <= a.passes; p += 2) {
+    q4_row_load<R>(nxt, a, r0, p + 1, lane);
+    q4_row_compute<M, R>(cur, a, xs, off, p, lane, acc);
+    q4_row_load<R>(cur, a, r0, min(p + 2, a.passes - 1), lane);
+    q4_row_compute<M, R>(nxt, a, xs, off, p + 1, lane, acc);
+  }
+  if (p < a.passes) q4_row_compute<M, R>(cur, a, xs, off, p, lane, acc);
+
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const float total = wave_reduce_sum(acc[i][m]);
+      const int n = r0 + i;
+      if (lane == 0 && n < a.N)
+        a.y[(int64_t)m * a.ldy + n] = (uint16_t)f32_to_f16_bits(total + (a.bias ? a.bias[n] : 0.f));
+    }
+}
+
 struct QCall {
   const void* x; int64_t ldx;
   const uint8_t* w_pack; const void* scale; const void* zp;
@@ -75,6 +242,7 @@ struct QCall {
   const char* what;
 };
 
+static int log2i(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
 static bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 static bool ptr_aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
@@ -92,11 +260,60 @@ static bool q_fast_ok(const QCall& c) {
          c.K > 0 && c.ldx % 8 == 0 && ptr_aligned(c.x, 16) && ptr_aligned(c.w_pack, 16);
 }
 
-static int log2i(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
+
+static int env_flag(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : dflt;
+}
+
+template <int M, int R>
+static int launch_q4_rowwise_r(const Q4RowArgs& a, hipStream_t st, const char* what) {
+  const int rows_per_block = R * kQ4RowWaves;
+  const int blocks = (a.N + rows_per_block - 1) / rows_per_block;
+  const int lds = M * a.passes * (4 * 64 * 16 + 64 * 4);
+  q4_rowwise_gemv_kernel<M, R><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
+  return check_launch(what);
+}
+
+template <int M>
+static int launch_q4_rowwise(const QCall& c) {
+  Q4RowArgs a;
+  a.x = (const uint16_t*)c.x; a.ldx = c.ldx;
+  a.w_pack = c.w_pack; a.scale = (const uint16_t*)c.scale;
+  a.bias = c.bias; a.y = (uint16_t*)c.y; a.ldy = c.ldy;
+  a.N = c.N; a.K = c.K;
+  a.groups32 = c.K / 32;
+  a.passes = (a.groups32 + 63) / 64;
+  a.scales_per_row = c.K / c.gs;
+  a.gs_shift = log2i(c.gs / 32);
+  // Rows per wave: 2 when that still leaves at least eight waves per compute unit (measured
+  // on 14336 x 4096: 1 row 12.0 us, 2 rows 10.4 us, 4 rows 10.8 us).
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  }
+  const int r_env = env_flag("NPAMD_Q4_ROWS", 0);
+  const int r = r_env ? r_env : (c.N >= 16 * cus ? 2 : 1);
+  if (r >= 4) return launch_q4_rowwise_r<M, 4>(a, c.st, c.what);
+  if (r >= 2) return launch_q4_rowwise_r<M, 2>(a, c.st, c.what);
+  return launch_q4_rowwise_r<M, 1>(a, c.st, c.what);
+}
+
+// The row-wise kernel serves fp16 activations, one token (at two tokens the MFMA GEMV is as fast:
+// 13.5 vs 13.8 us on 14336 x 4096), x staged in at most 64 KiB of LDS.
+static bool q4_rowwise_ok(const QCall& c) {
+  const int passes = (c.K / 32 + 63) / 64;
+  return c.act == NPAMD_F16 && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4) <= 64 * 1024 &&
+         ptr_aligned(c.scale, 2) && env_flag("NPAMD_Q4_ROWWISE", 1) != 0;
+}
 
 template <int ACT>
 static int q_dispatch(const QCall& c, bool gemv) {
   if (q_fast_ok(c)) {
+    if (gemv && q4_rowwise_ok(c)) return launch_q4_rowwise<1>(c);
     using P = Q4Provider<ACT>;
     typename P::Args a{c.w_pack, (const uint16_t*)c.scale, c.K / 64, c.K / c.gs, log2i(c.gs / 32)};
     if (gemv) {

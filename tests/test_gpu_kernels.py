@@ -205,6 +205,39 @@ def _q_ref(oracle_lib, L, act):
     return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
 
 
+@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 64)])
+@pytest.mark.parametrize("gs", [32, 128])
+@pytest.mark.parametrize("m", [1, 2])
+def test_q4_rowwise_gemv(gpu, oracle_lib, n, k, gs, m):
+    """fp16, 1-2 tokens: the row-wise kernel (nibbles read as 64 + q, group offsets folded out).
+    Row counts that are not a multiple of the four-row batch, K of one partial pass, of
+    several passes and of a partial last pass."""
+    from neuropress_amd import kernels
+
+    if k % gs:
+        pytest.skip("K not a multiple of the group size")
+    L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=torch.float16, m=m, bias=True)
+    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
+    assert y.shape == (m, n) and y.dtype == torch.float16
+    _check(y, _q_ref(oracle_lib, L, torch.float16))
+
+
+def test_q4_rowwise_gemv_large_activations(gpu):
+    """Activations of a few hundred: the folded-out offset (72 * sum x) is then far larger than
+    the result.  Checked against the contraction with the unrounded weight (q - 8) * s in
+    float64 (what the reference's fused kernel computes, kernels/q4_linear.cu:113-122): the
+    only error left must be the fp16 rounding of the output."""
+    from neuropress_amd import kernels
+
+    L = cases.q4_layer(731, 96, 4096, gs=32, act=torch.float16, m=1)
+    x = (L["x"].float() * 300).to(torch.float16)
+    q = torch.stack([L["blob"] & 0xF, L["blob"] >> 4], dim=-1).reshape(96, 4096).double() - 8
+    w = q * L["scale"].double().reshape(96, 128).repeat_interleave(32, dim=1)
+    ref = x.double() @ w.T
+    y = kernels.q_linear(x.to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, 32).cpu().double()
+    assert ((y - ref).abs() <= 2.0 ** -10 * ref.abs() + 1e-2).all()
+
+
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("gs", [32, 64, 128])
 @pytest.mark.parametrize("m", [1, 16, 17, 200])
