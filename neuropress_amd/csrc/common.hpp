@@ -51,6 +51,12 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);  // RNE (v_cvt_pk_bf16_f32)
 }
 
+template <int ACT>
+__device__ __forceinline__ float act_bits_to_f32(uint32_t v) {
+  if constexpr (ACT == NPAMD_BF16) return bf16_bits_to_f32(v);
+  else return f16_bits_to_f32(v);
+}
+
 // Two packed fp16 values -> two packed bf16 values (RNE of the exact f32 value).
 __device__ __forceinline__ uint32_t f16x2_to_bf16x2(uint32_t h2) {
   const f16x2 v = __builtin_bit_cast(f16x2, h2);

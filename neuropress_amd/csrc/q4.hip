@@ -69,7 +69,7 @@ q4_dequant_kernel(const uint32_t* __restrict__ w_pack, const uint16_t* __restric
 }
 
 // ---------------------------------------------------------------------------
-// Row-wise GEMV for 4-bit symmetric weights, fp16 activations, 1 or 2 tokens.
+// Row-wise GEMV for 4-bit symmetric weights, one token.
 //
 // A lane takes 16 bytes of one weight row = 32 nibbles = one 32-k group, so the
 // weight stream is read with plain coalesced 16-byte loads and the kernel is
@@ -84,6 +84,7 @@ q4_dequant_kernel(const uint32_t* __restrict__ w_pack, const uint16_t* __restric
 // reads are conflict-free.  f32 accumulation; a group's sum is up to ~500 times
 // larger than its useful part, i.e. nine of the 24 bits: the result still carries
 // more bits than the fp16 output keeps (measured: error = output rounding).
+// bf16 activations: 7 mantissa bits leave room for 128 + q only, three shifts.
 // ---------------------------------------------------------------------------
 struct Q4RowArgs {
   const uint16_t* x; int64_t ldx;
@@ -98,8 +99,12 @@ struct Q4RowArgs {
 };
 
 // Operands by value (a bit cast applied directly to a vector element reads element 0).
-__device__ __forceinline__ float fdot2_f16(uint32_t a, uint32_t b, float c) {
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+template <int ACT>
+__device__ __forceinline__ float fdot2_act(uint32_t a, uint32_t b, float c) {
+  if constexpr (ACT == NPAMD_BF16)
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+  else
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
 }
 
 // (v & mask) | magic in one instruction; the compiler emits two when both constants are literals.
@@ -128,11 +133,13 @@ __device__ __forceinline__ void q4_row_load(Q4RowItem<R>& it, const Q4RowArgs& a
   }
 }
 
-template <int M, int R>
+template <int ACT, int M, int R>
 __device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4RowArgs& a, const u32x4* xs,
                                                const float* off, int p, int lane, float (&acc)[R][M]) {
   const bool live = p * 64 + lane < a.groups32;
-  const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+  // fp16: 1024 + q (nibble in mantissa bits 0..3) and 64 + q (bits 4..7).
+  // bf16 has 7 mantissa bits: only 128 + q (bits 0..3 of 0x4300), so three shifts.
+  const uint32_t magic_lo = ACT == NPAMD_BF16 ? 0x43004300u : 0x64006400u, magic_hi = 0x54005400u;
   u32x4 xv[M][4];
   float of[M];
 #pragma unroll
@@ -150,18 +157,24 @@ __device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4R
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t u = wd[j], u8 = u >> 8;
-      const uint32_t p0 = and_or(u, 0x000F000Fu, magic_lo);   // (1024 + q0, 1024 + q4)
-      const uint32_t p1 = and_or(u, 0x00F000F0u, magic_hi);   // (64 + q1, 64 + q5)
-      const uint32_t p2 = and_or(u8, 0x000F000Fu, magic_lo);  // (1024 + q2, 1024 + q6)
-      const uint32_t p3 = and_or(u8, 0x00F000F0u, magic_hi);  // (64 + q3, 64 + q7)
+      uint32_t p0, p1, p2, p3;
+      p0 = and_or(u, 0x000F000Fu, magic_lo);   // (b + q0, b + q4)
+      p2 = and_or(u8, 0x000F000Fu, magic_lo);  // (b + q2, b + q6)
+      if constexpr (ACT == NPAMD_BF16) {
+        p1 = and_or(u >> 4, 0x000F000Fu, magic_lo);   // (128 + q1, 128 + q5)
+        p3 = and_or(u >> 12, 0x000F000Fu, magic_lo);  // (128 + q3, 128 + q7)
+      } else {
+        p1 = and_or(u, 0x00F000F0u, magic_hi);   // (64 + q1, 64 + q5)
+        p3 = and_or(u8, 0x00F000F0u, magic_hi);  // (64 + q3, 64 + q7)
+      }
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         const u32x4 xx = xv[m][j];
         float t = g_acc[m];
-        t = fdot2_f16(p0, xx.x, t);
-        t = fdot2_f16(p1, xx.y, t);
-        t = fdot2_f16(p2, xx.z, t);
-        t = fdot2_f16(p3, xx.w, t);
+        t = fdot2_act<ACT>(p0, xx.x, t);
+        t = fdot2_act<ACT>(p1, xx.y, t);
+        t = fdot2_act<ACT>(p2, xx.z, t);
+        t = fdot2_act<ACT>(p3, xx.w, t);
         g_acc[m] = t;
       }
     }
@@ -171,7 +184,7 @@ __device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4R
   }
 }
 
-template <int M, int R>
+template <int ACT, int M, int R>
 __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4RowArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // xs[m][pass][piece 0..3][lane] (16-byte vectors), then off[m][pass][lane] (floats).
@@ -181,7 +194,8 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r0 = (blockIdx.x * kQ4RowWaves + wave) * R;
 
-  // The first pass of weights is requested before x is staged.
+  // The first pass of weights is requested before x is staged (requesting two here is
+  // slower: 11.5 vs 9.2 us on 14336 x 4096).
   Q4RowItem<R> cur, nxt;
   q4_row_load<R>(cur, a, r0, 0, lane);
 
@@ -196,13 +210,13 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
       u32x4 v = {0u, 0u, 0u, 0u};
       if (g < a.groups32) v = permute_a_0415(xg[j]);
       const uint32_t d[4] = {v.x, v.y, v.z, v.w};  // (k0,k4) (k1,k5) (k2,k6) (k3,k7)
-      sum_even += f16_bits_to_f32(d[0] & 0xFFFFu) + f16_bits_to_f32(d[0] >> 16) +
-                  f16_bits_to_f32(d[2] & 0xFFFFu) + f16_bits_to_f32(d[2] >> 16);
-      sum_odd += f16_bits_to_f32(d[1] & 0xFFFFu) + f16_bits_to_f32(d[1] >> 16) +
-                 f16_bits_to_f32(d[3] & 0xFFFFu) + f16_bits_to_f32(d[3] >> 16);
+      sum_even += act_bits_to_f32<ACT>(d[0] & 0xFFFFu) + act_bits_to_f32<ACT>(d[0] >> 16) +
+                  act_bits_to_f32<ACT>(d[2] & 0xFFFFu) + act_bits_to_f32<ACT>(d[2] >> 16);
+      sum_odd += act_bits_to_f32<ACT>(d[1] & 0xFFFFu) + act_bits_to_f32<ACT>(d[1] >> 16) +
+                 act_bits_to_f32<ACT>(d[3] & 0xFFFFu) + act_bits_to_f32<ACT>(d[3] >> 16);
       xs[((size_t)m * a.passes * 4 + (size_t)(g >> 6) * 4 + j) * 64 + (g & 63)] = v;
     }
-    off[i] = 1032.f * sum_even + 72.f * sum_odd;
+    off[i] = ACT == NPAMD_BF16 ? 136.f * (sum_even + sum_odd) : 1032.f * sum_even + 72.f * sum_odd;
   }
   __syncthreads();
   if (r0 >= a.N) return;
@@ -216,11 +230,11 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
   int p = 0;
   for (; p + 2 <= a.passes; p += 2) {
     q4_row_load<R>(nxt, a, r0, p + 1, lane);
-    q4_row_compute<M, R>(cur, a, xs, off, p, lane, acc);
+    q4_row_compute<ACT, M, R>(cur, a, xs, off, p, lane, acc);
     q4_row_load<R>(cur, a, r0, min(p + 2, a.passes - 1), lane);
-    q4_row_compute<M, R>(nxt, a, xs, off, p + 1, lane, acc);
+    q4_row_compute<ACT, M, R>(nxt, a, xs, off, p + 1, lane, acc);
   }
-  if (p < a.passes) q4_row_compute<M, R>(cur, a, xs, off, p, lane, acc);
+  if (p < a.passes) q4_row_compute<ACT, M, R>(cur, a, xs, off, p, lane, acc);
 
 #pragma unroll
   for (int i = 0; i < R; ++i)
@@ -229,7 +243,7 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
       const float total = wave_reduce_sum(acc[i][m]);
       const int n = r0 + i;
       if (lane == 0 && n < a.N)
-        a.y[(int64_t)m * a.ldy + n] = (uint16_t)f32_to_f16_bits(total + (a.bias ? a.bias[n] : 0.f));
+        store_from_f32<ACT>(a.y, (int64_t)m * a.ldy + n, total + (a.bias ? a.bias[n] : 0.f));
     }
 }
 
@@ -266,16 +280,16 @@ static int env_flag(const char* name, int dflt) {
   return (v && *v) ? atoi(v) : dflt;
 }
 
-template <int M, int R>
+template <int ACT, int M, int R>
 static int launch_q4_rowwise_r(const Q4RowArgs& a, hipStream_t st, const char* what) {
   const int rows_per_block = R * kQ4RowWaves;
   const int blocks = (a.N + rows_per_block - 1) / rows_per_block;
   const int lds = M * a.passes * (4 * 64 * 16 + 64 * 4);
-  q4_rowwise_gemv_kernel<M, R><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
+  q4_rowwise_gemv_kernel<ACT, M, R><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
   return check_launch(what);
 }
 
-template <int M>
+template <int ACT, int M>
 static int launch_q4_rowwise(const QCall& c) {
   Q4RowArgs a;
   a.x = (const uint16_t*)c.x; a.ldx = c.ldx;
@@ -297,23 +311,27 @@ static int launch_q4_rowwise(const QCall& c) {
   }
   const int r_env = env_flag("NPAMD_Q4_ROWS", 0);
   const int r = r_env ? r_env : (c.N >= 16 * cus ? 2 : 1);
-  if (r >= 4) return launch_q4_rowwise_r<M, 4>(a, c.st, c.what);
-  if (r >= 2) return launch_q4_rowwise_r<M, 2>(a, c.st, c.what);
-  return launch_q4_rowwise_r<M, 1>(a, c.st, c.what);
+  if (r >= 4) return launch_q4_rowwise_r<ACT, M, 4>(a, c.st, c.what);
+  if (r >= 2) return launch_q4_rowwise_r<ACT, M, 2>(a, c.st, c.what);
+  return launch_q4_rowwise_r<ACT, M, 1>(a, c.st, c.what);
 }
 
-// The row-wise kernel serves fp16 activations, one token (at two tokens the MFMA GEMV is as fast:
+// bf16: the row-wise kernel keeps the unrounded weight (q - 8) * s, while the dequant-then-matmul
+// path it is checked against rounds every weight to bf16 (8 bits); at K = 14336 the two differ by
+// up to 4.5e-2, more than the 1e-2 parity bound, so bf16 stays on the MFMA GEMV (which rounds the
+// same way) unless NPAMD_Q4_ROWWISE_BF16=1 asks for the faster, more exact kernel.
+// The row-wise kernel serves one token (at two tokens the MFMA GEMV is as fast:
 // 13.5 vs 13.8 us on 14336 x 4096), x staged in at most 64 KiB of LDS.
 static bool q4_rowwise_ok(const QCall& c) {
   const int passes = (c.K / 32 + 63) / 64;
-  return c.act == NPAMD_F16 && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4) <= 64 * 1024 &&
+  return (c.act == NPAMD_F16 || env_flag("NPAMD_Q4_ROWWISE_BF16", 0) != 0) && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4) <= 64 * 1024 &&
          ptr_aligned(c.scale, 2) && env_flag("NPAMD_Q4_ROWWISE", 1) != 0;
 }
 
 template <int ACT>
 static int q_dispatch(const QCall& c, bool gemv) {
   if (q_fast_ok(c)) {
-    if (gemv && q4_rowwise_ok(c)) return launch_q4_rowwise<1>(c);
+    if (gemv && q4_rowwise_ok(c)) return launch_q4_rowwise<ACT, 1>(c);
     using P = Q4Provider<ACT>;
     typename P::Args a{c.w_pack, (const uint16_t*)c.scale, c.K / 64, c.K / c.gs, log2i(c.gs / 32)};
     if (gemv) {

@@ -205,21 +205,23 @@ def _q_ref(oracle_lib, L, act):
     return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
 
 
-@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 64)])
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 64), (4200, 256)])
 @pytest.mark.parametrize("gs", [32, 128])
 @pytest.mark.parametrize("m", [1, 2])
-def test_q4_rowwise_gemv(gpu, oracle_lib, n, k, gs, m):
-    """fp16, 1-2 tokens: the row-wise kernel (nibbles read as 64 + q, group offsets folded out).
-    Row counts that are not a multiple of the four-row batch, K of one partial pass, of
-    several passes and of a partial last pass."""
+def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m):
+    """One fp16 token takes the row-wise kernel (nibbles read as base + q, group offsets folded
+    out), two tokens and bf16 the MFMA GEMV.  Row counts that are not a multiple of the rows per wave
+    (and enough rows for two per wave), K of one partial pass, of several passes and of a
+    partial last pass."""
     from neuropress_amd import kernels
 
     if k % gs:
         pytest.skip("K not a multiple of the group size")
-    L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=torch.float16, m=m, bias=True)
+    L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=act, m=m, bias=True)
     y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
-    assert y.shape == (m, n) and y.dtype == torch.float16
-    _check(y, _q_ref(oracle_lib, L, torch.float16))
+    assert y.shape == (m, n) and y.dtype == act
+    _check(y, _q_ref(oracle_lib, L, act))
 
 
 def test_q4_rowwise_gemv_large_activations(gpu):
