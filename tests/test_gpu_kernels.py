@@ -206,7 +206,7 @@ def _q_ref(oracle_lib, L, act):
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 64), (4200, 256)])
+@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 128), (4200, 256)])
 @pytest.mark.parametrize("gs", [32, 128])
 @pytest.mark.parametrize("m", [1, 2])
 def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m):
@@ -216,8 +216,6 @@ def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m):
     partial last pass."""
     from neuropress_amd import kernels
 
-    if k % gs:
-        pytest.skip("K not a multiple of the group size")
     L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=act, m=m, bias=True)
     y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
     assert y.shape == (m, n) and y.dtype == act
