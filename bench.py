@@ -267,7 +267,10 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": round(gbs_main, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs_main / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(gbs_main / HBM_PEAK_GBS, 4),
+            # FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch of this kernel on this workload, from
+            # the rocprofv3 --pmc runs summarised in profiles/vq_sliced_gemv_cfg3_14336x4096_m1.md
+            "traffic": 12795 * 1024 * 2 + 896 * 1024,
             "kernel": "sliced_gemv_kernel<bf16>", "algorithmic_bytes_per_launch": alg,
             "avg_launch_us": round(us_main, 3),
             "streamed_bytes_per_launch": sl0.total_bytes + sl0.n_workgroups * (8192 * 16) + sl0.n_partials * n * 4,
@@ -343,6 +346,37 @@ def main():
                                rot, steps_s * 2, 3, dev)
                 add(name, "a:gemv", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
             del cc
+            torch.cuda.empty_cache()
+        # config 4: residual VQ (65536 + 256 entry codebooks, Zipf(1.1) indices, per-row scale / bias), fp16
+        def zipf(gq, nc, count):
+            pz = 1.0 / torch.arange(1, nc + 1, dtype=torch.float64) ** 1.1
+            return torch.multinomial(pz / pz.sum(), count, replacement=True, generator=gq)
+
+        for nn_, kk in ((4096, 4096), (1024, 4096)):
+            g = gen(1004)
+            cnt = nn_ * kk // 8
+            cbm = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.float16).to(dev)
+            cbr = (torch.randn(256, 8, generator=g) * 0.02).to(torch.float16).to(dev)
+            pm = zipf(g, 65536, cnt).to(torch.int32).to(torch.int16).view(torch.uint8)
+            pr = zipf(g, 256, cnt).to(torch.uint8)
+            rsc = (torch.rand(nn_, generator=g) + 0.5).to(torch.float16).to(dev)
+            rbi = (torch.randn(nn_, generator=g) * 0.01).to(torch.float16).to(dev)
+            rot = max(2, min(64, POOL_BYTES // (pm.numel() + pr.numel())))
+            pms = [pm.to(dev).clone() for _ in range(rot)]
+            prs = [pr.to(dev).clone() for _ in range(rot)]
+            alg4 = lambda m: cnt * 3 + (65536 + 256) * 16 + nn_ * 4 + m * kk * 2 + m * nn_ * 2
+            for m in (1, 384):
+                xm = [torch.randn(m, kk, generator=gen(40 + m)).to(torch.float16).to(dev) for _ in range(2)]
+                if m == 1:
+                    f = lambda i: kernels.rvq_linear(xm[i % 2], pms[i], 16, prs[i], 8, cbm, cbr, rsc, rbi, nn_)
+                    band = "a:fused-gemv"
+                else:
+                    f = lambda i: torch.nn.functional.linear(
+                        xm[i % 2], kernels.rvq_dequant(pms[i], 16, prs[i], 8, cbm, cbr, rsc, rbi, nn_, kk, torch.float16))
+                    band = "c:decode+gemm"
+                t = time_graph(f, rot, steps_s * 2, 3, dev)
+                add(f"cfg4 rvq {nn_}x{kk} f16", band, m, t, alg4(m), 2.0 * m * nn_ * kk)
+            del pms, prs
             torch.cuda.empty_cache()
         # config 5: int4 group-affine, 14336x4096 fp16
         from neuropress_amd.t2n.packing import BitPacking4
