@@ -1,0 +1,106 @@
+"""Every entry point inside a HIP graph: replays (with eager work and synchronisation between
+them) must reproduce the eager result bit for bit.  The library launches plain kernels only
+(no allocation, no memset, no synchronisation), which is what makes the calls capturable."""
+
+import pytest
+import torch
+
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def _capture_and_replay(gpu, fn, make_inputs, n_replays=3):
+    """fn(inputs) -> tensor.  Captures fn on static inputs, then for each replay copies fresh
+    inputs in, replays, and compares with fn run eagerly on the same inputs."""
+    static = make_inputs(0)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        fn(static)  # warm up outside the capture (lazy module state, LDS attribute calls)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            out = fn(static)
+    for i in range(1, n_replays + 1):
+        fresh = make_inputs(i)
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = fn(fresh)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i} differs from the eager call"
+        _ = torch.randn(1024, device=gpu).sum().item()  # unrelated eager work between replays
+
+
+@pytest.mark.parametrize("m,tile", [(1, False), (16, False), (40, True)])
+def test_vq_fused_kernels_in_a_graph(gpu, m, tile):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(11, 200, 512, 65536, bits=16, act=torch.bfloat16, m=m, bias=True, std=0.05)
+    packed, cb, bias = L["packed"].to(gpu), L["cb"].to(torch.bfloat16).to(gpu), L["bias"].to(gpu)
+    mk = lambda i: [torch.randn(m, 512, generator=cases.gen(100 + i)).to(torch.bfloat16).to(gpu)]
+    if tile:
+        fn = lambda inp: kernels.vq_gemm_tile(inp[0], packed, cb, 16, 200, bias)
+    else:
+        fn = lambda inp: kernels.vq_linear(inp[0], packed, cb, 16, 8, bias, 200)
+    _capture_and_replay(gpu, fn, mk)
+
+
+def test_vq_dequant_and_widen_in_a_graph(gpu):
+    from neuropress_amd import kernels
+    from neuropress_amd.transforms.vq_packing import IndexPacking
+
+    cb = (torch.randn(1024, 8, generator=cases.gen(3)) * 0.05).to(torch.float16).to(gpu)
+
+    def mk(i):
+        idx = torch.randint(0, 1024, (64 * 32,), generator=cases.gen(200 + i))
+        return [IndexPacking.pack(idx, 10).to(gpu)]
+
+    _capture_and_replay(gpu, lambda inp: kernels.vq_dequant(inp[0], cb, 10, 64, 256, torch.bfloat16), mk)
+    _capture_and_replay(gpu, lambda inp: kernels.widen_indices_u16(inp[0], 64 * 32, 10), mk)
+
+
+@pytest.mark.parametrize("m", [1, 3])
+def test_sliced_gemv_in_a_graph(gpu, m):
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(12, 300, 256, 20000, act=torch.float16, m=m, std=0.05)
+    sl = kernels.vq_slice_indices(L["packed"], L["bits"], 300, 256, 8, 20000, device=gpu)
+    cb = L["cb"].to(gpu)
+    ws = torch.empty(sl.workspace_bytes(m) // 4, device=gpu, dtype=torch.float32)
+    mk = lambda i: [torch.randn(m, 256, generator=cases.gen(300 + i)).to(torch.float16).to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.vq_linear_sliced(inp[0], sl, cb, None, workspace=ws), mk)
+
+
+@pytest.mark.parametrize("m", [1, 4, 40])
+def test_rvq_in_a_graph(gpu, m):
+    from neuropress_amd import kernels
+
+    L = cases.rvq_layer(13, 80, 256, act=torch.float16, m=m)
+    a = [L[k].to(gpu) for k in ("pm", "pr", "cbm", "cbr", "scale", "wbias")]
+    mk = lambda i: [torch.randn(m, 256, generator=cases.gen(400 + i)).to(torch.float16).to(gpu)]
+    fn = lambda inp: kernels.rvq_linear(inp[0], a[0], L["bm"], a[1], L["br"], a[2], a[3], a[4], a[5], 80, None)
+    _capture_and_replay(gpu, fn, mk)
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 4, 40])
+def test_q4_in_a_graph(gpu, act, m):
+    """One fp16 token: the row-wise kernel; otherwise the MFMA GEMV (m <= 16) or the tile GEMM."""
+    from neuropress_amd import kernels
+
+    L = cases.q4_layer(14, 136, 512, gs=32, act=act, m=m, bias=True)
+    blob, sc, bias = L["blob"].to(gpu), L["scale"].to(gpu), L["bias"].to(gpu)
+    mk = lambda i: [torch.randn(m, 512, generator=cases.gen(500 + i)).to(act).to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.q_linear(inp[0], blob, sc, 4, 32, None, bias), mk)
+
+
+def test_q_dequant_in_a_graph(gpu):
+    from neuropress_amd import kernels
+    from neuropress_amd.t2n.packing import BitPacking4
+
+    sc = (torch.rand(64 * 8, generator=cases.gen(5)) * 0.02).to(torch.float16).to(gpu)
+    mk = lambda i: [BitPacking4.compress(
+        torch.randint(0, 16, (64, 256), generator=cases.gen(600 + i), dtype=torch.int64).to(torch.uint8)).to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.q_dequant(inp[0], sc, 4, 32, None, torch.float16), mk)
