@@ -155,8 +155,13 @@ int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, 
  * contents irrelevant before the call; afterwards it holds, per token, the
  * n_partials partial-sum vectors [n_partials][N] (f32) whose sum over the first
  * axis is the un-biased result.  With y == NULL only those are produced.
+ * `column_perm`: NULL, or K int32 column numbers (16-byte aligned, each < ldx):
+ * the kernel then reads x[m, column_perm[k]] wherever it would read x[m, k],
+ * i.e. the x[..., column_perm] the reference applies before every VQ matmul
+ * (neuropress/nn/np_vq_linear.py:1027-1028) without a separate gather kernel.
  */
-int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_sliced_header* header_host,
+int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
+                         const npamd_sliced_header* header_host,
                          const void* blob, const void* codebook, int codebook_dtype,
                          const float* bias, void* y, int64_t ldy, int M, int act_dtype,
                          void* workspace, int64_t workspace_bytes, void* stream);

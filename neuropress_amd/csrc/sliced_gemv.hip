@@ -18,6 +18,7 @@ struct SlicedArgs {
   const uint16_t* x;  // first token of the launch; a token is K/8 vectors of eight 16-bit values
   int64_t ldx;        // elements between tokens
   int64_t token_stride;  // floats between the partial sums of consecutive tokens
+  const int32_t* column_perm;  // optional [K]: the kernel reads x[perm[k]] where it would read x[k]
   const u32x4* codebook;
   const SlicedWorkgroup* wgs;
   const uint32_t* rowmap;
@@ -98,7 +99,7 @@ __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, floa
   }
 }
 
-template <int ACT, int M>
+template <int ACT, int M, bool PERM>
 __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs a) {
   constexpr int MP = M > 2 ? 4 : M;  // token slots per group in LDS
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -125,13 +126,28 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
     // Thread t stages token t % MP of group t / MP (256 groups x 4 tokens at most).
     const int xg = tid / MP, xm = tid % MP;
-    const u32x4 xt = reinterpret_cast<const u32x4*>(a.x + (int64_t)min(xm, M - 1) * a.ldx)[wg.g_begin + min(xg, g_count - 1)];
+    const uint16_t* xrow = a.x + (int64_t)min(xm, M - 1) * a.ldx;
+    const int xvec = (int)wg.g_begin + min(xg, g_count - 1);
+    u32x4 xt, perm_lo, perm_hi;
+    if constexpr (PERM) {  // the eight source columns of this vector; the elements follow below
+      perm_lo = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec];
+      perm_hi = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec + 1];
+    } else {
+      xt = reinterpret_cast<const u32x4*>(xrow)[xvec];
+    }
     __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
     // The first quads (past the strip's end: its last quad again, or quad 0
     // of the blob for a wave without a strip; no branch around a load).
 #pragma unroll
     for (int i = 0; i < kQuadsInFlight; ++i) load_quad(q[i], strip_lane, max(min(i, nq - 1), 0));
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PERM) {
+      const uint32_t pc[8] = {perm_lo.x, perm_lo.y, perm_lo.z, perm_lo.w, perm_hi.x, perm_hi.y, perm_hi.z, perm_hi.w};
+      uint32_t e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = xrow[pc[j]];
+      xt = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
@@ -201,25 +217,32 @@ __global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restr
   }
 }
 
-template <int ACT, int M>
-int launch_sliced_tokens(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
+template <int ACT, int M, bool PERM>
+int launch_sliced_tokens_p(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
   static int reserved = 0;
   if (reserved == 0) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M, PERM>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess)
       return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(e));
     reserved = kLdsBytes;
   }
-  sliced_gemv_kernel<ACT, M><<<n_workgroups, kSlicedTasks, kLdsBytes, st>>>(a);
+  sliced_gemv_kernel<ACT, M, PERM><<<n_workgroups, kSlicedTasks, kLdsBytes, st>>>(a);
   return NPAMD_OK;
+}
+
+template <int ACT, int M>
+int launch_sliced_tokens(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
+  return a.column_perm ? launch_sliced_tokens_p<ACT, M, true>(a, n_workgroups, st, what)
+                       : launch_sliced_tokens_p<ACT, M, false>(a, n_workgroups, st, what);
 }
 
 template <int ACT>
 int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void* x, int64_t ldx,
-                  const void* codebook, const float* bias, void* y, int64_t ldy, int M, float* workspace,
-                  hipStream_t st, const char* what) {
+                  const void* codebook, const int32_t* column_perm, const float* bias, void* y, int64_t ldy,
+                  int M, float* workspace, hipStream_t st, const char* what) {
   SlicedArgs a;
+  a.column_perm = column_perm;
   a.codebook = (const u32x4*)codebook;
   a.wgs = (const SlicedWorkgroup*)(blob + h.off_workgroups);
   a.rowmap = (const uint32_t*)(blob + h.off_rowmap);
@@ -248,9 +271,9 @@ int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void*
 
 using namespace npamd;
 
-extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_sliced_header* hp,
-                                    const void* blob, const void* codebook, int codebook_dtype,
-                                    const float* bias, void* y, int64_t ldy, int M, int act_dtype,
+extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
+                                    const npamd_sliced_header* hp, const void* blob, const void* codebook,
+                                    int codebook_dtype, const float* bias, void* y, int64_t ldy, int M, int act_dtype,
                                     void* workspace, int64_t workspace_bytes, void* stream) {
   const char* what = "npamd_vq_gemv_sliced";
   NPAMD_REQUIRE(hp != nullptr, "%s: header is null", what);
@@ -271,12 +294,13 @@ extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const npamd_slic
   NPAMD_REQUIRE(ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(codebook) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(blob) % 16) == 0 &&
-                    (reinterpret_cast<uintptr_t>(workspace) % 16) == 0,
-                "%s: x, codebook, blob and workspace must be 16-byte aligned (ldx a multiple of 8)", what);
+                    (reinterpret_cast<uintptr_t>(workspace) % 16) == 0 &&
+                    (reinterpret_cast<uintptr_t>(column_perm) % 16) == 0,
+                "%s: x, column_perm, codebook, blob and workspace must be 16-byte aligned (ldx a multiple of 8)", what);
   NPAMD_REQUIRE(workspace_bytes >= npamd_vq_sliced_workspace_bytes(&h, M), "%s: workspace of %lld bytes, %lld needed",
                 what, (long long)workspace_bytes, (long long)npamd_vq_sliced_workspace_bytes(&h, M));
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == NPAMD_BF16)
-    return launch_sliced<NPAMD_BF16>(h, (const uint8_t*)blob, x, ldx, codebook, bias, y, ldy, M, (float*)workspace, st, what);
-  return launch_sliced<NPAMD_F16>(h, (const uint8_t*)blob, x, ldx, codebook, bias, y, ldy, M, (float*)workspace, st, what);
+    return launch_sliced<NPAMD_BF16>(h, (const uint8_t*)blob, x, ldx, codebook, column_perm, bias, y, ldy, M, (float*)workspace, st, what);
+  return launch_sliced<NPAMD_F16>(h, (const uint8_t*)blob, x, ldx, codebook, column_perm, bias, y, ldy, M, (float*)workspace, st, what);
 }

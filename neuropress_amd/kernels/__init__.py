@@ -283,6 +283,7 @@ def vq_linear_sliced(
     bias: torch.Tensor | None = None,
     workspace: torch.Tensor | None = None,
     partials_only: bool = False,
+    column_perm: torch.Tensor | None = None,
 ) -> torch.Tensor | None:
     """Decode GEMV over the slice-list form, ``M <= 16`` (``npamd_vq_gemv_sliced``).
 
@@ -290,6 +291,8 @@ def vq_linear_sliced(
     *workspace*: optional float32 scratch of ``sliced.workspace_bytes(M) / 4`` elements;
     after the call it holds the ``[M, n_partials, N]`` partial sums.  With
     *partials_only* nothing else is computed and None is returned.
+    *column_perm*: int32 ``[K]``; the kernel then computes with ``x[:, column_perm]``
+    (the reference's input permutation, np_vq_linear.py:1027-1028) without materialising it.
     """
     what = "vq_linear_sliced"
     _check_device(what, x, sliced.blob, centroids, bias, workspace)
@@ -300,6 +303,10 @@ def vq_linear_sliced(
     if cb.dtype != x.dtype:
         raise RuntimeError(f"{what}: centroids must be in x's dtype ({x.dtype}), got {cb.dtype}")
     m, k = x.shape
+    if column_perm is not None:
+        if column_perm.dtype != torch.int32 or column_perm.numel() != sliced.k or not column_perm.is_contiguous():
+            raise RuntimeError(f"{what}: column_perm must be a contiguous int32 tensor of K={sliced.k} entries")
+        _check_device(what, x, column_perm)
     if k != sliced.k or cb.shape[0] != sliced.nc or cb.shape[1] != sliced.vl:
         raise RuntimeError(f"{what}: slice lists were built for K={sliced.k}, codebook [{sliced.nc}, {sliced.vl}]")
     need = sliced.workspace_bytes(max(m, 1))
@@ -310,7 +317,7 @@ def vq_linear_sliced(
     y = None if partials_only else torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
     b32 = _bias_f32(bias)
     _lib.call(
-        "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), sliced.header_ptr, sliced.blob.data_ptr(),
+        "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), _ptr(column_perm), sliced.header_ptr, sliced.blob.data_ptr(),
         cb.data_ptr(), _DT[cb.dtype], _ptr(b32), _ptr(y), sliced.n, m, _DT[x.dtype],
         workspace.data_ptr(), workspace.numel() * 4, _stream(x),
     )  # fmt: skip

@@ -461,14 +461,16 @@ class NPVQLinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """Band dispatch by token count (reference: neuropress/nn/np_vq_linear.py:1014-1058)."""
+        if self.backend in _FUSED_BACKENDS and x.dtype in (torch.float16, torch.bfloat16):
+            m = x.numel() // self.in_features
+            if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and self._sliced_ready(x):
+                return self._forward_sliced(x)  # applies column_perm inside the kernel
         if self.column_perm is not None:
             x = x[..., self.column_perm]
         if self.backend in _FUSED_BACKENDS:
             if x.dtype not in (torch.float16, torch.bfloat16):
                 return self._forward_dequant_gemm(x)  # fp32 activations: decode + GEMM
             m = x.numel() // self.in_features
-            if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and self._sliced_ready(x):
-                return self._forward_sliced(x)
             if m > _fused_max_tokens(self.backend):
                 if (
                     self.backend != VQBackend.CUDA_LUT
@@ -531,13 +533,21 @@ class NPVQLinear(nn.Module):
         from .. import kernels
 
         *leading, _ = x.shape
+        perm = None
+        if self.column_perm is not None:
+            perm = self._derived.get("perm_i32")
+            if perm is None or perm.device != x.device:
+                perm = self.column_perm.to(device=x.device, dtype=torch.int32).contiguous()
+                self._derived["perm_i32"] = perm
         try:
             y = kernels.vq_linear_sliced(
                 x.reshape(-1, self.in_features), self._derived["sliced"],
-                self.proxy.centroids_as(x.dtype), self._bias_f32(),
+                self.proxy.centroids_as(x.dtype), self._bias_f32(), column_perm=perm,
             )  # fmt: skip
         except RuntimeError as exc:
             self._fallback("vq_linear_sliced", "decode + GEMM", exc)
+            if self.column_perm is not None:
+                x = x[..., self.column_perm]
             return self._forward_dequant_gemm(x)
         return y.reshape(*leading, self.out_features)
 

@@ -187,3 +187,28 @@ def test_module_without_prepared_lists_inside_capture_uses_fused_gemv(gpu, monke
     torch.cuda.synchronize()
     assert "sliced" not in layer._derived
     assert torch.equal(y, layer(x)) or (y.float() - layer(x).float()).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 3, 6])
+def test_column_permutation_is_applied_inside_the_sliced_kernel(gpu, oracle_lib, act, m, monkeypatch):
+    """x[..., column_perm] (reference: np_vq_linear.py:1027-1028): the slice-list GEMV reads the
+    permuted columns itself (m <= 4); larger m permutes with torch first.  Both must equal the
+    oracle fed with the permuted activations."""
+    from neuropress_amd import kernels
+    from neuropress_amd.nn import np_vq_linear as mod
+
+    monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    n, k, nc = 200, 384, 20000
+    L = cases.vq_layer(51, n, k, nc, act=act, m=m, bias=True, std=0.05)
+    perm = torch.randperm(k, generator=cases.gen(52))
+    layer = mod.NPVQLinear(mod.VQProxy(L["cb"]).to(gpu), L["packed"], L["bits"], n, k, 8, "cuda_wmma",
+                           bias=L["bias"].float(), column_perm=perm).to(gpu)
+    seen = []
+    real = kernels.vq_linear_sliced
+    monkeypatch.setattr(kernels, "vq_linear_sliced",
+                        lambda *a, **kw: (seen.append(kw.get("column_perm") is not None), real(*a, **kw))[1])
+    y = layer(L["x"].to(gpu))
+    assert seen == ([True] if m <= 4 else [])
+    Lp = dict(L, x=L["x"][:, perm].contiguous())
+    _check(y, _vq_ref(oracle_lib, Lp, act))

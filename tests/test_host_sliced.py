@@ -165,10 +165,10 @@ def test_gemv_sliced_validates_before_touching_the_gpu():
     hp = ctypes.addressof(hdr)
 
     def call(**kw):
-        a = dict(x=16, ldx=k, hdr=hp, blob=16, cb=16, cbdt=_lib.F16, bias=None, y=16, ldy=n, m=1,
+        a = dict(x=16, ldx=k, perm=None, hdr=hp, blob=16, cb=16, cbdt=_lib.F16, bias=None, y=16, ldy=n, m=1,
                  act=_lib.F16, ws=16, wsb=1 << 30, st=None)  # fmt: skip
         a.update(kw)
-        _lib.call("npamd_vq_gemv_sliced", a["x"], a["ldx"], a["hdr"], a["blob"], a["cb"], a["cbdt"], a["bias"],
+        _lib.call("npamd_vq_gemv_sliced", a["x"], a["ldx"], a["perm"], a["hdr"], a["blob"], a["cb"], a["cbdt"], a["bias"],
                   a["y"], a["ldy"], a["m"], a["act"], a["ws"], a["wsb"], a["st"])  # fmt: skip
 
     with pytest.raises(RuntimeError, match="header is null"):
@@ -185,6 +185,8 @@ def test_gemv_sliced_validates_before_touching_the_gpu():
         call(x=None)
     with pytest.raises(RuntimeError, match="16-byte aligned"):
         call(x=8)
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        call(perm=4)
     with pytest.raises(RuntimeError, match="workspace of"):
         call(wsb=16)
     bad = ctypes.create_string_buffer(b"\0" * 128, 128)
