@@ -15,6 +15,7 @@ from .kernel_lowering import (  # noqa: F401
     KernelLowering,
     LoweringConfig,
     is_lowered,
+    prepare_decode,
     unlower_model,
 )
 from .nn import (  # noqa: F401

@@ -2,8 +2,12 @@
 // Nothing in this file touches the GPU.
 #include <string.h>
 
+#include <stdlib.h>
+
 #include <algorithm>
+#include <atomic>
 #include <numeric>
+#include <thread>
 #include <vector>
 
 #include "common.hpp"
@@ -14,6 +18,30 @@ using namespace npamd;
 namespace {
 
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// Host threads for the builder: NPAMD_BUILD_THREADS, else the core count, at most 16.
+int builder_threads() {
+  const char* v = getenv("NPAMD_BUILD_THREADS");
+  int t = (v && *v) ? atoi(v) : (int)std::thread::hardware_concurrency();
+  return t < 1 ? 1 : (t > 16 ? 16 : t);
+}
+
+// fn(i) for i in [0, count), dealt dynamically to the builder's threads.
+template <class Fn>
+void parallel_for(int count, Fn fn) {
+  const int threads = std::min(builder_threads(), count);
+  if (threads <= 1) {
+    for (int i = 0; i < count; ++i) fn(i);
+    return;
+  }
+  std::atomic<int> next{0};
+  std::vector<std::thread> pool;
+  for (int t = 0; t < threads; ++t)
+    pool.emplace_back([&] {
+      for (int i = next.fetch_add(1); i < count; i = next.fetch_add(1)) fn(i);
+    });
+  for (auto& th : pool) th.join();
+}
 
 inline uint32_t host_read_index(const uint8_t* packed, int64_t n_bytes, int64_t i, int bits) {
   const int64_t bit = i * (int64_t)bits;
@@ -102,13 +130,22 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   // Indices transposed to [G][N] so a (group, row range) scan is contiguous.
   std::vector<uint32_t> idx_t((size_t)n_idx);
   std::vector<int64_t> slice_count((size_t)S, 0);
-  for (int n = 0; n < N; ++n)
-    for (int g = 0; g < G; ++g) {
-      uint32_t v = host_read_index(packed, n_bytes, (int64_t)n * G + g, bits);
-      if (v > (uint32_t)nc - 1u) v = (uint32_t)nc - 1u;  // same clamp as the decode kernels
-      idx_t[(size_t)g * N + n] = v;
-      slice_count[v / slice_rows]++;
-    }
+  {
+    const int chunk = 256;  // rows per work item
+    const int chunks = (N + chunk - 1) / chunk;
+    std::vector<std::vector<int64_t>> counts((size_t)chunks, std::vector<int64_t>((size_t)S, 0));
+    parallel_for(chunks, [&](int c) {
+      for (int n = c * chunk; n < std::min(N, (c + 1) * chunk); ++n)
+        for (int g = 0; g < G; ++g) {
+          uint32_t v = host_read_index(packed, n_bytes, (int64_t)n * G + g, bits);
+          if (v > (uint32_t)nc - 1u) v = (uint32_t)nc - 1u;  // same clamp as the decode kernels
+          idx_t[(size_t)g * N + n] = v;
+          counts[(size_t)c][v / slice_rows]++;
+        }
+    });
+    for (auto& c : counts)
+      for (int s = 0; s < S; ++s) slice_count[(size_t)s] += c[(size_t)s];
+  }
 
   const Geometry geo = plan_geometry(N, G, slice_count, n_idx, target_workgroups);
   std::vector<int> partial_base((size_t)S);
@@ -138,15 +175,18 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   }
   const int n_wg = (int)jobs.size();
 
+  // Every workgroup is built on its own (quad numbers local to the workgroup), then the entry
+  // sections are concatenated in workgroup order.
   std::vector<SlicedWorkgroup> wgs((size_t)n_wg);
   std::vector<uint32_t> rowmap((size_t)n_wg * kSlicedTasks, kSlicedNoRow);
-  std::vector<uint8_t> quads;
-  std::vector<std::vector<uint32_t>> task((size_t)geo.rows_per_block);
-  std::vector<int> order;
-  int64_t real_entries = 0;
-  int groups_max = 1;
+  std::vector<std::vector<uint8_t>> wg_quads((size_t)n_wg);
+  std::vector<int64_t> wg_entries((size_t)n_wg, 0);
 
-  for (int w = 0; w < n_wg; ++w) {
+  parallel_for(n_wg, [&](int w) {
+    std::vector<std::vector<uint32_t>> task((size_t)geo.rows_per_block);
+    std::vector<int> order;
+    std::vector<uint8_t>& quads = wg_quads[(size_t)w];
+    int64_t real_entries = 0;
     const Job& job = jobs[w];
     SlicedWorkgroup& wg = wgs[w];
     memset(&wg, 0, sizeof(wg));
@@ -158,7 +198,6 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
     wg.partial = (uint32_t)(partial_base[job.slice] + job.part);
     wg.g_begin = (uint32_t)g_begin;
     wg.g_count = (uint32_t)(g_end - g_begin);
-    groups_max = std::max(groups_max, g_end - g_begin);
 
     for (int r = 0; r < rows; ++r) task[(size_t)r].clear();
     for (int g = g_begin; g < g_end; ++g) {
@@ -197,6 +236,25 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
           put_entry(&quads[base + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12], (int)(i % 4), e);
         }
       }
+    }
+    wg_entries[(size_t)w] = real_entries;
+  });
+
+  std::vector<uint8_t> quads;
+  int64_t real_entries = 0;
+  int groups_max = 1;
+  {
+    size_t total = 0;
+    for (auto& q : wg_quads) total += q.size();
+    quads.reserve(std::max<size_t>(total, kSlicedQuadBytes));
+    for (int w = 0; w < n_wg; ++w) {
+      const uint32_t base = (uint32_t)(quads.size() / kSlicedQuadBytes);
+      for (int s = 0; s < kSlicedWaves; ++s)
+        if (wgs[(size_t)w].wave[s].steps) wgs[(size_t)w].wave[s].quad_begin += base;
+      quads.insert(quads.end(), wg_quads[(size_t)w].begin(), wg_quads[(size_t)w].end());
+      std::vector<uint8_t>().swap(wg_quads[(size_t)w]);
+      real_entries += wg_entries[(size_t)w];
+      groups_max = std::max(groups_max, (int)wgs[(size_t)w].g_count);
     }
   }
   if (quads.empty()) quads.resize(kSlicedQuadBytes, 0);  // waves without a strip still load quad 0

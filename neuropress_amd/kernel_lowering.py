@@ -21,7 +21,7 @@ from pathlib import Path
 import torch
 from torch import nn
 
-__all__ = ["AutoKernelLowering", "KernelLowering", "LoweringConfig", "is_lowered", "unlower_model"]
+__all__ = ["AutoKernelLowering", "KernelLowering", "LoweringConfig", "is_lowered", "prepare_decode", "unlower_model"]
 
 LOGGER = logging.getLogger(__name__)
 
@@ -177,3 +177,16 @@ def unlower_model(model: nn.Module) -> None:
     for pname in [n for n, _ in model.named_children() if n.startswith(("_vq_proxy_", "_vq_res_proxy_"))]:
         delattr(model, pname)
     LOGGER.info("unlower_model: restored %d module(s) to quantized-weight form", len(replacements))
+
+
+def prepare_decode(model: nn.Module) -> int:
+    """Build, for every lowered VQ layer that is on a GPU and uses it, the slice-list form its
+    1-4 token calls read (``NPVQLinear.prepare_sliced``); returns the number of layers prepared.
+
+    The layers would otherwise do this host work at their first short call.  Call it after
+    moving the model to the GPU and before capturing a HIP graph (a capture must not contain
+    the host round trip).  No counterpart in the reference.
+    """
+    from .nn.np_vq_linear import NPVQLinear
+
+    return sum(1 for m in model.modules() if isinstance(m, NPVQLinear) and m.prepare_sliced())

@@ -268,9 +268,18 @@ def vq_slice_indices(
     size = ctypes.c_int64(0)
     args = (host.data_ptr(), host.numel(), int(bits), int(out_features), int(in_features),
             int(vector_len), int(num_centroids), int(target_workgroups))  # fmt: skip
-    _lib.call("npamd_vq_sliced_build", *args, None, 0, ctypes.byref(size))
-    blob = torch.empty(size.value, dtype=torch.uint8, pin_memory=dev.type == "cuda")
-    _lib.call("npamd_vq_sliced_build", *args, blob.data_ptr(), blob.numel(), ctypes.byref(size))
+    # One build into a buffer sized for the usual case (3 bytes per index, a third of padding,
+    # the tables); only if that is too small is the size asked for and the build repeated.
+    n_idx = int(out_features) * (int(in_features) // max(int(vector_len), 1))
+    blob = torch.empty(4 * n_idx + (2 << 20), dtype=torch.uint8)
+    lib = _lib.load()
+    rc = lib.npamd_vq_sliced_build(*args, blob.data_ptr(), blob.numel(), ctypes.byref(size))
+    if rc != 0 and size.value > blob.numel():
+        blob = torch.empty(size.value, dtype=torch.uint8)
+        rc = lib.npamd_vq_sliced_build(*args, blob.data_ptr(), blob.numel(), ctypes.byref(size))
+    if rc != 0:
+        raise RuntimeError(f"npamd_vq_sliced_build failed (code {rc}): {lib.npamd_last_error().decode('utf-8', 'replace')}")
+    blob = blob[: size.value]
     _lib.call("npamd_vq_sliced_check", blob.data_ptr(), blob.numel())
     header = bytes(blob[: _lib.SLICED_HEADER_BYTES].numpy().tobytes())
     return SlicedIndices(blob.to(dev), header)

@@ -212,3 +212,20 @@ def test_column_permutation_is_applied_inside_the_sliced_kernel(gpu, oracle_lib,
     assert seen == ([True] if m <= 4 else [])
     Lp = dict(L, x=L["x"][:, perm].contiguous())
     _check(y, _vq_ref(oracle_lib, Lp, act))
+
+
+def test_prepare_decode_builds_the_lists_of_every_eligible_layer(gpu, monkeypatch):
+    import neuropress_amd
+    from neuropress_amd.nn import np_vq_linear as mod
+
+    monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    big = cases.vq_layer(61, 128, 256, 20000, act=torch.float16)
+    small = cases.vq_layer(62, 128, 256, 256, act=torch.float16)  # 256-row codebook: stays on the fused GEMV
+    model = torch.nn.Sequential(
+        mod.NPVQLinear(mod.VQProxy(big["cb"]), big["packed"], big["bits"], 128, 256, 8, "cuda_wmma"),
+        mod.NPVQLinear(mod.VQProxy(small["cb"]), small["packed"], small["bits"], 128, 256, 8, "cuda_wmma"),
+    )
+    assert neuropress_amd.prepare_decode(model) == 0  # still on the CPU
+    model.to(gpu)
+    assert neuropress_amd.prepare_decode(model) == 1
+    assert "sliced" in model[0]._derived and "sliced" not in model[1]._derived
