@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-sweep]
 
-One "step" = one decode-step call (M=1 token) of BASELINE config 3's up/gate
+One "step" = one decode-step call (M=1 token) of the benchmark's configuration 3 up/gate
 layer (Llama-3-8B MLP, N=14336, K=4096, vector length 8, 65536-entry fp16
 codebook, 16-bit indices, bf16 activations) on synthetic seeded data already
 resident in HBM, through the kernels NPVQLinear uses for it: the slice-list

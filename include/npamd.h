@@ -169,7 +169,7 @@ int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
 /* ------------------------------------------------- residual VQ (RVQ) ---- */
 /*
  * Two codebooks + per-output-row fp16 scale and bias (no counterpart in the
- * reference; BASELINE config 4):
+ * reference; the benchmark's residual-VQ configuration):
  *   W[n, g*VL+j] = f16(f16(f16(Cm[im(n,g),j] + Cr[ir(n,g),j]) * s[n]) + b[n])
  * row_scale / row_bias: fp16 [N] or NULL.  Both codebooks fp16, same VL.
  */

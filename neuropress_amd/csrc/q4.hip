@@ -2,7 +2,7 @@
 //
 //   q = (w_pack[n, k/vpb] >> ((k%vpb)*nbits)) & mask ;  w = (float(q) - zp) * float(scale)
 //
-// Fast kernels cover the layout the BASELINE config uses (4 bits, symmetric,
+// Fast kernels cover the Q4_0 / GPTQ layout the benchmark uses (4 bits, symmetric,
 // group size a power-of-two multiple of 32, K % 64 == 0); every other valid
 // combination (1/2/8 bits, zero points, odd K) runs the element-wise fallback.
 #include <stdlib.h>

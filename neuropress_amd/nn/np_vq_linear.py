@@ -241,7 +241,7 @@ class NPVQLinear(nn.Module):
 
         ``W[n, :] = ((Cm[im] + Cr[ir]) * row_scale[n]) + row_bias[n]``
 
-    each operation rounded to fp16 (BASELINE config 4; not in the reference).
+    each operation rounded to fp16 (the benchmark's residual-VQ configuration; not in the reference).
     """
 
     def __init__(

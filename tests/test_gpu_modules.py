@@ -1,4 +1,4 @@
-"""GPU tests of the drop-in modules and of the full BASELINE sizes.
+"""GPU tests of the drop-in modules and of the full benchmark sizes (Llama-3-8B layers).
 
 Module tests: every band of NPVQLinear / NPLinear on the GPU against the
 torch-op specification of the same layer on the CPU.  Full-size tests use
@@ -107,7 +107,7 @@ def test_residual_module_bands(gpu, monkeypatch):
         _close(layer(x.to(gpu)), x.float() @ w.T)
 
 
-# ------------------------------------------------------- BASELINE full sizes ---
+# ------------------------------------------------------ benchmark full sizes ---
 
 
 @pytest.fixture(scope="module")

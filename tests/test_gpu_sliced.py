@@ -68,7 +68,7 @@ def test_sliced_gemv_zipf_indices(gpu, oracle_lib):
 
 
 def test_sliced_gemv_full_size_and_fused_gemv_agree(gpu, oracle_lib):
-    """BASELINE config 3 shape (14336 x 4096, 65536 x 8 codebook, bf16), one token: against the
+    """The headline benchmark shape (14336 x 4096, 65536 x 8 codebook, bf16), one token: against the
     oracle, against the fused GEMV (same f32-accumulated sum in another order), run to run,
     and through the partial sums left in the workspace."""
     from neuropress_amd import kernels
