@@ -290,7 +290,7 @@ def main():
                           "TFLOPs": round(flops / us_ / 1e6, 1), "mfma_frac": round(flops / us_ / 1e6 / MFMA_PEAK_TFLOPS, 4)})
 
         steps_s = max(10, args.steps // 10)
-        for m in (2, 4):
+        for m in (2, 4, 7):
             xm2 = [torch.randn(m, k, generator=gen(50 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
             ws2 = torch.empty(sl0.workspace_bytes(m) // 4, device=dev, dtype=torch.float32)
             t = time_graph(lambda i: kernels.vq_linear_sliced(xm2[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2),

@@ -146,7 +146,7 @@ int npamd_vq_sliced_check(const void* blob_host, int64_t blob_bytes);
 int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, int M);
 
 /*
- * Decode GEMV over the slice-list form, M <= NPAMD_GEMV_MAX_M (up to four tokens
+ * Decode GEMV over the slice-list form, M <= NPAMD_GEMV_MAX_M (up to seven tokens
  * share one pass over the entries; more tokens take further passes):
  *   y[m, n] = sum_k x[m, k] * codebook[idx(n, k/VL), k%VL] (+ bias[n]).
  * `header_host` is a host copy of the blob's header, `blob` the whole blob in

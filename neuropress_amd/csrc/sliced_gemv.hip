@@ -1,7 +1,7 @@
 // Decode GEMV over the slice-list form of the indices (see sliced_format.hpp).
 //
 // One workgroup of 16 waves holds the activations of its group range (up to 4 KiB
-// per token, up to four tokens per launch), one 8192-row codebook slice (128 KiB)
+// per token, up to seven tokens per launch), one 8192-row codebook slice (128 KiB)
 // and a zero row in LDS.  Every lane owns one output row and
 // walks the entries filed under (slice, group range, row): two 16-byte LDS reads
 // (codebook row, activation vector) and four packed dot products per entry, the
@@ -55,8 +55,9 @@ struct Quad {
 constexpr int kQuadsInFlight = 3;
 // LDS map: activations of the group range, then the slice, then the zero row that
 // padding entries select.  Both bases fit the 16-bit offset field of an LDS read.
-constexpr int kMaxTokens = 4;  // tokens per launch: one codebook read feeds up to four dot products
-constexpr int kLdsX = 0;       // [group][token] vectors, tokens padded to a power of two
+constexpr int kMaxTokens = 7;  // tokens per pass over the entries (an eighth token's activations would not fit in LDS)
+constexpr int kLdsX = 0;       // [token][group] vectors: a token's 256 vectors are contiguous, so the
+                               // lanes of a read spread over all sixteen 16-byte bank groups
 constexpr int kLdsSlice = kSlicedMaxGroups * 16 * kMaxTokens;
 constexpr int kLdsBytes = kLdsSlice + (kSlicedMaxSliceRows + 1) * 16;
 static_assert(kLdsBytes <= kSlicedLdsBytes && kLdsSlice < 65536, "LDS map");
@@ -78,7 +79,6 @@ __device__ __forceinline__ uint32_t low_field(uint32_t v) {
 // Per entry: one codebook row and M activation vectors from LDS, 4 M dot products.
 template <int ACT, int M>
 __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, float (&acc)[M][2]) {
-  constexpr int kShift = 4 + (M > 2 ? 2 : M - 1);  // log2 of the bytes per group in LDS
   const uint32_t row[4] = {low_field<0xFFFFu>(q.d0), q.d0 >> 16, low_field<0xFFFFu>(q.d1), q.d1 >> 16};
   const uint32_t grp[4] = {low_field<0xFFu>(q.d2), (q.d2 >> 8) & 0xFFu, (q.d2 >> 16) & 0xFFu, q.d2 >> 24};
   constexpr int kBatch = M > 2 ? 2 : 4;  // entries whose LDS reads are issued together
@@ -88,9 +88,9 @@ __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, floa
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {
       c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + (row[j0 + j] << 4));
-      const uint8_t* xg = lds + kLdsX + (grp[j0 + j] << kShift);
+      const uint8_t* xg = lds + kLdsX + (grp[j0 + j] << 4);
 #pragma unroll
-      for (int m = 0; m < M; ++m) xv[j][m] = *reinterpret_cast<const u32x4*>(xg + m * 16);
+      for (int m = 0; m < M; ++m) xv[j][m] = *reinterpret_cast<const u32x4*>(xg + m * (kSlicedMaxGroups * 16));
     }
 #pragma unroll
     for (int j = 0; j < kBatch; ++j)
@@ -101,7 +101,6 @@ __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, floa
 
 template <int ACT, int M, bool PERM>
 __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs a) {
-  constexpr int MP = M > 2 ? 4 : M;  // token slots per group in LDS
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   u32x4* xl = reinterpret_cast<u32x4*>(lds + kLdsX);
   u32x4* cb = reinterpret_cast<u32x4*>(lds + kLdsSlice);
@@ -124,16 +123,20 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     u32x4 t[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
-    // Thread t stages token t % MP of group t / MP (256 groups x 4 tokens at most).
-    const int xg = tid / MP, xm = tid % MP;
-    const uint16_t* xrow = a.x + (int64_t)min(xm, M - 1) * a.ldx;
+    // Thread t stages group t % 256 of tokens t / 256 and t / 256 + 4 (256 groups x 7 tokens at most).
+    constexpr int kXLoads = M > 4 ? 2 : 1;
+    const int xg = tid & (kSlicedMaxGroups - 1), xm = tid / kSlicedMaxGroups;
     const int xvec = (int)wg.g_begin + min(xg, g_count - 1);
-    u32x4 xt, perm_lo, perm_hi;
+    const uint16_t* xrow[kXLoads];
+    u32x4 xt[kXLoads], perm_lo, perm_hi;
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) xrow[i] = a.x + (int64_t)min(xm + 4 * i, M - 1) * a.ldx;
     if constexpr (PERM) {  // the eight source columns of this vector; the elements follow below
       perm_lo = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec];
       perm_hi = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec + 1];
     } else {
-      xt = reinterpret_cast<const u32x4*>(xrow)[xvec];
+#pragma unroll
+      for (int i = 0; i < kXLoads; ++i) xt[i] = reinterpret_cast<const u32x4*>(xrow[i])[xvec];
     }
     __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
     // The first quads (past the strip's end: its last quad again, or quad 0
@@ -143,15 +146,20 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (PERM) {
       const uint32_t pc[8] = {perm_lo.x, perm_lo.y, perm_lo.z, perm_lo.w, perm_hi.x, perm_hi.y, perm_hi.z, perm_hi.w};
-      uint32_t e[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = xrow[pc[j]];
-      xt = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+      for (int i = 0; i < kXLoads; ++i) {
+        uint32_t e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = xrow[i][pc[j]];
+        xt[i] = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+      }
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
-    if (xg < g_count && xm < M) xl[tid] = xt;
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i)
+      if (xg < g_count && xm + 4 * i < M) xl[(xm + 4 * i) * kSlicedMaxGroups + xg] = xt[i];
     if (tid == kSlicedTasks - 1) cb[kSlicedPadRow] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
   }
   const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
@@ -258,7 +266,10 @@ int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void*
       case 1: rc = launch_sliced_tokens<ACT, 1>(a, h.n_workgroups, st, what); break;
       case 2: rc = launch_sliced_tokens<ACT, 2>(a, h.n_workgroups, st, what); break;
       case 3: rc = launch_sliced_tokens<ACT, 3>(a, h.n_workgroups, st, what); break;
-      default: rc = launch_sliced_tokens<ACT, 4>(a, h.n_workgroups, st, what); break;
+      case 4: rc = launch_sliced_tokens<ACT, 4>(a, h.n_workgroups, st, what); break;
+      case 5: rc = launch_sliced_tokens<ACT, 5>(a, h.n_workgroups, st, what); break;
+      case 6: rc = launch_sliced_tokens<ACT, 6>(a, h.n_workgroups, st, what); break;
+      default: rc = launch_sliced_tokens<ACT, 7>(a, h.n_workgroups, st, what); break;
     }
     if (rc != NPAMD_OK) return rc;
   }

@@ -56,15 +56,16 @@ def _env_int(names: tuple[str, ...], default: int) -> int:
 # band ends at 16 here (2 in the reference, whose GEMV re-reads the weight per token).
 _FUSED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_FUSED_MAX_TOKENS",), 16)
 
-# Decode steps (1-4 tokens) of layers whose codebook is too large to sit in a
+# Decode steps (1-7 tokens) of layers whose codebook is too large to sit in a
 # compute unit's LDS next to the GEMV's buffers (more than 4096 rows): the fused
 # GEMV then pays one L2 lookup per index (34-35 us on a 14336 x 4096 layer with a
 # 65536-row codebook, any token count up to 16), while the slice-list GEMV
-# (kernels.vq_linear_sliced) keeps 8192-row codebook slices in LDS: 12.8 / 17.2 /
-# 24.5 / 29.1 us at 1 / 2 / 3 / 4 tokens, 38 us at 5.  The slice lists are built
-# on the host at first use (about 25 MB per such layer, on top of the packed
+# (kernels.vq_linear_sliced) keeps 8192-row codebook slices in LDS: 12.8 / 15.5 /
+# 21.3 / 24.1 / 29.2 / 32.0 us at 1 / 2 / 4 / 5 / 6 / 7 tokens; an eighth token needs
+# a second pass over the entries (40.8 us vs 36.4 us fused).  The slice lists are
+# built on the host at first use (about 25 MB per such layer, on top of the packed
 # stream the other bands keep reading).  0 disables the path.
-_SLICED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_SLICED_MAX_TOKENS",), 4)
+_SLICED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_SLICED_MAX_TOKENS",), 7)
 _SLICED_MIN_CENTROIDS: int = 4097
 _SLICED_MIN_INDICES: int = _env_int(("NEUROPRESS_VQ_SLICED_MIN_INDICES",), 1 << 20)
 

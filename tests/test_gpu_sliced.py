@@ -46,7 +46,7 @@ def _run(gpu, L, act, **kw):
         (96, 12296, 65536, 16),  # K / 8 = 1537 groups: two group ranges are forced
     ],
 )
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 7])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 9, 16])
 def test_sliced_gemv_matches_oracle(gpu, oracle_lib, act, n, k, nc, bits, m):
     L = cases.vq_layer(900 + n + m, n, k, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
     y, _ = _run(gpu, L, act)
@@ -124,7 +124,7 @@ def test_sliced_wrapper_errors(gpu):
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act, monkeypatch):
-    """NPVQLinear: up to 4 tokens on a layer with a large codebook use the slice lists, more
+    """NPVQLinear: up to 7 tokens on a layer with a large codebook use the slice lists, more
     tokens the fused GEMV; both match the oracle; a HIP graph captured after
     prepare_sliced() replays to the same bits."""
     from neuropress_amd import kernels
@@ -132,7 +132,7 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
 
     monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
     n, k, nc = 384, 512, 20000
-    L = cases.vq_layer(41, n, k, nc, act=act, m=6, bias=True, std=0.05)
+    L = cases.vq_layer(41, n, k, nc, act=act, m=9, bias=True, std=0.05)
     proxy = mod.VQProxy(L["cb"]).to(gpu)
     layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], n, k, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
     calls = []
@@ -142,13 +142,13 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
     ref = _vq_ref(oracle_lib, L, act)
     y1 = layer(x[:1])
     y2 = layer(x[:2].reshape(1, 2, k))
-    y4 = layer(x[:4])
-    y6 = layer(x)
-    assert calls == [1, 2, 4] and y2.shape == (1, 2, n)
+    y7 = layer(x[:7])
+    y9 = layer(x)
+    assert calls == [1, 2, 7] and y2.shape == (1, 2, n)
     _check(y1, ref[:1])
     _check(y2.reshape(2, n), ref[:2])
-    _check(y4, ref[:4])
-    _check(y6, ref)
+    _check(y7, ref[:7])
+    _check(y9, ref)
     # Graph capture: no host work may happen inside; the lists already exist.
     assert layer.prepare_sliced()
     static_x = x[:1].clone()
@@ -178,7 +178,7 @@ def test_module_without_prepared_lists_inside_capture_uses_fused_gemv(gpu, monke
     with torch.cuda.stream(s):
         monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 0)
         layer(x)  # warm the fused path outside the capture
-        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 4)
+        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 7)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=s):
@@ -190,10 +190,10 @@ def test_module_without_prepared_lists_inside_capture_uses_fused_gemv(gpu, monke
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m", [1, 3, 6])
+@pytest.mark.parametrize("m", [1, 3, 6, 10])
 def test_column_permutation_is_applied_inside_the_sliced_kernel(gpu, oracle_lib, act, m, monkeypatch):
     """x[..., column_perm] (reference: np_vq_linear.py:1027-1028): the slice-list GEMV reads the
-    permuted columns itself (m <= 4); larger m permutes with torch first.  Both must equal the
+    permuted columns itself (m <= 7); larger m permutes with torch first.  Both must equal the
     oracle fed with the permuted activations."""
     from neuropress_amd import kernels
     from neuropress_amd.nn import np_vq_linear as mod
@@ -209,7 +209,7 @@ def test_column_permutation_is_applied_inside_the_sliced_kernel(gpu, oracle_lib,
     monkeypatch.setattr(kernels, "vq_linear_sliced",
                         lambda *a, **kw: (seen.append(kw.get("column_perm") is not None), real(*a, **kw))[1])
     y = layer(L["x"].to(gpu))
-    assert seen == ([True] if m <= 4 else [])
+    assert seen == ([True] if m <= 7 else [])
     Lp = dict(L, x=L["x"][:, perm].contiguous())
     _check(y, _vq_ref(oracle_lib, Lp, act))
 
