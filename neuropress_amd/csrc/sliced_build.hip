@@ -65,6 +65,48 @@ inline uint32_t get_entry(const uint8_t* quad_lane, int j) {
   return (uint32_t)quad_lane[2 * j] | ((uint32_t)quad_lane[2 * j + 1] << 8) | ((uint32_t)quad_lane[8 + j] << 16);
 }
 
+// Order the entries of the 64 tasks of a strip so that, step by step, the LDS reads of a
+// wave collide as little as possible.  A 64-lane 16-byte LDS read is served in two halves of 32
+// lanes; a half takes as many cycles as its fullest 16-byte bank group holds distinct addresses
+// ((address / 16) % 16, two being free) -- measured: 2.2 ns conflict-free, 3.6 ns with four
+// addresses per group, 13.4 ns with sixteen.  Random rows give about five per group.  A lane may
+// sum its entries in any order, so for every step each lane takes, among its remaining
+// entries, the one whose activation vector (group % 16; shared vectors count once) and codebook
+// row (row % 16) fall into the emptiest groups of its half.
+void spread_bank_groups(std::vector<uint32_t>* const* tasks, int lanes, int64_t steps) {
+  constexpr int kXWeight = 2;  // the activation read is repeated per token
+  for (int64_t t = 0; t < steps; ++t) {
+    for (int half = 0; half < 2; ++half) {
+      int g_count[16] = {0}, r_count[16] = {0};
+      uint8_t g_seen[kSlicedMaxGroups] = {0};
+      for (int lane = half * 32; lane < std::min(lanes, half * 32 + 32); ++lane) {
+        std::vector<uint32_t>& e = *tasks[lane];
+        if ((int64_t)e.size() <= t) continue;
+        size_t best = (size_t)t;
+        int best_cost = 1 << 30;
+        for (size_t i = (size_t)t; i < e.size(); ++i) {
+          const uint32_t row = e[i] & 0xFFFFu, g = e[i] >> 16;
+          const int gc = g_seen[g] ? 0 : std::max(0, g_count[g & 15] - 1);
+          const int rc = std::max(0, r_count[row & 15] - 1);
+          const int cost = kXWeight * gc + rc;
+          if (cost < best_cost) {
+            best_cost = cost;
+            best = i;
+            if (cost == 0) break;
+          }
+        }
+        std::swap(e[(size_t)t], e[best]);
+        const uint32_t row = e[(size_t)t] & 0xFFFFu, g = e[(size_t)t] >> 16;
+        if (!g_seen[g]) {
+          g_seen[g] = 1;
+          ++g_count[g & 15];
+        }
+        ++r_count[row & 15];
+      }
+    }
+  }
+}
+
 // How the layer is cut: `row_blocks` row ranges of `rows_per_block` rows, and per
 // slice `parts[s]` group ranges.  One workgroup per (slice, group range, row block).
 struct Geometry {
@@ -182,6 +224,8 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   std::vector<std::vector<uint8_t>> wg_quads((size_t)n_wg);
   std::vector<int64_t> wg_entries((size_t)n_wg, 0);
 
+  const char* spread_env = getenv("NPAMD_SLICED_SPREAD");
+  const bool spread = !(spread_env && *spread_env == '0');
   parallel_for(n_wg, [&](int w) {
     std::vector<std::vector<uint32_t>> task((size_t)geo.rows_per_block);
     std::vector<int> order;
@@ -219,6 +263,11 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
       const int lanes = std::min(64, rows - first);
       const int64_t steps = (int64_t)task[(size_t)order[(size_t)first]].size();
       const int64_t nq = (steps + 3) / 4;
+      if (spread) {
+        std::vector<uint32_t>* strip_tasks[64];
+        for (int lane = 0; lane < lanes; ++lane) strip_tasks[lane] = &task[(size_t)order[(size_t)(first + lane)]];
+        spread_bank_groups(strip_tasks, lanes, steps);
+      }
       wg.wave[s].quad_begin = nq ? (uint32_t)(quads.size() / kSlicedQuadBytes) : 0u;
       wg.wave[s].steps = (uint32_t)steps;
       const size_t base = quads.size();
