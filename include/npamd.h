@@ -77,11 +77,19 @@ int npamd_vq_gemv(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_b
  * inside the kernel, dense weight never written.
  * Replaces vq_gemm_triton (neuropress/kernels/vq_triton.py:119-179) and the
  * WMMA GEMM branch of vq_linear_wmma (neuropress/kernels/vq_linear_wmma.cu:261-394).
+ * `workspace` (all three *_gemm_tile entry points): NULL, or 16-byte aligned device
+ * memory of npamd_gemm_tile_workspace_bytes(M, N, K) bytes.  With it, layers
+ * whose column blocks would not fill the GPU (few output features) split K over
+ * more workgroups and add the f32 partial tiles in a second kernel; without it,
+ * or when it is too small, K is not split.  Contents irrelevant before and after.
  */
 int npamd_vq_gemm_tile(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_bytes,
                        int bits, const void* codebook, int codebook_dtype, int nc, int vl,
                        const float* bias, void* y, int64_t ldy, int M, int N, int K,
-                       int act_dtype, void* stream);
+                       int act_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Bytes of workspace the *_gemm_tile entry points can use for this shape (0: K is not split). */
+int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K);
 
 /*
  * Widen a bit-stream to one uint16 per index (the layout the fast kernels
@@ -193,7 +201,7 @@ int npamd_rvq_gemm_tile(const void* x, int64_t ldx,
                         const void* cb_main_f16, int nc_main, const void* cb_res_f16, int nc_res,
                         const void* row_scale_f16, const void* row_bias_f16, int vl,
                         const float* bias, void* y, int64_t ldy, int M, int N, int K,
-                        int act_dtype, void* stream);
+                        int act_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------- group-affine n-bit (Q4) ---- */
 /*
@@ -226,7 +234,7 @@ int npamd_q_gemv(const void* x, int64_t ldx, const uint8_t* w_pack, const void* 
 int npamd_q_gemm_tile(const void* x, int64_t ldx, const uint8_t* w_pack, const void* scale_f16,
                       const void* zero_point_f16, const float* bias, void* y, int64_t ldy,
                       int M, int N, int K, int nbits, int group_size, int act_dtype,
-                      void* stream);
+                      void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------ diagnostics ---- */
 /*

@@ -15,7 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libnpamd.so"
 
 F16, BF16, F32 = 0, 1, 2
 GEMV_MAX_M = 16
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -24,13 +24,15 @@ _int = ctypes.c_int
 # name -> argtypes, exactly the order of include/npamd.h
 _VQ_LINEAR = [_vp, _i64, _vp, _i64, _int, _vp, _int, _int, _int, _vp, _vp, _i64,
               _int, _int, _int, _int, _vp]  # fmt: skip
+_WS = [_vp, _i64]  # workspace pointer and size, before the stream, in the *_gemm_tile entry points
 _RVQ_LINEAR = [_vp, _i64, _vp, _i64, _int, _vp, _i64, _int, _vp, _int, _vp, _int, _vp, _vp, _int,
                _vp, _vp, _i64, _int, _int, _int, _int, _vp]  # fmt: skip
 _Q_LINEAR = [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _vp]
 SIGNATURES: dict[str, list] = {
     "npamd_vq_dequant": [_vp, _i64, _int, _vp, _int, _int, _i64, _vp, _int, _vp],
     "npamd_vq_gemv": _VQ_LINEAR,
-    "npamd_vq_gemm_tile": _VQ_LINEAR,
+    "npamd_vq_gemm_tile": _VQ_LINEAR[:-1] + _WS + [_vp],
+    "npamd_gemm_tile_workspace_bytes": [_int, _int, _int],
     "npamd_vq_widen_u16": [_vp, _i64, _int, _i64, _vp, _vp],
     "npamd_vq_sliced_build": [_vp, _i64, _int, _int, _int, _int, _int, _int, _vp, _i64,
                               ctypes.POINTER(_i64)],  # fmt: skip
@@ -40,15 +42,15 @@ SIGNATURES: dict[str, list] = {
     "npamd_rvq_dequant": [_vp, _i64, _int, _vp, _i64, _int, _vp, _int, _vp, _int, _vp, _vp, _int,
                           _int, _int, _vp, _int, _vp],  # fmt: skip
     "npamd_rvq_gemv": _RVQ_LINEAR,
-    "npamd_rvq_gemm_tile": _RVQ_LINEAR,
+    "npamd_rvq_gemm_tile": _RVQ_LINEAR[:-1] + _WS + [_vp],
     "npamd_q_dequant": [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _int, _vp],
     "npamd_q_gemv": _Q_LINEAR,
-    "npamd_q_gemm_tile": _Q_LINEAR,
+    "npamd_q_gemm_tile": _Q_LINEAR[:-1] + _WS + [_vp],
     "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
     "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],
 }
 
-_RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64}
+_RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64, "npamd_gemm_tile_workspace_bytes": _i64}
 SLICED_HEADER_BYTES = 128
 
 _lib: ctypes.CDLL | None = None

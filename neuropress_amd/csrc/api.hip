@@ -81,6 +81,21 @@ GemvPlan plan_gemv(int N, int chunks) {
   return p;
 }
 
+int plan_tile_splits(int M, int N, int chunks, int mw) {
+  const int env = env_int("NPAMD_TILE_SPLITS", 0);
+  const int cus = device_cu_count();
+  const int blocks = ((N + 63) / 64) * ((M + 128 * mw - 1) / (128 * mw));
+  int splits = 1;
+  if (env > 0) splits = env;
+  else if (blocks * 10 < cus * 7) splits = cus / blocks;
+  const int max_by_k = chunks / 8 > 1 ? chunks / 8 : 1;
+  if (splits > max_by_k) splits = max_by_k;
+  if (splits > 16) splits = 16;
+  return splits < 1 ? 1 : splits;
+}
+
+extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K);
+
 int plan_tile_mw(int M) {
   const int mw_env = env_int("NPAMD_TILE_MW", 0);
   if (mw_env >= 1 && mw_env <= 3) return mw_env;
@@ -90,6 +105,12 @@ int plan_tile_mw(int M) {
 
 }  // namespace npamd
 
-extern "C" int npamd_version(void) { return 1; }
+extern "C" int npamd_version(void) { return 2; }
+
+extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K < 64) return 0;
+  const int splits = npamd::plan_tile_splits(M, N, K / 64, npamd::plan_tile_mw(M));
+  return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
+}
 
 extern "C" const char* npamd_last_error(void) { return npamd::error_text(); }

@@ -25,6 +25,12 @@
 //           operand pair), keeps kDepth steps in flight in registers and
 //           writes a finished pair to LDS one iteration before its step.
 // One block barrier per macro-step, executed by all eight waves.
+//
+// Layers with few output columns (N = 4096: 64 column blocks) would leave most
+// compute units idle, and the decode rate per compute unit is the limit; for
+// them K is split over blockIdx.z, every split writes an f32 partial tile and
+// a second kernel adds the splits (two or more addends in a fixed order), the
+// bias, and rounds.
 #pragma once
 
 #include "providers.hpp"
@@ -45,6 +51,11 @@ struct GemmShape {
   int M, N, K;
   int chunks;  // K / 64 = number of macro-steps
   int steps;   // == chunks
+  // Split-K: blockIdx.z = split; split z contracts chunks [z * split_chunks, ...) and, when
+  // splits > 1, stores its f32 tile to partials[z][M][N] (no bias) for splitk_reduce_kernel.
+  int splits;
+  int split_chunks;
+  float* partials;
 };
 
 constexpr int kDepth = 8;  // steps in flight per producer wave (2 operands each)
@@ -73,22 +84,24 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: role branch is scalar
   const int m0 = blockIdx.y * BM;
   const int n0 = blockIdx.x * kTileCols;
+  const int chunk0 = blockIdx.z * s.split_chunks;                 // first chunk of this split
+  const int steps = min(s.split_chunks, s.chunks - chunk0);       // its number of macro-steps
 
   // Column blocks walk k in rotated order (iteration t contracts chunk
   // (t + rot) mod steps): at any instant different blocks read different parts
   // of the index rows and of x, which spreads the traffic over the L2 channels
   // instead of all blocks hitting the same few address bits in lock step.
-  const int rot = (int)((blockIdx.x * 7u) % (unsigned)s.steps);
+  const int rot = (int)((blockIdx.x * 7u) % (unsigned)steps);
   auto chunk_of = [&](int step) {
     const int kc = step + rot;
-    return kc >= s.steps ? kc - s.steps : kc;
+    return chunk0 + (kc >= steps ? kc - steps : kc);
   };
 
   // Both software pipelines are unrolled by their depth with no branches inside
   // (a branch would make the compiler drain every outstanding load at the join),
   // so all waves run `total` iterations: steps rounded up to a multiple of kDepth.
   // The padding iterations decode clamped addresses into buffers nobody reads.
-  const int total = (s.steps + kDepth - 1) / kDepth * kDepth;
+  const int total = (steps + kDepth - 1) / kDepth * kDepth;
 
   if (wave >= 4) {
     // ====================== producer wave q ================================
@@ -115,7 +128,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     typename Provider::PairRaw raws[kDepth];
     u32x4 ops[kDepth][2];
     auto load_raw = [&](typename Provider::PairRaw& raw, int step) {
-      prov.load_pair(raw, ncol, chunk_of(min(step, s.steps - 1)), jp);
+      prov.load_pair(raw, ncol, chunk_of(min(step, steps - 1)), jp);
     };
     auto store_w = [&](const u32x4 (&b)[2], int step) {
       uint8_t* dst = ws + (step & 1) * kWBufBytes + col * kRowBytes + jp * 32;
@@ -208,7 +221,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   load_x(xr[0], 0);
   store_x(xr[0], 0);
 #pragma unroll
-  for (int p = 1; p <= kXDepth; ++p) load_x(xr[p % kXDepth], min(p, s.steps - 1));
+  for (int p = 1; p <= kXDepth; ++p) load_x(xr[p % kXDepth], min(p, steps - 1));
   block_sync_lds();
 
   for (int t0 = 0; t0 < total; t0 += kXDepth) {
@@ -216,8 +229,8 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     for (int d = 0; d < kXDepth; ++d) {
       const int step = t0 + d;
       store_x(xr[(d + 1) % kXDepth], (step + 1) & 1);
-      load_x(xr[(d + 1) % kXDepth], min(step + 1 + kXDepth, s.steps - 1));
-      if (wave_active && step < s.steps) mma(step);
+      load_x(xr[(d + 1) % kXDepth], min(step + 1 + kXDepth, steps - 1));
+      if (wave_active && step < steps) mma(step);
       block_sync_lds();
     }
   }
@@ -229,16 +242,45 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     const int n = n0 + t * 32 + c;
     if (n >= s.N) continue;
     const float bv = s.bias ? s.bias[n] : 0.f;
+    float* part = s.partials + (size_t)blockIdx.z * s.M * s.N;
 #pragma unroll
     for (int mt = 0; mt < MW; ++mt) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int m = m0 + wrow0 + mt * 32 + 8 * (i / 4) + 4 * h + (i % 4);
-        if (m < s.M) store_from_f32<ACT>(s.y, (int64_t)m * s.ldy + n, acc[mt][t][i] + bv);
+        if (m >= s.M) continue;
+        if (s.splits > 1) part[(size_t)m * s.N + n] = acc[mt][t][i];
+        else store_from_f32<ACT>(s.y, (int64_t)m * s.ldy + n, acc[mt][t][i] + bv);
       }
     }
   }
 }
+
+// y[m][n] = round(sum over the splits of partials[z][m][n] + bias[n]); four columns per thread.
+template <int ACT>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float* __restrict__ partials, int splits, int M, int N,
+                     const float* __restrict__ bias, void* __restrict__ y, int64_t ldy) {
+  const int64_t quads_per_row = (N + 3) / 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= quads_per_row * M) return;
+  const int m = (int)(i / quads_per_row);
+  const int n = (int)(i - (int64_t)m * quads_per_row) * 4;
+  float sum[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < splits; ++z) {
+    const float* p = partials + ((size_t)z * M + m) * N + n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n + j < N) sum[j] += p[j];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (n + j < N) store_from_f32<ACT>(y, (int64_t)m * ldy + n + j, sum[j] + (bias ? bias[n + j] : 0.f));
+}
+
+// Number of K splits for a tile GEMM of this shape: 1 while the (column block, row block) grid
+// covers most compute units, else as many as fill them, each at least 8 macro-steps long.
+int plan_tile_splits(int M, int N, int chunks, int mw);
 
 // Rows per block: 128*MW with MW = ceil(M / 128) capped at 3, so that M <= 384
 // is one row block and every weight element is decoded exactly once.
@@ -249,7 +291,7 @@ template <int ACT, class Provider, int MW>
 int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs, hipStream_t st,
                         const char* what) {
   constexpr int BM = 128 * MW;
-  const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM);
+  const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
   const int lds = 2 * BM * kRowBytes + 2 * kWBufBytes;
   static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
   if (!attr_set) {
@@ -261,14 +303,27 @@ int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs
     attr_set = true;
   }
   tile_gemm_kernel<ACT, Provider, MW><<<grid, 512, lds, st>>>(s, pargs);
+  if (s.splits > 1) {
+    const int64_t quads = (int64_t)s.M * ((s.N + 3) / 4);
+    splitk_reduce_kernel<ACT><<<(unsigned)((quads + 255) / 256), 256, 0, st>>>(s.partials, s.splits, s.M, s.N,
+                                                                             s.bias, s.y, s.ldy);
+  }
   return check_launch(what);
 }
 
+// `workspace` (f32, may be null) decides whether K may be split: it must hold splits * M * N floats.
 template <int ACT, class Provider>
 int launch_tile_gemm(GemmShape s, const typename Provider::Args& pargs, hipStream_t st,
-                     const char* what) {
+                     const char* what, void* workspace = nullptr, int64_t workspace_bytes = 0) {
   s.steps = s.chunks;
-  switch (plan_tile_mw(s.M)) {
+  const int mw = plan_tile_mw(s.M);
+  int splits = workspace ? plan_tile_splits(s.M, s.N, s.chunks, mw) : 1;
+  while (splits > 1 && (int64_t)splits * s.M * s.N * 4 > workspace_bytes) --splits;
+  s.splits = splits;
+  s.split_chunks = (s.chunks + splits - 1) / splits;
+  s.splits = (s.chunks + s.split_chunks - 1) / s.split_chunks;  // no empty split
+  s.partials = (float*)workspace;
+  switch (mw) {
     case 1: return launch_tile_gemm_mw<ACT, Provider, 1>(s, pargs, st, what);
     case 2: return launch_tile_gemm_mw<ACT, Provider, 2>(s, pargs, st, what);
     default: return launch_tile_gemm_mw<ACT, Provider, 3>(s, pargs, st, what);

@@ -254,6 +254,8 @@ struct QCall {
   int M, N, K, nbits, gs, act;
   hipStream_t st;
   const char* what;
+  void* ws = nullptr;      // tile GEMM only: f32 scratch for split-K partial tiles (may stay null)
+  int64_t ws_bytes = 0;
 };
 
 static int log2i(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
@@ -339,7 +341,7 @@ static int q_dispatch(const QCall& c, bool gemv) {
       return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
     }
     GemmShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, c.K / 64, 0};
-    return launch_tile_gemm<ACT, P>(s, a, c.st, c.what);
+    return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
   }
   const QElem e{c.w_pack, (const uint16_t*)c.scale, (const uint16_t*)c.zp, c.K, c.nbits, c.gs, c.act};
   if (gemv) return launch_generic_gemv<ACT>(c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, e, c.st, c.what);
@@ -414,8 +416,11 @@ extern "C" int npamd_q_gemv(const void* x, int64_t ldx, const uint8_t* w_pack, c
 extern "C" int npamd_q_gemm_tile(const void* x, int64_t ldx, const uint8_t* w_pack,
                                  const void* scale_f16, const void* zero_point_f16, const float* bias,
                                  void* y, int64_t ldy, int M, int N, int K, int nbits, int group_size,
-                                 int act_dtype, void* stream) {
-  const QCall c{x, ldx, w_pack, scale_f16, zero_point_f16, bias, y, ldy, M, N, K, nbits, group_size,
-                act_dtype, (hipStream_t)stream, "npamd_q_gemm_tile"};
+                                 int act_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+  QCall c{x, ldx, w_pack, scale_f16, zero_point_f16, bias, y, ldy, M, N, K, nbits, group_size,
+          act_dtype, (hipStream_t)stream, "npamd_q_gemm_tile"};
+  NPAMD_REQUIRE(workspace == nullptr || ptr_aligned(workspace, 16), "npamd_q_gemm_tile: workspace must be 16-byte aligned");
+  c.ws = workspace;
+  c.ws_bytes = workspace_bytes;
   return q_run(c, false);
 }

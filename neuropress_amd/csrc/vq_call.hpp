@@ -17,6 +17,8 @@ struct VqCall {
   int M, N, K, act;
   hipStream_t st;
   const char* what;
+  void* ws = nullptr;      // tile GEMM only: f32 scratch for split-K partial tiles (may stay null)
+  int64_t ws_bytes = 0;
 };
 
 inline bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

@@ -12,12 +12,12 @@ int run_vq(const VqCall& c, const GemmShape& s) {
     if (c.cb_dtype == NPAMD_F16) {
       using P = VqProvider<ACT, BITS, true>;
       typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-      return launch_tile_gemm<ACT, P>(s, a, c.st, c.what);
+      return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
     }
   }
   using P = VqProvider<ACT, BITS, false>;
   typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what);
+  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
 template <int ACT>
@@ -36,7 +36,7 @@ int run_rvq(const VqCall& c, const GemmShape& s) {
   typename P::Args a{c.packed, c.packed_r, (const u32x4*)c.cb, (const u32x4*)c.cb_r,
                      (const uint16_t*)c.row_scale, (const uint16_t*)c.row_bias,
                      (uint32_t)c.nc - 1u, (uint32_t)c.nc_r - 1u, s.chunks};
-  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what);
+  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
 template <int ACT>
@@ -57,6 +57,7 @@ int run(const VqCall& c) {
   const int rc = validate(c, 0);
   if (rc < 0) return rc;
   if (rc == 1) return NPAMD_OK;
+  NPAMD_REQUIRE(c.ws == nullptr || (aligned(c.ws, 16) && c.ws_bytes >= 0), "%s: workspace must be 16-byte aligned", c.what);
   return c.act == NPAMD_BF16 ? dispatch<NPAMD_BF16>(c) : dispatch<NPAMD_F16>(c);
 }
 
@@ -65,10 +66,12 @@ int run(const VqCall& c) {
 extern "C" int npamd_vq_gemm_tile(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_bytes,
                              int bits, const void* codebook, int codebook_dtype, int nc, int vl,
                              const float* bias, void* y, int64_t ldy, int M, int N, int K,
-                             int act_dtype, void* stream) {
+                             int act_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   VqCall c{x, ldx, packed, n_bytes, bits, codebook, codebook_dtype, nc, vl,
                nullptr, 0, 0, nullptr, 0, nullptr, nullptr,
                bias, y, ldy, M, N, K, act_dtype, (hipStream_t)stream, "npamd_vq_gemm_tile"};
+  c.ws = workspace;
+  c.ws_bytes = workspace_bytes;
   return run(c);
 }
 
@@ -78,10 +81,12 @@ extern "C" int npamd_rvq_gemm_tile(const void* x, int64_t ldx,
                               const void* cb_main_f16, int nc_main, const void* cb_res_f16, int nc_res,
                               const void* row_scale_f16, const void* row_bias_f16, int vl,
                               const float* bias, void* y, int64_t ldy, int M, int N, int K,
-                              int act_dtype, void* stream) {
+                              int act_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   if (!packed_res) return fail(NPAMD_ERR_INVALID, "npamd_rvq_gemm_tile: residual stream is null");
   VqCall c{x, ldx, packed_main, n_bytes_main, bits_main, cb_main_f16, NPAMD_F16, nc_main, vl,
                packed_res, n_bytes_res, bits_res, cb_res_f16, nc_res, row_scale_f16, row_bias_f16,
                bias, y, ldy, M, N, K, act_dtype, (hipStream_t)stream, "npamd_rvq_gemm_tile"};
+  c.ws = workspace;
+  c.ws_bytes = workspace_bytes;
   return run(c);
 }

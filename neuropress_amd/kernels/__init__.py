@@ -84,6 +84,19 @@ def _x2d(x: torch.Tensor, what: str) -> torch.Tensor:
     return x
 
 
+def _tile_workspace(entry: str, m: int, n: int, k: int, device) -> tuple[int | None, int]:
+    """Scratch for the tile GEMM's split-K (layers with few output features); (None, 0) for the
+    other entry points and for shapes the library does not split.  Allocated per call from
+    torch's caching allocator, so it is stream-ordered and capturable like the output."""
+    if not entry.endswith("_gemm_tile"):
+        return None, 0
+    need = int(_lib.load().npamd_gemm_tile_workspace_bytes(int(m), int(n), int(k)))
+    if need <= 0:
+        return None, 0
+    ws = torch.empty(need // 4, device=device, dtype=torch.float32)
+    return ws, need
+
+
 # ---------------------------------------------------------------------------
 # VQ
 # ---------------------------------------------------------------------------
@@ -181,10 +194,12 @@ def _vq_fused(
         out_features = total // groups
     y = torch.empty((m, out_features), device=x.device, dtype=x.dtype)
     b32 = _bias_f32(bias)
+    ws, ws_bytes = _tile_workspace(entry, m, out_features, k, x.device)
+    extra = (_ptr(ws), ws_bytes) if entry.endswith("_gemm_tile") else ()
     _lib.call(
         entry, x.data_ptr(), x.stride(0), packed.data_ptr(), packed.numel(), int(bits),
         cb.data_ptr(), _DT[cb.dtype], cb.shape[0], vl, _ptr(b32), y.data_ptr(), y.stride(0),
-        m, out_features, k, _DT[x.dtype], _stream(x),
+        m, out_features, k, _DT[x.dtype], *extra, _stream(x),
     )  # fmt: skip
     return y
 
@@ -439,12 +454,15 @@ def rvq_linear(
         tile = m > _lib.GEMV_MAX_M
     y = torch.empty((m, out_features), device=x.device, dtype=x.dtype)
     b32 = _bias_f32(bias)
+    entry = "npamd_rvq_gemm_tile" if tile else "npamd_rvq_gemv"
+    ws, ws_bytes = _tile_workspace(entry, m, out_features, k, x.device)
+    extra = (_ptr(ws), ws_bytes) if tile else ()
     _lib.call(
-        "npamd_rvq_gemm_tile" if tile else "npamd_rvq_gemv",
+        entry,
         x.data_ptr(), x.stride(0), pm.data_ptr(), pm.numel(), int(bits_main), pr.data_ptr(),
         pr.numel(), int(bits_res), cm.data_ptr(), cm.shape[0], cr.data_ptr(), cr.shape[0],
         _ptr(sc), _ptr(rb), cm.shape[1], _ptr(b32), y.data_ptr(), y.stride(0), m, out_features, k,
-        _DT[x.dtype], _stream(x),
+        _DT[x.dtype], *extra, _stream(x),
     )  # fmt: skip
     return y
 
@@ -508,9 +526,11 @@ def _q_fused(entry, x, w_pack, scale, nbits, group_size, zero_point, bias):
     m = x2.shape[0]
     y = torch.empty((m, n), device=x.device, dtype=x.dtype)
     b32 = _bias_f32(bias)
+    ws, ws_bytes = _tile_workspace(entry, m, n, k, x.device)
+    extra = (_ptr(ws), ws_bytes) if entry.endswith("_gemm_tile") else ()
     _lib.call(entry, x2.data_ptr(), x2.stride(0), wp.data_ptr(), sc.data_ptr(), _ptr(zp), _ptr(b32),
               y.data_ptr(), y.stride(0), m, n, k, int(nbits), int(group_size), _DT[x.dtype],
-              _stream(x))  # fmt: skip
+              *extra, _stream(x))  # fmt: skip
     return y.reshape(*lead, n)
 
 

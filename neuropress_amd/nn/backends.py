@@ -106,3 +106,19 @@ class Backend(_StrEnum):
     CUDA_ZERO_ESCAPE = "cuda_zero_escape"
     GEMLITE = "gemlite"
     AUTO = "auto"
+
+
+def tile_band_ok(
+    m: int, n: int, k: int, cus: int, min_fraction: float, split_max_tokens: int, long_k: int
+) -> bool:
+    """Whether the tile-decode GEMM has enough workgroups for ``m`` tokens on an
+    ``n x k`` layer.  Mirrors the kernel's own plan: without a split when the
+    (64 columns x up to 384 rows) grid covers ``min_fraction`` of ``cus`` compute
+    units; otherwise up to 16 reduction splits of at least 512 input features."""
+    blocks = -(-n // 64) * -(-m // 384)
+    if blocks >= min_fraction * cus:
+        return True
+    splits = max(1, min(cus // blocks, k // 512, 16))
+    if splits * blocks < min_fraction * cus:
+        return False
+    return m <= split_max_tokens or k >= long_k

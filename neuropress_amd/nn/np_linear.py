@@ -29,7 +29,7 @@ import torch.nn.functional as F
 
 from ..qweights import ScalarQScheme, ScalarQWeight, is_scalar_qweight
 from ..t2n.packing import BitPacking
-from .backends import Backend, LinearBackend, is_hip_backend_available
+from .backends import Backend, LinearBackend, is_hip_backend_available, tile_band_ok
 
 log = logging.getLogger(__name__)
 
@@ -37,8 +37,14 @@ log = logging.getLogger(__name__)
 # Measured on one MI355X (14336 x 4096, group 32): fused GEMM 38-42 us up to 128
 # tokens and 72 us at 256 against 56-62 / 78 us for decode + GEMM; 104 vs 84 us at 384.
 _Q_TILE_MAX_TOKENS: int = int(os.environ.get("NEUROPRESS_Q_TILE_MAX_TOKENS", "256"))
-# As for the VQ path: narrow layers leave most compute units idle in the fused GEMM.
+# As for the VQ path: the fused GEMM splits the reduction when the layer has few
+# output features; a layer that still leaves most compute units idle takes decode +
+# GEMM.  Measured (fused vs decode + GEMM): 4096 x 14336 39-46 vs 58-93 us up to 128
+# tokens, 75 vs 91 us at 256; 4096 x 4096 20-25 vs 32-41 us up to 128, 36 vs 37 us
+# at 256; 1024 x 4096 (not enough workgroups even when split) 17-19 vs 16-20 us.
 _Q_TILE_MIN_GRID_FRACTION: float = 0.7
+_Q_TILE_SPLIT_MAX_TOKENS: int = 128
+_Q_TILE_SPLIT_LONG_K: int = 8192
 _Q_FUSED_MAX_TOKENS: int = 16
 
 _ALLOW_FALLBACK: bool = os.environ.get("NEUROPRESS_ALLOW_KERNEL_FALLBACK", "").strip() in (
@@ -267,8 +273,10 @@ class NPLinear(nn.Module):
         if cus is None:
             cus = torch.cuda.get_device_properties(x.device).multi_processor_count
             self._derived["cus"] = cus
-        blocks = -(-self.out_features // 64) * -(-m // 384)
-        return blocks >= _Q_TILE_MIN_GRID_FRACTION * cus
+        return tile_band_ok(
+            m, self.out_features, self.in_features, cus,
+            _Q_TILE_MIN_GRID_FRACTION, _Q_TILE_SPLIT_MAX_TOKENS, _Q_TILE_SPLIT_LONG_K,
+        )  # fmt: skip
 
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:
         """HIP path by token count; takes the place of np_linear.py:731-761."""

@@ -37,7 +37,7 @@ import torch.nn.functional as F
 
 from ..qweights import VQScheme, VQWeight, is_vq_weight
 from ..transforms.vq_packing import IndexPacking
-from .backends import Backend, VQBackend, is_hip_backend_available
+from .backends import Backend, VQBackend, is_hip_backend_available, tile_band_ok
 
 log = logging.getLogger(__name__)
 
@@ -81,10 +81,18 @@ _TILE_MAX_TOKENS: int = _env_int(
     ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 256
 )
 
-# The tile GEMM gives each workgroup 64 output columns (and up to 384 rows), so a
-# layer with few output features leaves most of the GPU idle; below this fraction
-# of the compute units the decode + GEMM band is used instead.
+# The tile GEMM gives each workgroup 64 output columns (and up to 384 rows).  When
+# that grid covers less than this fraction of the compute units the kernel splits
+# the reduction over up to 16 workgroups per tile (at least 512 input features
+# each); a layer that still cannot cover the fraction takes decode + GEMM.
 _TILE_MIN_GRID_FRACTION: float = 0.7
+
+# Upper end of the band for layers that need the split.  Measured on one MI355X,
+# tile GEMM vs decode + GEMM: 4096 x 14336 layer 51-60 vs 75-113 us up to 128
+# tokens and 82 vs 101 us at 256; 4096 x 4096 layer 25-31 vs 30-39 us up to 128
+# tokens, 39 vs 36 us at 256.
+_TILE_SPLIT_MAX_TOKENS: int = 128
+_TILE_SPLIT_LONG_K: int = 8192  # from this many input features on, _TILE_MAX_TOKENS applies
 
 # Opt-in: when a HIP kernel call fails, warn once and run torch ops instead (the
 # reference's behaviour).  Off by default so a missing or broken kernel library
@@ -476,7 +484,7 @@ class NPVQLinear(nn.Module):
                 if (
                     self.backend != VQBackend.CUDA_LUT
                     and m <= _TILE_MAX_TOKENS
-                    and self._tile_grid_fills_gpu(x, m)
+                    and self._tile_band_ok(x, m)
                 ):
                     return self._forward_tile_gemm(x)
                 return self._forward_dequant_gemm(x)
@@ -552,17 +560,20 @@ class NPVQLinear(nn.Module):
             return self._forward_dequant_gemm(x)
         return y.reshape(*leading, self.out_features)
 
-    def _tile_grid_fills_gpu(self, x: torch.Tensor, m: int) -> bool:
-        """True when the tile GEMM's grid (64 columns x up to 384 rows per workgroup)
-        covers at least ``_TILE_MIN_GRID_FRACTION`` of the device's compute units."""
+    def _tile_band_ok(self, x: torch.Tensor, m: int) -> bool:
+        """True when the tile GEMM's grid (64 columns x up to 384 rows per workgroup,
+        times the reduction splits the kernel adds for layers with few output
+        features) covers at least ``_TILE_MIN_GRID_FRACTION`` of the compute units."""
         if not x.is_cuda:
             return True
         cus = self._derived.get("cus")
         if cus is None:
             cus = torch.cuda.get_device_properties(x.device).multi_processor_count
             self._derived["cus"] = cus
-        blocks = -(-self.out_features // 64) * -(-m // 384)
-        return blocks >= _TILE_MIN_GRID_FRACTION * cus
+        return tile_band_ok(
+            m, self.out_features, self.in_features, cus,
+            _TILE_MIN_GRID_FRACTION, _TILE_SPLIT_MAX_TOKENS, _TILE_SPLIT_LONG_K,
+        )  # fmt: skip
 
     # -- torch-op paths ---------------------------------------------------
 

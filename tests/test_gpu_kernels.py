@@ -322,3 +322,35 @@ def test_strided_x_and_stream(gpu, oracle_lib):
         y = kernels.vq_linear(xbig[:, :256], L["packed"].to(gpu), L["cb"].to(gpu), 8, 8, None, 48)
     s.synchronize()
     _check(y, _vq_ref(oracle_lib, L, torch.float16))
+
+
+# ------------------------------------------------------------------ split-K ---
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [17, 130, 400])
+@pytest.mark.parametrize("k", [1024, 2048 + 64])
+def test_vq_gemm_tile_split_k(gpu, oracle_lib, act, m, k):
+    """Few output columns and a long K: the tile GEMM splits K over blockIdx.z and adds the
+    f32 partial tiles in a second kernel (K not a multiple of the split length included)."""
+    from neuropress_amd import _lib, kernels
+
+    n = 200
+    assert _lib.load().npamd_gemm_tile_workspace_bytes(m, n, k) >= 2 * m * n * 4
+    L = cases.vq_layer(800 + m + k, n, k, 65536, bits=16, act=act, m=m, bias=True, std=0.05)
+    y = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), 16, n, L["bias"].to(gpu))
+    assert y.shape == (m, n) and y.dtype == act
+    _check(y, _vq_ref(oracle_lib, L, act))
+
+
+@pytest.mark.parametrize("m", [40, 300])
+def test_q4_and_rvq_gemm_tile_split_k(gpu, oracle_lib, m):
+    from neuropress_amd import kernels
+
+    Q = cases.q4_layer(820 + m, 136, 2048, gs=32, act=torch.float16, m=m, bias=True)
+    y = kernels.q_gemm_tile(Q["x"].to(gpu), Q["blob"].to(gpu), Q["scale"].to(gpu), 4, 32, None, Q["bias"].to(gpu))
+    _check(y, _q_ref(oracle_lib, Q, torch.float16))
+    R = cases.rvq_layer(830 + m, 80, 1024, act=torch.float16, m=m)
+    y = kernels.rvq_linear(R["x"].to(gpu), R["pm"].to(gpu), R["bm"], R["pr"].to(gpu), R["br"], R["cbm"].to(gpu),
+                           R["cbr"].to(gpu), R["scale"].to(gpu), R["wbias"].to(gpu), 80, None, tile=True)
+    _check(y, _rvq_ref(oracle_lib, R, torch.float16))

@@ -353,3 +353,20 @@ def test_c_abi_validates_arguments_without_a_gpu():
     with pytest.raises(RuntimeError, match="exceeds the fused limit"):
         _lib.call("npamd_vq_gemv", None, 64, None, 1 << 20, 8, None, 0, 16, 8, None, None, 4, 17, 4, 64, 0, None)
     _lib.call("npamd_vq_dequant", None, 0, 8, None, 16, 8, 0, None, 0, None)  # empty: success, no launch
+
+
+def test_tile_band_rule_counts_reduction_splits():
+    """Layers with few output features take the tile band only while the kernel's
+    reduction split can fill the compute units (256 here) and, for short
+    reductions, only up to the split band's token limit."""
+    from neuropress_amd.nn.backends import tile_band_ok
+
+    def ok(m, n, k):
+        return tile_band_ok(m, n, k, 256, 0.7, 128, 8192)
+
+    assert ok(64, 14336, 4096) and ok(256, 14336, 4096)  # grid fills the GPU by itself
+    assert ok(64, 4096, 14336) and ok(256, 4096, 14336)  # 64 tiles x 4 splits, long reduction
+    assert ok(128, 4096, 4096) and not ok(129, 4096, 4096)  # short reduction: up to 128 tokens
+    assert not ok(17, 1024, 4096)  # 16 tiles x 8 splits = half the compute units
+    assert not ok(17, 4096, 512)  # no split possible below 1024 input features
+    assert ok(17, 2048, 4096)  # 32 tiles x 8 splits
