@@ -345,6 +345,16 @@ def main():
                 t = time_graph(lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_),
                                rot, steps_s * 2, 3, dev)
                 add(name, "a:gemv", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
+                if m == 1 and bits == 12:
+                    # the same call with a column permutation: gathered inside the GEMV, or by torch in front of it
+                    perm = torch.randperm(kk, generator=gen(90)).to(dev)
+                    p32 = perm.to(torch.int32)
+                    t = time_graph(lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_,
+                                                               column_perm=p32), rot, steps_s * 2, 3, dev)
+                    add(name + " column_perm", "a:gemv, gather fused", m, t, vq_alg_bytes(cc, m) + kk * 4, 2.0 * m * nn_ * kk)
+                    t = time_graph(lambda i: kernels.vq_linear(xm[i % 2][:, perm], cc["pool"][i], cc["d_cb"], bits, 8, None,
+                                                               nn_), rot, steps_s * 2, 3, dev)
+                    add(name + " column_perm", "a:torch gather + gemv", m, t, vq_alg_bytes(cc, m) + kk * 8, 2.0 * m * nn_ * kk)
             del cc
             torch.cuda.empty_cache()
         # config 4: residual VQ (65536 + 256 entry codebooks, Zipf(1.1) indices, per-row scale / bias), fp16

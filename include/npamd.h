@@ -73,6 +73,27 @@ int npamd_vq_gemv(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_b
                   int act_dtype, void* stream);
 
 /*
+ * The same GEMV with the reference's column permutation folded in:
+ *   y[m, n] = sum_k x[m, column_perm[k]] * W[n, k] (+ bias[n]),
+ * i.e. vq_linear applied to x[..., column_perm] (neuropress/nn/np_vq_linear.py:1027-1028)
+ * without the separate gather kernel.  column_perm: K int32 column numbers, each < K,
+ * 16-byte aligned.  Every workgroup copies the M rows of x into LDS and permutes them there,
+ * so this entry point takes M * K <= 16384 elements, VL = 8, 4/8/12/16-bit indices and
+ * K % 64 == 0 only;
+ * other requests return NPAMD_ERR_UNSUPPORTED (gather x yourself and call npamd_vq_gemv).
+ */
+int npamd_vq_gemv_perm(const void* x, int64_t ldx, const int32_t* column_perm,
+                       const uint8_t* packed, int64_t n_bytes, int bits,
+                       const void* codebook, int codebook_dtype, int nc, int vl,
+                       const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                       int act_dtype, void* stream);
+
+/* 1 when npamd_vq_gemv_perm takes this shape AND its LDS copies of x do not cost the kernel
+ * workgroups per compute unit (then it beats a separate gather by about 2.5 us per call);
+ * 0 otherwise: gather x yourself and call npamd_vq_gemv.  Host-only arithmetic. */
+int npamd_vq_gemv_perm_supported(int M, int N, int K, int nc, int vl, int bits);
+
+/*
  * Tile-decode MFMA GEMM, any M >= 1: same contraction, weight tiles decoded
  * inside the kernel, dense weight never written.
  * Replaces vq_gemm_triton (neuropress/kernels/vq_triton.py:119-179) and the

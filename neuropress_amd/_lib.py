@@ -31,6 +31,8 @@ _Q_LINEAR = [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _
 SIGNATURES: dict[str, list] = {
     "npamd_vq_dequant": [_vp, _i64, _int, _vp, _int, _int, _i64, _vp, _int, _vp],
     "npamd_vq_gemv": _VQ_LINEAR,
+    "npamd_vq_gemv_perm": _VQ_LINEAR[:2] + [_vp] + _VQ_LINEAR[2:],
+    "npamd_vq_gemv_perm_supported": [_int] * 6,
     "npamd_vq_gemm_tile": _VQ_LINEAR[:-1] + _WS + [_vp],
     "npamd_gemm_tile_workspace_bytes": [_int, _int, _int],
     "npamd_vq_widen_u16": [_vp, _i64, _int, _i64, _vp, _vp],

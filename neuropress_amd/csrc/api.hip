@@ -56,6 +56,7 @@ static int device_cu_count() {
 // as soon as the grid starts: jobs per wave is kept near jobs / (16 waves * CUs).
 // NPAMD_GEMV_R / NPAMD_GEMV_SPW override the choice (tuning aid).
 bool gemv_lds_codebook_enabled() { return env_int("NPAMD_GEMV_LDS_CB", 1) != 0; }
+bool gemv_lds_activations_forced() { return env_int("NPAMD_GEMV_LDS_X", 0) != 0; }
 
 GemvPlan plan_gemv(int N, int chunks) {
   const int steps = (chunks + 3) / 4;
@@ -79,6 +80,16 @@ GemvPlan plan_gemv(int N, int chunks) {
   p.steps_per_wave = spw;
   p.waves = (steps + spw - 1) / spw;
   return p;
+}
+
+bool gemv_perm_keeps_occupancy(int M, int N, int chunks, int cb_bytes) {
+  const GemvPlan plan = plan_gemv(N, chunks);
+  const int red = ((plan.waves * M * 16 * plan.R + 3) & ~3) * (int)sizeof(float);
+  const int cbl = (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) ? cb_bytes : 0;
+  const int xb = M * chunks * 64 * 2;
+  const int lds = red + (cbl > xb ? cbl : xb) + xb;
+  const int blocks = (N + 16 * plan.R - 1) / (16 * plan.R);
+  return lds <= 80 * 1024 || (blocks <= device_cu_count() && lds <= 160 * 1024);
 }
 
 int plan_tile_splits(int M, int N, int chunks, int mw) {

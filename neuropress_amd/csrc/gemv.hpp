@@ -29,7 +29,14 @@ struct GemvShape {
   int chunks;          // K / 64 (K % 64 == 0 is a precondition of this kernel)
   int steps;           // ceil(chunks / 4)
   int steps_per_wave;  // steps each wave of the block covers
+  // Optional gather of the activation columns: the kernel contracts x[m, perm[k]] with W[n, k].
+  // Only with the X_LDS variant (every block first copies the permuted rows of x into LDS).
+  const int32_t* perm = nullptr;
 };
+
+// Largest M * K (elements) whose activations the GEMV stages in LDS (32 KiB; the unpermuted
+// copy shares its place with the codebook of up to 64 KiB).
+constexpr int kGemvLdsActivationsMax = 16 * 1024;
 
 // R = 4 keeps 32 gathered operands (128 registers) live per lane, so it is
 // limited to 8 waves per block; R <= 2 fits the 128-register budget of 16 waves.
@@ -39,7 +46,11 @@ constexpr int kGemvMaxWaves = (R >= 4) ? 8 : 16;
 // CB_LDS: the block first copies the whole codebook into LDS and gathers from
 // there (ds_read_b128) instead of from L1/L2.  Pays off when the table is too
 // big for L1 (> 32 KiB) yet fits LDS, or is so small that the copy is free.
-template <int ACT, class Provider, int R, bool CB_LDS>
+// X_LDS: the block also copies x (all M rows, all of K) into LDS, applying the
+// column permutation s.perm on the way when there is one, and reads its A
+// operands from there: the gather x[m, perm[k]] costs K element loads per block
+// instead of a kernel of its own in front of this one.
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS>
 __global__ void __launch_bounds__(kGemvMaxWaves<R> * 64)
 fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][M][16*R] (+ codebook copy)
@@ -47,15 +58,57 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int n_waves = blockDim.x >> 6;
+  // LDS after the reduction buffer (16-byte aligned): the codebook copy, then the copy of x.
+  // While x is being permuted its unpermuted copy lies where the codebook goes afterwards, so
+  // the region in front of x is max(codebook, x) bytes.
+  const int red_floats = (n_waves * s.M * 16 * R + 3) & ~3;
+  uint8_t* const lds0 = reinterpret_cast<uint8_t*>(red) + red_floats * (int)sizeof(float);
+  int cb_lds_bytes = 0;
+  if constexpr (CB_LDS) cb_lds_bytes = prov.codebook_rows() * 16;
+  const uint16_t* x_lds = nullptr;
+  if constexpr (X_LDS) {
+    // Rows of x: a coalesced copy into LDS, then (with a permutation) a second LDS buffer filled
+    // by 2-byte LDS reads at the permuted columns -- element gathers are an order of magnitude
+    // cheaper from LDS than through the vector memory path, and every block needs all of them.
+    const int K = s.chunks * 64;
+    const int k8s = s.chunks * 8;  // 8-element pieces per row
+    const int items = s.M * k8s;
+    const int x_bytes = s.M * K * 2;
+    uint16_t* const xs = reinterpret_cast<uint16_t*>(lds0 + (s.perm ? max(cb_lds_bytes, x_bytes) : cb_lds_bytes));
+    uint16_t* const xraw = s.perm ? reinterpret_cast<uint16_t*>(lds0) : xs;
+    const uint16_t* xg = reinterpret_cast<const uint16_t*>(s.x);
+    for (int i = threadIdx.x; i < items; i += blockDim.x) {
+      const int m = i / k8s;
+      const int k8 = i - m * k8s;
+      *reinterpret_cast<u32x4*>(xraw + (int64_t)i * 8) =
+          *reinterpret_cast<const u32x4*>(xg + (int64_t)m * s.ldx + k8 * 8);
+    }
+    if (s.perm) {
+      __syncthreads();
+      for (int i = threadIdx.x; i < items; i += blockDim.x) {
+        const int m = i / k8s;
+        const int k8 = i - m * k8s;
+        const uint16_t* xr = xraw + (int64_t)m * K;
+        const u32x4 p0 = *reinterpret_cast<const u32x4*>(s.perm + k8 * 8);
+        const u32x4 p1 = *reinterpret_cast<const u32x4*>(s.perm + k8 * 8 + 4);
+        u32x4 v;
+        v.x = (uint32_t)xr[p0.x] | ((uint32_t)xr[p0.y] << 16);
+        v.y = (uint32_t)xr[p0.z] | ((uint32_t)xr[p0.w] << 16);
+        v.z = (uint32_t)xr[p1.x] | ((uint32_t)xr[p1.y] << 16);
+        v.w = (uint32_t)xr[p1.z] | ((uint32_t)xr[p1.w] << 16);
+        *reinterpret_cast<u32x4*>(xs + (int64_t)i * 8) = v;
+      }
+      if constexpr (CB_LDS) __syncthreads();  // the codebook overwrites the unpermuted copy
+    }
+    x_lds = xs;
+  }
   if constexpr (CB_LDS) {
-    // codebook copy lives after the reduction buffer, 16-byte aligned
-    const int red_floats = (n_waves * s.M * 16 * R + 3) & ~3;
-    u32x4* cb_lds = reinterpret_cast<u32x4*>(red + red_floats);
+    u32x4* cb_lds = reinterpret_cast<u32x4*>(lds0);
     const u32x4* src = prov.global_codebook();
     for (int i = threadIdx.x; i < prov.codebook_rows(); i += blockDim.x) cb_lds[i] = src[i];
-    __syncthreads();
     prov.use_codebook(cb_lds);
   }
+  if constexpr (CB_LDS || X_LDS) __syncthreads();
   const int c = lane & 15;
   const int q = lane >> 4;
   const int row0 = blockIdx.x * (16 * R);
@@ -70,7 +123,8 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   // their operand is zeroed afterwards, so all gathers of a step are in flight
   // together instead of each sitting behind its own branch and wait.
   const int x_row = min(c, s.M - 1);
-  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(s.x) + (int64_t)x_row * s.ldx;
+  const uint16_t* xrow = X_LDS ? x_lds + (int64_t)x_row * (s.chunks * 64)
+                               : reinterpret_cast<const uint16_t*>(s.x) + (int64_t)x_row * s.ldx;
   const bool x_lane = c < s.M;
   const u32x4 zero4{0, 0, 0, 0};
 
@@ -155,28 +209,37 @@ GemvPlan plan_gemv(int N, int chunks);
 // Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
+bool gemv_lds_activations_forced();  // NPAMD_GEMV_LDS_X=1: stage x in LDS also without a permutation (tuning aid)
 
-template <int ACT, class Provider, int R, bool CB_LDS>
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false>
 int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const GemvPlan& plan,
                         int cb_bytes, hipStream_t st, const char* what) {
   s.steps_per_wave = plan.steps_per_wave;
   const int blocks = (s.N + 16 * R - 1) / (16 * R);
   const int red_floats = (plan.waves * s.M * 16 * R + 3) & ~3;
-  const int lds = red_floats * (int)sizeof(float) + (CB_LDS ? cb_bytes : 0);
+  const int x_bytes = X_LDS ? s.M * s.chunks * 64 * 2 : 0;
+  const int cb_lds_bytes = CB_LDS ? cb_bytes : 0;
+  const int lds = red_floats * (int)sizeof(float) + x_bytes +
+                  ((X_LDS && s.perm) ? (cb_lds_bytes > x_bytes ? cb_lds_bytes : x_bytes) : cb_lds_bytes);
   if (lds > 64 * 1024) {
     static int reserved = 0;  // per instantiation: largest dynamic-LDS size enabled so far
     if (lds > reserved) {
       const hipError_t e = hipFuncSetAttribute(
-          reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS>),
+          reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS>),
           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
       if (e != hipSuccess)
         return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
       reserved = lds;
     }
   }
-  fused_gemv_kernel<ACT, Provider, R, CB_LDS><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
+  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);
 }
+
+// Whether the LDS copies of x leave the kernel's occupancy alone: two blocks per compute unit
+// (80 KiB each) while the grid has more blocks than compute units, else one (160 KiB).  Measured
+// on a 8192 x 2048 layer with a 64 KiB codebook: 4.8 us up to 76.5 KiB per block, 6.9 us at 80.5.
+bool gemv_perm_keeps_occupancy(int M, int N, int chunks, int cb_bytes);
 
 // cb_bytes: size of the (single) codebook for providers that can stage it in LDS, else 0.
 template <int ACT, class Provider>
@@ -185,6 +248,17 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
   s.steps = (s.chunks + 3) / 4;
   const GemvPlan plan = plan_gemv(s.N, s.chunks);
   if constexpr (Provider::kLdsCodebook) {
+    const bool x_fits = (int64_t)s.M * s.chunks * 64 <= kGemvLdsActivationsMax;
+    if (s.perm || (x_fits && gemv_lds_activations_forced())) {  // with a permutation the caller has checked the size
+      if (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) {
+        if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true, true>(s, pargs, plan, cb_bytes, st, what);
+        if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true, true>(s, pargs, plan, cb_bytes, st, what);
+        return launch_fused_gemv_r<ACT, Provider, 1, true, true>(s, pargs, plan, cb_bytes, st, what);
+      }
+      if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, false, true>(s, pargs, plan, 0, st, what);
+      if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, false, true>(s, pargs, plan, 0, st, what);
+      return launch_fused_gemv_r<ACT, Provider, 1, false, true>(s, pargs, plan, 0, st, what);
+    }
     if (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) {
       if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true>(s, pargs, plan, cb_bytes, st, what);
       if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true>(s, pargs, plan, cb_bytes, st, what);

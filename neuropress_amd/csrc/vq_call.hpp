@@ -19,6 +19,7 @@ struct VqCall {
   const char* what;
   void* ws = nullptr;      // tile GEMM only: f32 scratch for split-K partial tiles (may stay null)
   int64_t ws_bytes = 0;
+  const int32_t* perm = nullptr;  // fused GEMV only: contract x[m, perm[k]] with W[n, k]
 };
 
 inline bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

@@ -41,6 +41,14 @@ int run_rvq(const VqCall& c, const GemvShape& s) {
 template <int ACT>
 int dispatch(const VqCall& c) {
   GemvShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K / 64, 0, 0};
+  if (c.perm) {
+    // The gather is done while x is copied to LDS, which only the MFMA kernel for plain VQ does.
+    if (!(fast_ok(c) && !c.packed_r && (int64_t)c.M * c.K <= kGemvLdsActivationsMax && aligned(c.perm, 16)))
+      return fail(NPAMD_ERR_UNSUPPORTED,
+                  "%s: column_perm needs VL = 8, 4/8/12/16-bit indices, K %% 64 == 0, 16-byte aligned "
+                  "buffers and M * K <= %d (got M=%d K=%d)", c.what, kGemvLdsActivationsMax, c.M, c.K);
+    s.perm = c.perm;
+  }
   if (fast_ok(c)) {
     if (!c.packed_r) return run_vq_bits<ACT>(c, s);
     const bool res_ok = aligned(c.packed_r, 16) && aligned(c.cb_r, 16);
@@ -69,6 +77,25 @@ extern "C" int npamd_vq_gemv(const void* x, int64_t ldx, const uint8_t* packed, 
                nullptr, 0, 0, nullptr, 0, nullptr, nullptr,
                bias, y, ldy, M, N, K, act_dtype, (hipStream_t)stream, "npamd_vq_gemv"};
   return run(c);
+}
+
+extern "C" int npamd_vq_gemv_perm(const void* x, int64_t ldx, const int32_t* column_perm,
+                                  const uint8_t* packed, int64_t n_bytes, int bits,
+                                  const void* codebook, int codebook_dtype, int nc, int vl,
+                                  const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                                  int act_dtype, void* stream) {
+  VqCall c{x, ldx, packed, n_bytes, bits, codebook, codebook_dtype, nc, vl,
+               nullptr, 0, 0, nullptr, 0, nullptr, nullptr,
+               bias, y, ldy, M, N, K, act_dtype, (hipStream_t)stream, "npamd_vq_gemv_perm"};
+  c.perm = column_perm;
+  return run(c);
+}
+
+extern "C" int npamd_vq_gemv_perm_supported(int M, int N, int K, int nc, int vl, int bits) {
+  const bool bits_ok = bits == 4 || bits == 8 || bits == 12 || bits == 16;
+  if (!(vl == 8 && bits_ok && K > 0 && K % 64 == 0 && M >= 1 && M <= NPAMD_GEMV_MAX_M && N >= 1 && nc >= 1)) return 0;
+  if ((int64_t)M * K > kGemvLdsActivationsMax) return 0;
+  return gemv_perm_keeps_occupancy(M, N, K / 64, nc * 16) ? 1 : 0;
 }
 
 extern "C" int npamd_rvq_gemv(const void* x, int64_t ldx,

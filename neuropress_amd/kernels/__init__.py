@@ -172,6 +172,7 @@ def _vq_fused(
     bits: int,
     out_features: int | None,
     bias: torch.Tensor | None,
+    column_perm: torch.Tensor | None = None,
 ) -> torch.Tensor:
     _check_device(entry, x, packed_indices, centroids, bias)
     x = _x2d(x, entry)
@@ -196,8 +197,15 @@ def _vq_fused(
     b32 = _bias_f32(bias)
     ws, ws_bytes = _tile_workspace(entry, m, out_features, k, x.device)
     extra = (_ptr(ws), ws_bytes) if entry.endswith("_gemm_tile") else ()
+    perm = ()
+    if column_perm is not None:
+        if column_perm.dtype != torch.int32 or column_perm.numel() != k or not column_perm.is_contiguous():
+            raise RuntimeError(f"{entry}: column_perm must be a contiguous int32 tensor of K={k} entries")
+        if column_perm.device != x.device:
+            raise RuntimeError(f"{entry}: column_perm must live on x's device")
+        perm = (column_perm.data_ptr(),)
     _lib.call(
-        entry, x.data_ptr(), x.stride(0), packed.data_ptr(), packed.numel(), int(bits),
+        entry, x.data_ptr(), x.stride(0), *perm, packed.data_ptr(), packed.numel(), int(bits),
         cb.data_ptr(), _DT[cb.dtype], cb.shape[0], vl, _ptr(b32), y.data_ptr(), y.stride(0),
         m, out_features, k, _DT[x.dtype], *extra, _stream(x),
     )  # fmt: skip
@@ -212,11 +220,28 @@ def vq_linear(
     vector_len: int,
     bias: torch.Tensor | None = None,
     out_features: int | None = None,
+    column_perm: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Fused decode GEMV, ``M <= 16`` (reference: neuropress/kernels/__init__.py:209-245)."""
+    """Fused decode GEMV, ``M <= 16`` (reference: neuropress/kernels/__init__.py:209-245).
+
+    ``column_perm`` (int32 ``[K]``, optional, not in the reference's signature): compute
+    ``vq_linear(x[..., column_perm], ...)`` with the gather done inside the kernel; see
+    :func:`vq_linear_perm_supported` for the shapes that take it.
+    """
     if centroids.dim() == 2 and centroids.shape[1] != vector_len:
         raise RuntimeError("vq_linear: vector_len does not match the codebook")
+    if column_perm is not None:
+        return _vq_fused("npamd_vq_gemv_perm", x, packed_indices, centroids, bits, out_features, bias,
+                         column_perm)  # fmt: skip
     return _vq_fused("npamd_vq_gemv", x, packed_indices, centroids, bits, out_features, bias)
+
+
+def vq_linear_perm_supported(m: int, n: int, k: int, num_centroids: int, vector_len: int, bits: int) -> bool:
+    """Whether :func:`vq_linear` should be given ``column_perm`` for this shape: the kernel takes it
+    (``M * K <= 16384``, VL 8, 4/8/12/16-bit indices, ``K % 64 == 0``) and its LDS copy of x
+    does not reduce the workgroups per compute unit."""
+    return bool(_lib.load().npamd_vq_gemv_perm_supported(int(m), int(n), int(k), int(num_centroids),
+                                                         int(vector_len), int(bits)))  # fmt: skip
 
 
 class SlicedIndices:

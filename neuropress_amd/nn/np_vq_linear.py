@@ -474,6 +474,8 @@ class NPVQLinear(nn.Module):
             m = x.numel() // self.in_features
             if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and self._sliced_ready(x):
                 return self._forward_sliced(x)  # applies column_perm inside the kernel
+            if self.column_perm is not None and self._perm_fusable(x, m):
+                return self._fused(x, tile=False, perm=self._perm_i32(x.device))
         if self.column_perm is not None:
             x = x[..., self.column_perm]
         if self.backend in _FUSED_BACKENDS:
@@ -538,16 +540,32 @@ class NPVQLinear(nn.Module):
             return False  # no host work inside a capture: the fused GEMV runs instead
         return self.prepare_sliced()
 
+    def _perm_i32(self, device: torch.device) -> torch.Tensor:
+        """``column_perm`` as the int32 device tensor the kernels read (cached)."""
+        perm = self._derived.get("perm_i32")
+        if perm is None or perm.device != device:
+            perm = self.column_perm.to(device=device, dtype=torch.int32).contiguous()
+            self._derived["perm_i32"] = perm
+        return perm
+
+    def _perm_fusable(self, x: torch.Tensor, m: int) -> bool:
+        """Whether the fused GEMV gathers ``x[..., column_perm]`` itself for this call."""
+        if not x.is_cuda or self.is_residual or m > min(_fused_max_tokens(self.backend), 16):
+            return False
+        if "perm_i32" not in self._derived and torch.cuda.is_current_stream_capturing():
+            return False  # the int32 copy is made outside a capture
+        from .. import kernels
+
+        bits = self.bits if self.bits in _FAST_BITS else 16
+        return kernels.vq_linear_perm_supported(
+            m, self.out_features, self.in_features, self.proxy.num_centroids, self.vector_len, bits
+        )
+
     def _forward_sliced(self, x: torch.Tensor) -> torch.Tensor:
         from .. import kernels
 
         *leading, _ = x.shape
-        perm = None
-        if self.column_perm is not None:
-            perm = self._derived.get("perm_i32")
-            if perm is None or perm.device != x.device:
-                perm = self.column_perm.to(device=x.device, dtype=torch.int32).contiguous()
-                self._derived["perm_i32"] = perm
+        perm = self._perm_i32(x.device) if self.column_perm is not None else None
         try:
             y = kernels.vq_linear_sliced(
                 x.reshape(-1, self.in_features), self._derived["sliced"],
@@ -679,7 +697,7 @@ class NPVQLinear(nn.Module):
             self._derived["zero_cb"] = z
         return z
 
-    def _fused(self, x: torch.Tensor, tile: bool) -> torch.Tensor:
+    def _fused(self, x: torch.Tensor, tile: bool, perm: torch.Tensor | None = None) -> torch.Tensor:
         from .. import kernels
 
         *leading, _ = x.shape
@@ -697,7 +715,8 @@ class NPVQLinear(nn.Module):
             if tile:
                 y = fn(x2d, stream, cb, bits, self.out_features, self._bias_f32())
             else:
-                y = fn(x2d, stream, cb, bits, self.vector_len, self._bias_f32(), self.out_features)
+                y = fn(x2d, stream, cb, bits, self.vector_len, self._bias_f32(), self.out_features,
+                       column_perm=perm)  # fmt: skip
         return y.reshape(*leading, self.out_features)
 
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:

@@ -134,6 +134,52 @@ def test_vq_gemv_fast_path(gpu, oracle_lib, act, bits, nc, m):
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,nc", [(4, 16), (8, 256), (12, 4096), (16, 65536)])
+@pytest.mark.parametrize("m", [1, 2, 5, 16])
+def test_vq_gemv_column_perm(gpu, oracle_lib, act, bits, nc, m):
+    """npamd_vq_gemv_perm == the plain GEMV fed with x[:, column_perm] (reference:
+    np_vq_linear.py:1027-1028), checked against the oracle on the permuted activations.  x has a
+    row stride larger than K, so a kernel that ignored the permutation or the stride would fail."""
+    from neuropress_amd import kernels
+
+    n, k = 100, 320
+    L = cases.vq_layer(700 + bits + m, n, k, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
+    perm = torch.randperm(k, generator=cases.gen(9 + m))
+    xw = torch.zeros(m, k + 64, dtype=act)
+    xw[:, :k] = L["x"]
+    x_gpu = xw.to(gpu)[:, :k]  # stride k + 64
+    assert kernels.vq_linear_perm_supported(m, n, k, nc, 8, bits)
+    y = kernels.vq_linear(x_gpu, L["packed"].to(gpu), L["cb"].to(gpu), bits, 8, L["bias"].to(gpu),
+                          out_features=n, column_perm=perm.to(torch.int32).to(gpu))
+    assert y.shape == (m, n) and y.dtype == act
+    _check(y, _vq_ref(oracle_lib, dict(L, x=L["x"][:, perm].contiguous()), act))
+    # bit-identical to the unpermuted kernel on pre-gathered activations
+    y2 = kernels.vq_linear(L["x"][:, perm].contiguous().to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 8,
+                           L["bias"].to(gpu), out_features=n)
+    assert torch.equal(y, y2)
+
+
+def test_vq_gemv_column_perm_limits(gpu):
+    """Shapes the permuted GEMV does not take are refused with a message, not computed wrongly."""
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(41, 64, 4096, 256, bits=8, act=torch.float16, m=9)  # 9 * 4096 > 16384 elements
+    perm = torch.randperm(4096, generator=cases.gen(1)).to(torch.int32).to(gpu)
+    assert not kernels.vq_linear_perm_supported(9, 64, 4096, 256, 8, 8)
+    assert kernels.vq_linear_perm_supported(1, 14336, 4096, 4096, 8, 16)  # 73 KiB of LDS: two blocks per CU
+    assert not kernels.vq_linear_perm_supported(2, 14336, 4096, 4096, 8, 16)  # 82 KiB: one block per CU
+    with pytest.raises(RuntimeError, match="column_perm needs"):
+        kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), 8, 8, None, 64, column_perm=perm)
+    with pytest.raises(RuntimeError, match="int32"):
+        kernels.vq_linear(L["x"][:4].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), 8, 8, None, 64,
+                          column_perm=perm.long())
+    y = kernels.vq_linear(L["x"][:4].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), 8, 8, None, 64, column_perm=perm)
+    w = L["cb"][L["idx"]].reshape(64, 4096).float()
+    ref = L["x"][:4][:, perm.cpu().long()].float() @ w.T
+    assert (y.float().cpu() - ref).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 def test_vq_gemv_precast_codebook(gpu, oracle_lib, act):
     from neuropress_amd import kernels
 

@@ -136,6 +136,29 @@ def test_narrow_layers_take_the_split_tile_band(gpu, monkeypatch):
     assert _lib.load().npamd_gemm_tile_workspace_bytes(17, 2048, 4096) > 0  # the split is in use
 
 
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+def test_column_perm_is_folded_into_the_fused_gemv(gpu, act, monkeypatch):
+    """A layer with column_perm and a small codebook: up to 16 tokens (while M * K fits the kernel's
+    LDS copy of x) the fused GEMV gathers the columns itself; more tokens gather with torch first."""
+    from neuropress_amd import kernels
+
+    n, k, nc = 96, 1024, 4096
+    L = cases.vq_layer(81, n, k, nc, bits=12, bias=True, std=0.05)
+    perm = torch.randperm(k, generator=cases.gen(82))
+    layer = NPVQLinear(VQProxy(L["cb"]).to(gpu), L["packed"], 12, n, k, 8, "cuda_wmma", bias=L["bias"].float(),
+                       column_perm=perm).to(gpu)
+    seen = []
+    real = kernels.vq_linear
+    monkeypatch.setattr(kernels, "vq_linear",
+                        lambda *a, **kw: (seen.append(kw.get("column_perm") is not None), real(*a, **kw))[1])
+    w = L["cb"][L["idx"]].reshape(n, k).to(act).float()
+    for m in (1, 4, 16):
+        x = torch.randn(m, k, generator=cases.gen(m)).to(act)
+        _close(layer(x.to(gpu)), torch.nn.functional.linear(x[:, perm].float(), w, L["bias"].float()))
+    assert seen == [True, True, True]
+    assert layer._derived["perm_i32"].dtype == torch.int32
+
+
 # ------------------------------------------------------ benchmark full sizes ---
 
 
