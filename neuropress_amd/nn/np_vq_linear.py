@@ -36,7 +36,13 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from ..qweights import VQScheme, VQWeight, is_vq_weight
-from ..transforms.vq_packing import IndexPacking
+from ..transforms.vq_entropy_packing import decode_to_flat
+from ..transforms.vq_packing import (
+    IndexPacking,
+    NTieredIndexPacking,
+    TieredIndexPacking,
+    ZeroEscapePacking,
+)
 from .backends import Backend, VQBackend, is_hip_backend_available, tile_band_ok
 
 log = logging.getLogger(__name__)
@@ -101,10 +107,11 @@ _ALLOW_FALLBACK: bool = os.environ.get("NEUROPRESS_ALLOW_KERNEL_FALLBACK", "").s
     "1", "true", "yes",
 )  # fmt: skip
 
-_FUSED_BACKENDS = frozenset({VQBackend.CUDA_WMMA, VQBackend.CUDA_LUT, VQBackend.CUDA})
-_UNSUPPORTED_BACKENDS = frozenset(
-    {VQBackend.CUDA_TIERED, VQBackend.CUDA_NTIER, VQBackend.CUDA_ZERO_ESCAPE}
-)
+# Backends that run the HIP bands.  The three per-format members name, in the reference, kernels
+# that decode a prefix-coded stream inside the GEMV; here such layers are expanded to the fixed-width
+# stream at construction, so the members are labels that route like CUDA_WMMA.
+_CODED_BACKENDS = frozenset({VQBackend.CUDA_TIERED, VQBackend.CUDA_NTIER, VQBackend.CUDA_ZERO_ESCAPE})
+_FUSED_BACKENDS = frozenset({VQBackend.CUDA_WMMA, VQBackend.CUDA_LUT, VQBackend.CUDA}) | _CODED_BACKENDS
 
 # Latched once the tile GEMM fails with fallback allowed, so later calls go
 # straight to decode + GEMM (reference: np_vq_linear.py:91-93).
@@ -152,11 +159,16 @@ def _resolve_vq_backend(
         val = str(backend)
     if val != "auto":
         return VQBackend(val)  # raises ValueError for unknown strings
-    if use_tiered or use_ntier or use_zero_escape:
+    if not (torch.cuda.is_available() and is_hip_backend_available()):
         return VQBackend.COMPILE
-    if torch.cuda.is_available() and is_hip_backend_available():
-        return VQBackend.CUDA_WMMA
-    return VQBackend.COMPILE
+    # Same precedence as the reference (np_vq_linear.py:158-163); all four run the same kernels.
+    if use_zero_escape:
+        return VQBackend.CUDA_ZERO_ESCAPE
+    if use_ntier:
+        return VQBackend.CUDA_NTIER
+    if use_tiered:
+        return VQBackend.CUDA_TIERED
+    return VQBackend.CUDA_WMMA
 
 
 def _vq_dequant_linear(
@@ -242,9 +254,14 @@ class VQProxy(nn.Module):
 class NPVQLinear(nn.Module):
     """Linear layer with a VQ-compressed weight and a shared codebook proxy.
 
-    Constructor arguments up to ``column_perm`` are the reference's
-    (neuropress/nn/np_vq_linear.py:493-513).  The entropy-coded-format arguments
-    are accepted for signature compatibility and rejected when set.  The
+    Constructor arguments up to ``zesc_row_offsets`` are the reference's
+    (neuropress/nn/np_vq_linear.py:493-513).  With ``use_tiered`` / ``tier_bits`` /
+    ``zero_escape`` the buffer passed as ``packed_indices`` is a prefix-coded one
+    (``transforms/vq_entropy_packing.py``): it is expanded once, here, into the
+    fixed-width stream all kernels read (``self.packed_indices``, ``self.bits`` wide),
+    so these layers run the same three bands as any other; the ``*_row_offsets``
+    arguments, which the reference's per-format kernels need, are accepted and
+    unused, and :meth:`to_qtensor` packs the indices back.  The
     ``residual_*`` / ``row_*`` arguments add an optional residual codebook and
     a per-output-row fp16 scale and bias on the decoded weight:
 
@@ -280,11 +297,6 @@ class NPVQLinear(nn.Module):
         row_bias: torch.Tensor | None = None,
     ) -> None:
         super().__init__()
-        if use_tiered or tier_bits is not None or zero_escape:
-            raise NotImplementedError(
-                "NPVQLinear: entropy-coded index formats (tiered / n-tier / zero-escape) "
-                "are not supported by this backend; use fixed-width IndexPacking."
-            )
         if in_features % vector_len:
             raise ValueError(f"in_features={in_features} not divisible by vector_len={vector_len}")
         if proxy.vector_len != vector_len:
@@ -295,19 +307,26 @@ class NPVQLinear(nn.Module):
         self.vector_len = vector_len
         self.bits = bits
         self.n_vectors = out_features * (in_features // vector_len)
-        self.use_tiered = False
+        # Same precedence as the reference's scheme (neuropress/transforms/vq.py:220-247).
+        self.zero_escape = bool(zero_escape)
+        self.tier_bits = None if zero_escape or tier_bits is None else list(tier_bits)
+        self.use_tiered = bool(use_tiered) and not zero_escape and tier_bits is None
         self.cold_bits = cold_bits
-        self.tier_bits = None
-        self.zero_escape = False
+        self._hot_bits = TieredIndexPacking.DEFAULT_HOT_BITS
+        self._coded_bits = bits
+        if self.zero_escape or self.tier_bits is not None or self.use_tiered:
+            packed_indices, bits = self._expand_prefix_coded(packed_indices, proxy.num_centroids)
+            self.bits = bits
         self.backend = _resolve_vq_backend(
             backend,
+            use_tiered=self.use_tiered,
+            use_ntier=self.tier_bits is not None,
+            use_zero_escape=self.zero_escape,
             bits=bits,
             out_features=out_features,
             num_centroids=proxy.num_centroids,
             vector_len=vector_len,
         )
-        if self.backend in _UNSUPPORTED_BACKENDS:
-            raise NotImplementedError(f"backend {self.backend.value!r} is not supported")
         need = IndexPacking.packed_nbytes(self.n_vectors, bits)
         if packed_indices.numel() < need:
             raise ValueError(
@@ -337,6 +356,41 @@ class NPVQLinear(nn.Module):
         self._register_optional("row_bias", None if row_bias is None else row_bias.to(torch.float16))
         # Derived, rebuilt on demand: f32 bias for the kernels, widened index stream.
         self._derived: dict = {}
+
+    def _expand_prefix_coded(self, coded: torch.Tensor, num_centroids: int) -> tuple[torch.Tensor, int]:
+        """Prefix-coded buffer -> ``(fixed-width stream, its bit width)``.
+
+        The reference keeps such layers in their coded form and decodes prefixes in
+        every GEMV (np_vq_linear.py:644-801, kernels/vq_linear_tiered.cu); here the
+        coded form is a storage format only.
+        """
+        self._coded_bits = self.bits  # the width argument as given (the reference's cold-tier width)
+        if self.use_tiered:
+            _, _, self.cold_bits, self._hot_bits, _ = TieredIndexPacking._parse_header(coded)
+        elif self.zero_escape:
+            self.cold_bits = ZeroEscapePacking._parse_header(coded)[1]
+        idx = decode_to_flat(
+            coded, use_tiered=self.use_tiered, tier_bits=self.tier_bits, zero_escape=self.zero_escape
+        )
+        if idx.numel() != self.n_vectors:
+            raise ValueError(
+                f"prefix-coded buffer holds {idx.numel()} indices, the layer needs {self.n_vectors}"
+            )
+        if idx.numel() and int(idx.max().item()) >= num_centroids:
+            raise ValueError("prefix-coded buffer names a codebook row past the end of the codebook")
+        width = IndexPacking.bits_for(num_centroids)
+        if width == 4 and idx.numel() % 2:
+            width = 8  # a 4-bit stream needs an even count
+        return IndexPacking.pack(idx, width), width
+
+    def _coded_indices(self) -> torch.Tensor:
+        """The layer's indices packed back into the prefix-coded format it was built from."""
+        idx = IndexPacking.unpack(self.packed_indices.cpu(), self.bits, self.n_vectors)
+        if self.zero_escape:
+            return ZeroEscapePacking.pack(idx, self.cold_bits)
+        if self.tier_bits is not None:
+            return NTieredIndexPacking.pack(idx, self.tier_bits)
+        return TieredIndexPacking.pack(idx, self.cold_bits, self._hot_bits)
 
     def _register_optional(self, name: str, t: torch.Tensor | None) -> None:
         if t is not None:
@@ -412,17 +466,22 @@ class NPVQLinear(nn.Module):
                 "Cannot reconstruct QTensor: no serde metadata stored. "
                 "Build via NPVQLinear.from_qtensor_linear() to enable to_qtensor()."
             )
+        coded = self.use_tiered or self.tier_bits is not None or self.zero_escape
         scheme = VQScheme(
             centroids=self.proxy.centroids,
             original_shape=(self.out_features, self.in_features),
-            is_packed_indices=self.bits,
+            is_packed_indices=self._coded_bits if coded else self.bits,
             column_permutation=self.column_perm,
+            use_tiered=self.use_tiered,
+            tier_bits=self.tier_bits,
+            zero_escape=self.zero_escape,
             residual_centroids=None if self.residual_proxy is None else self.residual_proxy.centroids,
             residual_bits=self.residual_bits,
             row_scale=self.row_scale,
             row_bias=self.row_bias,
         )
-        return VQWeight(self.packed_indices, scheme, self.packed_residual)
+        blob = self._coded_indices().to(self.packed_indices.device) if coded else self.packed_indices
+        return VQWeight(blob, scheme, self.packed_residual)
 
     # ------------------------------------------------------------------
     # Derived buffers
@@ -492,7 +551,7 @@ class NPVQLinear(nn.Module):
                 return self._forward_dequant_gemm(x)
         if self.backend == VQBackend.CUDA_LUT:
             return self._forward_cuda_lut(x)
-        if self.backend == VQBackend.CUDA_WMMA:
+        if self.backend == VQBackend.CUDA_WMMA or self.backend in _CODED_BACKENDS:
             return self._forward_cuda_wmma(x)
         if self.backend == VQBackend.CUDA:
             return self._forward_cuda(x)
@@ -746,12 +805,20 @@ class NPVQLinear(nn.Module):
     def extra_repr(self) -> str:
         perm_str = ", perm=True" if self.column_perm is not None else ""
         res_str = ", residual=True" if self.is_residual else ""
+        if self.zero_escape:
+            tiered_str = ", zero_escape=True"
+        elif self.tier_bits is not None:
+            tiered_str = f", ntier={self.tier_bits}"
+        elif self.use_tiered:
+            tiered_str = f", tiered=True(cold={self.cold_bits})"
+        else:
+            tiered_str = ""
         return (
             f"in={self.in_features}, out={self.out_features}, "
             f"vector_len={self.vector_len}, "
             f"num_centroids={self.proxy.num_centroids}, "
             f"bits={self.bits}, backend={self.backend.value}"
-            f"{perm_str}{res_str}"
+            f"{perm_str}{tiered_str}{res_str}"
         )
 
 

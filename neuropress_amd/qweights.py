@@ -72,7 +72,13 @@ class VQScheme:
         for d in self.original_shape:
             n_vec *= d
         n_vec //= self.vector_len
-        idx = IndexPacking.unpack(packed_indices, self.is_packed_indices, n_vec)
+        if self.zero_escape or self.tier_bits is not None or self.use_tiered:
+            from .transforms.vq_entropy_packing import decode_to_flat
+
+            idx = decode_to_flat(packed_indices, use_tiered=self.use_tiered, tier_bits=self.tier_bits,
+                                 zero_escape=self.zero_escape)  # fmt: skip
+        else:
+            idx = IndexPacking.unpack(packed_indices, self.is_packed_indices, n_vec)
         out = self.centroids.to(packed_indices.device)[idx].to(target_dtype)
         out = out.flatten().reshape(tuple(self.original_shape))
         if self.column_permutation is not None:
@@ -99,14 +105,37 @@ class VQWeight:
         in_features: int,
         column_permutation: torch.Tensor | None = None,
         bits: int = 0,
+        use_tiered: bool = False,
+        hot_bits: int = 4,
+        tier_bits: list[int] | None = None,
+        zero_escape: bool = False,
     ) -> VQWeight:
+        """Pack *indices* in the fixed-width format, or in a prefix-coded one when a flag names it
+        (the choice the reference makes in ``VQScheme.quantize_as_u8``, neuropress/transforms/vq.py:351-357)."""
+        from .transforms.vq_entropy_packing import NTieredIndexPacking, TieredIndexPacking, ZeroEscapePacking
+
+        if zero_escape:
+            use_tiered, tier_bits = False, None
+        elif tier_bits is not None:
+            use_tiered = False
         scheme = VQScheme(
             centroids=centroids,
             original_shape=(out_features, in_features),
             is_packed_indices=bits,
             column_permutation=column_permutation,
+            use_tiered=use_tiered,
+            tier_bits=tier_bits,
+            zero_escape=zero_escape,
         )
-        return cls(IndexPacking.pack(indices, scheme.is_packed_indices), scheme)
+        if zero_escape:
+            blob = ZeroEscapePacking.pack(indices, scheme.is_packed_indices)
+        elif tier_bits is not None:
+            blob = NTieredIndexPacking.pack(indices, tier_bits)
+        elif use_tiered:
+            blob = TieredIndexPacking.pack(indices, scheme.is_packed_indices, hot_bits)
+        else:
+            blob = IndexPacking.pack(indices, scheme.is_packed_indices)
+        return cls(blob, scheme)
 
     @property
     def shape(self) -> tuple:

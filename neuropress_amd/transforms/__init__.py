@@ -1,3 +1,8 @@
 """Wire formats consumed by the quantized-linear path."""
 
-from .vq_packing import IndexPacking  # noqa: F401
+from .vq_packing import (  # noqa: F401
+    IndexPacking,
+    NTieredIndexPacking,
+    TieredIndexPacking,
+    ZeroEscapePacking,
+)

@@ -97,3 +97,12 @@ class IndexPacking:
         byte0 = bit0 >> 3
         window = p[byte0] | (p[byte0 + 1] << 8) | (p[byte0 + 2] << 16) | (p[byte0 + 3] << 24)
         return (window >> (bit0 & 7)) & ((1 << bits) - 1)
+
+
+# The prefix-coded storage formats live in their own module; they are importable from here as in
+# the reference (neuropress/transforms/vq_packing.py:298, 612, 1037).
+from .vq_entropy_packing import (  # noqa: E402, F401
+    NTieredIndexPacking,
+    TieredIndexPacking,
+    ZeroEscapePacking,
+)

@@ -22,6 +22,12 @@
  *       the identity "residual codebook 0, scale 1, bias 0 == vq_decode".
  *   np_oracle_linear      -- textbook GEMM in double precision; compared with
  *       numpy float64 matmul.
+ *   np_oracle_tiered_unpack / ntier_unpack / zesc_unpack -- the reference holds
+ *       no byte-level vectors for these formats (its tests are round trips,
+ *       header fields and byte-count formulas); pinned by hand-assembled
+ *       buffers written out bit by bit from the format descriptions, by the
+ *       reference tests' header / byte-count assertions, and by round trips
+ *       through an independent packer (tests/test_host_entropy_packing.py).
  */
 #include <stdint.h>
 #include <string.h>
@@ -189,6 +195,115 @@ int np_oracle_pack_indices(const int64_t* idx, int64_t n, int bits, uint8_t* out
     }
   }
   return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* Prefix-coded index formats (storage forms of the index stream)      */
+/* ------------------------------------------------------------------ */
+
+static uint32_t rd_u32(const uint8_t* p) {
+  return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+/* `width` bits starting at stream bit `pos`, LSB first (same layout as the index stream). */
+static int64_t rd_bits(const uint8_t* stream, int64_t pos, int width) {
+  int64_t v = 0;
+  for (int b = 0; b < width; ++b) {
+    const int64_t q = pos + b;
+    v |= (int64_t)((stream[q >> 3] >> (q & 7)) & 1) << b;
+  }
+  return v;
+}
+
+/*
+ * Two-tier buffer -> indices, walking the indices in order with one cursor per
+ * stream.  Layout (neuropress/transforms/vq_packing.py:298-332, 461-521):
+ * header n, n_hot, cold_bits, hot_bits (uint32 LE; a 12-byte header without
+ * hot_bits, or a 4th word outside [4,16], means hot_bits = 4 and the streams
+ * start at byte 12: vq_packing.py:421-459); prefix bit i = 1 -> cold; hot
+ * stream (hot_bits each), cold stream (cold_bits each).
+ * Returns the index count, or -1 (short buffer) / -2 (counts disagree with the prefix stream).
+ */
+int64_t np_oracle_tiered_unpack(const uint8_t* buf, int64_t n_bytes, int64_t cap, int64_t* out) {
+  if (n_bytes < 12) return -1;
+  const int64_t n = rd_u32(buf), n_hot = rd_u32(buf + 4);
+  const int cold_bits = (int)rd_u32(buf + 8);
+  int hot_bits = 4;
+  int64_t at = 12;
+  if (n_bytes >= 16) {
+    const uint32_t cand = rd_u32(buf + 12);
+    if (cand >= 4 && cand <= 16) { hot_bits = (int)cand; at = 16; }
+  }
+  if (n > cap || n_hot > n) return -1;
+  const uint8_t* prefix = buf + at;
+  const uint8_t* hot = prefix + (n + 7) / 8;
+  const uint8_t* cold = hot + (n_hot * hot_bits + 7) / 8;
+  if (cold + ((n - n_hot) * cold_bits + 7) / 8 > buf + n_bytes) return -1;
+  int64_t ih = 0, ic = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    if (rd_bits(prefix, i, 1)) out[i] = rd_bits(cold, (ic++) * cold_bits, cold_bits);
+    else out[i] = rd_bits(hot, (ih++) * hot_bits, hot_bits);
+  }
+  return (ih == n_hot && ic == n - n_hot) ? n : -2;
+}
+
+/*
+ * N-tier buffer -> indices (neuropress/transforms/vq_packing.py:612-646, 842-908).
+ * Header magic 0x4E565154, n, D, then (count_k, bits_k) per tier; prefix stream
+ * k has one bit per index not claimed by tiers < k (0 = tier k); payload of tier
+ * k is index - 2^bits_(k-1) (tier 0: the index) in bits_k bits.  An index is
+ * decoded by descending the levels until a prefix bit is 0 (or the last tier).
+ */
+int64_t np_oracle_ntier_unpack(const uint8_t* buf, int64_t n_bytes, int64_t cap, int64_t* out) {
+  if (n_bytes < 12 || rd_u32(buf) != 0x4E565154u) return -1;
+  const int64_t n = rd_u32(buf + 4);
+  const int d = (int)rd_u32(buf + 8);
+  if (d < 2 || d > 4 || n_bytes < 12 + 8 * d || n > cap) return -1;
+  int64_t count[4], cursor_p[4] = {0, 0, 0, 0}, cursor_v[4] = {0, 0, 0, 0};
+  int bits[4];
+  const uint8_t* prefix[4];
+  const uint8_t* payload[4];
+  for (int k = 0; k < d; ++k) { count[k] = rd_u32(buf + 12 + 8 * k); bits[k] = (int)rd_u32(buf + 16 + 8 * k); }
+  const uint8_t* at = buf + 12 + 8 * d;
+  int64_t alive = n;
+  for (int k = 0; k < d - 1; ++k) { prefix[k] = at; at += (alive + 7) / 8; alive -= count[k]; }
+  for (int k = 0; k < d; ++k) { payload[k] = at; at += (count[k] * bits[k] + 7) / 8; }
+  if (at > buf + n_bytes) return -1;
+  for (int64_t i = 0; i < n; ++i) {
+    int k = 0;
+    while (k < d - 1 && rd_bits(prefix[k], cursor_p[k]++, 1)) ++k;
+    const int64_t base = k == 0 ? 0 : (int64_t)1 << bits[k - 1];
+    out[i] = base + rd_bits(payload[k], (cursor_v[k]++) * bits[k], bits[k]);
+  }
+  for (int k = 0; k < d; ++k) if (cursor_v[k] != count[k]) return -2;
+  return n;
+}
+
+/*
+ * Zero-escape buffer -> indices (neuropress/transforms/vq_packing.py:1037-1075, 1206-1277).
+ * Header magic 0x5A455343, n, cold_bits, n_zero, n_hot, n_warm; class stream of 2 bits per
+ * index: 0 -> index 0; 1 -> 1 + 4-bit payload; 2 -> 17 + 8-bit payload; 3 -> 257 + cold payload.
+ */
+int64_t np_oracle_zesc_unpack(const uint8_t* buf, int64_t n_bytes, int64_t cap, int64_t* out) {
+  if (n_bytes < 24 || rd_u32(buf) != 0x5A455343u) return -1;
+  const int64_t n = rd_u32(buf + 4);
+  const int cold_bits = (int)rd_u32(buf + 8);
+  const int64_t n_zero = rd_u32(buf + 12), n_hot = rd_u32(buf + 16), n_warm = rd_u32(buf + 20);
+  const int64_t n_cold = n - n_zero - n_hot - n_warm;
+  if (n > cap || n_cold < 0) return -1;
+  const uint8_t* cls = buf + 24;
+  const uint8_t* hot = cls + (2 * n + 7) / 8;
+  const uint8_t* warm = hot + (n_hot * 4 + 7) / 8;
+  const uint8_t* cold = warm + n_warm;
+  if (cold + (n_cold * cold_bits + 7) / 8 > buf + n_bytes) return -1;
+  int64_t seen[4] = {0, 0, 0, 0};
+  for (int64_t i = 0; i < n; ++i) {
+    const int c = (int)rd_bits(cls, 2 * i, 2);
+    const int64_t j = seen[c]++;
+    out[i] = c == 0 ? 0 : c == 1 ? 1 + rd_bits(hot, 4 * j, 4) : c == 2 ? 17 + rd_bits(warm, 8 * j, 8)
+                                                                      : 257 + rd_bits(cold, cold_bits * j, cold_bits);
+  }
+  return (seen[0] == n_zero && seen[1] == n_hot && seen[2] == n_warm) ? n : -2;
 }
 
 /* ------------------------------------------------------------------ */

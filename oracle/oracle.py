@@ -54,6 +54,9 @@ def _load() -> ctypes.CDLL:
     lib.np_oracle_bits_for.restype = _int
     lib.np_oracle_unpack_indices.argtypes = [_u8p, _i64, _int, _i64, _i64p]
     lib.np_oracle_pack_indices.argtypes = [_i64p, _i64, _int, _u8p]
+    for name in ("np_oracle_tiered_unpack", "np_oracle_ntier_unpack", "np_oracle_zesc_unpack"):
+        getattr(lib, name).argtypes = [_u8p, _i64, _i64, _i64p]
+        getattr(lib, name).restype = _i64
     lib.np_oracle_vq_decode.argtypes = [_u8p, _i64, _int, _u16p, _i64, _int, _i64, _int, _vp]
     lib.np_oracle_rvq_decode.argtypes = [
         _u8p, _i64, _int, _u8p, _i64, _int, _u16p, _i64, _u16p, _i64,
@@ -114,6 +117,18 @@ def pack_indices(idx: np.ndarray, bits: int) -> np.ndarray:
     rc = _load().np_oracle_pack_indices(_ptr(idx, _i64p), idx.size, bits, _ptr(out, _u8p))
     _check(rc, "pack_indices")
     return out
+
+
+def entropy_unpack(kind: str, packed: np.ndarray) -> np.ndarray:
+    """Indices of a prefix-coded buffer; kind in {"tiered", "ntier", "zero_escape"}."""
+    fn = {"tiered": "np_oracle_tiered_unpack", "ntier": "np_oracle_ntier_unpack",
+          "zero_escape": "np_oracle_zesc_unpack"}[kind]  # fmt: skip
+    packed = _c(packed, np.uint8)
+    out = np.empty(packed.size * 8, dtype=np.int64)  # an index costs at least one stream bit
+    n = getattr(_load(), fn)(_ptr(packed, _u8p), packed.size, out.size, _ptr(out, _i64p))
+    if n < 0:
+        raise ValueError(f"{fn}: malformed buffer (code {n})")
+    return out[:n].copy()
 
 
 def vq_decode(

@@ -159,6 +159,43 @@ def test_column_perm_is_folded_into_the_fused_gemv(gpu, act, monkeypatch):
     assert layer._derived["perm_i32"].dtype == torch.int32
 
 
+@pytest.mark.parametrize("kind", ["tiered", "ntier", "zero_escape"])
+def test_prefix_coded_layers_run_the_hip_bands(gpu, kind, monkeypatch):
+    """A weight stored in a two-tier / n-tier / zero-escape buffer (Zipf-distributed indices, as the
+    formats assume): "auto" lowering names the reference's per-format backend and the layer runs the
+    slice-list GEMV, the fused GEMV, the tile GEMM and decode + GEMM on its expanded stream."""
+    from neuropress_amd import kernels
+
+    monkeypatch.setattr(vqmod, "_SLICED_MIN_INDICES", 1)
+    monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
+    n, k, nc = 128, 512, 20000
+    g = cases.gen(91)
+    cb = (torch.randn(nc, 8, generator=g) * 0.05).half()
+    p = 1.0 / torch.arange(1, nc + 1, dtype=torch.float64) ** 1.1
+    idx = torch.multinomial(p / p.sum(), n * k // 8, replacement=True, generator=g)
+    kw = {"tiered": dict(use_tiered=True, hot_bits=8), "ntier": dict(tier_bits=[4, 8, 12, 15]),
+          "zero_escape": dict(zero_escape=True)}[kind]
+    model = nn.Sequential(attach_quantized_weight(nn.Linear(k, n, bias=True),
+                                                  VQWeight.from_indices(idx, cb, n, k, bits=15, **kw)))
+    bias = model[0].bias.detach().clone()
+    model.to(gpu)
+    AutoKernelLowering().apply(model)
+    model.to(gpu)  # the weight container is not a parameter: the lowered module's buffers move here
+    layer = model[0]
+    assert layer.backend.value == {"tiered": "cuda_tiered", "ntier": "cuda_ntier", "zero_escape": "cuda_zero_escape"}[kind]
+    assert layer.bits == 15 and layer.packed_indices.is_cuda
+    calls = []
+    for name in ("vq_linear_sliced", "vq_linear", "vq_gemm_tile", "vq_dequant"):
+        real = getattr(kernels, name)
+        monkeypatch.setattr(kernels, name, lambda *a, _r=real, _n=name, **kw_: (calls.append(_n), _r(*a, **kw_))[1])
+    w = cb[idx].reshape(n, k).float()
+    for m in (1, 12, 40, 100):
+        x = torch.randn(m, k, generator=cases.gen(m)).half()
+        _close(layer(x.to(gpu)), torch.nn.functional.linear(x.float(), w, bias.float()))
+    assert calls == ["vq_linear_sliced", "vq_linear", "vq_gemm_tile", "vq_dequant"]
+
+
 # ------------------------------------------------------ benchmark full sizes ---
 
 

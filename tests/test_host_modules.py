@@ -57,8 +57,8 @@ def test_from_qtensor_linear():
 def test_constructor_rejects_bad_input():
     proxy = VQProxy(torch.randn(16, 8))
     packed = torch.zeros(64, dtype=torch.uint8)
-    with pytest.raises(NotImplementedError, match="entropy-coded"):
-        NPVQLinear(proxy, packed, 4, 16, 64, 8, "default", use_tiered=True)
+    with pytest.raises(ValueError, match="prefix-coded buffer holds 0 indices"):
+        NPVQLinear(proxy, packed, 4, 16, 64, 8, "default", use_tiered=True)  # an all-zero tiered header
     with pytest.raises(ValueError, match="divisible"):
         NPVQLinear(proxy, packed, 4, 16, 60, 8, "default")
     with pytest.raises(ValueError, match="bytes"):
@@ -370,3 +370,63 @@ def test_tile_band_rule_counts_reduction_splits():
     assert not ok(17, 1024, 4096)  # 16 tiles x 8 splits = half the compute units
     assert not ok(17, 4096, 512)  # no split possible below 1024 input features
     assert ok(17, 2048, 4096)  # 32 tiles x 8 splits
+
+
+@pytest.mark.parametrize("kind", ["tiered", "tiered_hot8", "ntier", "zero_escape"])
+def test_prefix_coded_layers_expand_to_the_fixed_width_stream(kind):
+    """A layer built from a two-tier / n-tier / zero-escape buffer (reference:
+    np_vq_linear.py:504-511, 573-640) holds the same fixed-width stream, gives the same output and
+    packs back to the same bytes as the reference's formats define."""
+    from neuropress_amd.transforms.vq_packing import (
+        IndexPacking,
+        NTieredIndexPacking,
+        TieredIndexPacking,
+        ZeroEscapePacking,
+    )
+
+    n, k, nc = 24, 64, 1024
+    g = torch.Generator().manual_seed(11)
+    cb = torch.randn(nc, 8, generator=g) * 0.05
+    p = 1.0 / torch.arange(1, nc + 1, dtype=torch.float64) ** 1.1
+    idx = torch.multinomial(p / p.sum(), n * k // 8, replacement=True, generator=g)
+    kw = {"tiered": dict(use_tiered=True), "tiered_hot8": dict(use_tiered=True, hot_bits=8),
+          "ntier": dict(tier_bits=[4, 8, 10]), "zero_escape": dict(zero_escape=True)}[kind]
+    wq = VQWeight.from_indices(idx, cb, n, k, bits=10, **kw)
+    coded = wq.u8_blob
+    want = {"tiered": TieredIndexPacking.pack(idx, 10), "tiered_hot8": TieredIndexPacking.pack(idx, 10, 8),
+            "ntier": NTieredIndexPacking.pack(idx, [4, 8, 10]), "zero_escape": ZeroEscapePacking.pack(idx, 10)}[kind]
+    assert torch.equal(coded, want)
+    lin = attach_quantized_weight(nn.Linear(k, n, bias=True), wq)
+    plain = NPVQLinear(VQProxy(cb), IndexPacking.pack(idx, 10), 10, n, k, 8, "default", bias=lin.bias.detach())
+    layer = NPVQLinear.from_qtensor_linear(lin, VQProxy(cb), backend="default")
+    assert layer.bits == 10 and torch.equal(layer.packed_indices, plain.packed_indices)
+    assert (layer.use_tiered, layer.tier_bits, layer.zero_escape) == (
+        kind.startswith("tiered"), [4, 8, 10] if kind == "ntier" else None, kind == "zero_escape")
+    x = torch.randn(5, k, generator=g)
+    assert torch.equal(layer(x), plain(x))
+    assert {"tiered": "tiered=True(cold=10)", "tiered_hot8": "tiered=True(cold=10)", "ntier": "ntier=[4, 8, 10]",
+            "zero_escape": "zero_escape=True"}[kind] in layer.extra_repr()
+    back = layer.to_qtensor()
+    assert torch.equal(back.u8_blob, coded)  # byte-identical round trip, hot_bits included
+    assert (back.qscheme.use_tiered, back.qscheme.tier_bits, back.qscheme.zero_escape) == (
+        layer.use_tiered, layer.tier_bits, layer.zero_escape)
+    w = cb.half()[idx].reshape(n, k).float()  # the proxy keeps the codebook in fp16
+    assert torch.equal(back.qscheme.dequantize(back.u8_blob, torch.float32), w)
+    with pytest.raises(ValueError, match="past the end of the codebook"):
+        NPVQLinear(VQProxy(cb[:512]), coded, 10, n, k, 8, "default", **{a: b for a, b in kw.items() if a != "hot_bits"})
+
+
+def test_prefix_coded_backends_resolve_like_the_reference(monkeypatch):
+    """"auto" with a format flag: zero-escape > n-tier > tiered when the HIP backend can run
+    (np_vq_linear.py:158-163), COMPILE otherwise; the explicit members are accepted."""
+    import neuropress_amd.nn.np_vq_linear as vqmod
+
+    res = vqmod._resolve_vq_backend
+    assert res("auto", use_tiered=True).value == "compile"  # no GPU here
+    monkeypatch.setattr(vqmod.torch.cuda, "is_available", lambda: True)
+    monkeypatch.setattr(vqmod, "is_hip_backend_available", lambda: True)
+    assert res("auto", use_tiered=True, use_ntier=True, use_zero_escape=True).value == "cuda_zero_escape"
+    assert res("auto", use_tiered=True, use_ntier=True).value == "cuda_ntier"
+    assert res("auto", use_tiered=True).value == "cuda_tiered"
+    assert res("auto").value == "cuda_wmma"
+    assert res("cuda_tiered").value == "cuda_tiered"
