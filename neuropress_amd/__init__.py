@@ -28,4 +28,20 @@ from .nn import (  # noqa: F401
     linearize_vq_weights,
 )
 
+
+
+def save_quantized_model(model, path, recipe_config_json=None):
+    """Write a (lowered or unlowered) quantized model to one safetensors file (``t2n.model_io``)."""
+    from .t2n.model_io import save_quantized_model as _save
+
+    return _save(model, path, recipe_config_json)
+
+
+def load_quantized_model(model, path, kernel_lowering="auto"):
+    """Load such a file into *model* and, by default, lower it (``t2n.model_io``)."""
+    from .t2n.model_io import load_quantized_model as _load
+
+    return _load(model, path, kernel_lowering)
+
+
 __version__ = "0.1.0"
