@@ -257,6 +257,42 @@ int npamd_q_gemm_tile(const void* x, int64_t ldx, const uint8_t* w_pack, const v
                       int M, int N, int K, int nbits, int group_size, int act_dtype,
                       void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ------------------------------------- neighbours of the linear on a decode step ---- */
+/*
+ * Fused RMSNorm over the last dimension, one pass over x:
+ *   out[m, i] = round(x[m, i] * rsqrt(mean_i(x[m, i]^2) + eps) * weight[i]),  f32 arithmetic.
+ * Replaces rms_norm (neuropress/kernels/rms_norm.cu:27-110).  x, weight, out share `dtype`
+ * (NPAMD_F16 / NPAMD_BF16 / NPAMD_F32); ldx, ldo are row strides in elements.
+ */
+int npamd_rms_norm(const void* x, int64_t ldx, const void* weight, void* out, int64_t ldo,
+                   int M, int H, float eps, int dtype, void* stream);
+
+/*
+ * Embedding lookup in a VQ-compressed table (NPVQEmbedding.forward,
+ * neuropress/nn/np_vq_embedding.py:120-142):
+ *   row[t, g*VL + v] = codebook[indices[ids[t], g], v]
+ *   out[t, j] = cast(f16(row[t, inv_perm[j]] * scale))
+ * `indices`: [vocab, groups] 16-bit indices (read as unsigned); `inv_perm`: NULL or `groups*VL`
+ * int32 column numbers; the multiply is skipped (no rounding) when scale == 1.  ids outside
+ * [0, vocab) are clamped.  out: [n_ids, groups*VL] of out_dtype.
+ */
+int npamd_vq_embedding(const int64_t* ids, int64_t n_ids, const int16_t* indices, int64_t vocab,
+                       int groups, const void* codebook_f16, int nc, int vl,
+                       const int32_t* inv_perm, float scale, void* out, int out_dtype, void* stream);
+
+/*
+ * Embedding lookup in a group-affine n-bit table, n in {1, 2, 4, 8} (_emb_dequant and
+ * NPEmbedding.forward, neuropress/nn/np_embedding.py:120-183, 455-473):
+ *   v = f16((q - zp) * scale) in f32 arithmetic (zp = 2^(n-1) when zero_point_f16 is NULL),
+ *   v = 0 where ids[t] == padding_idx (pass -1 for none),
+ *   out = round(cast(v) * embed_scale), the multiply skipped when embed_scale == 1.
+ * w_pack: [vocab, dim * n / 8] codes, low bits first; scale / zero point: [vocab * dim / group_size] f16.
+ */
+int npamd_q_embedding(const int64_t* ids, int64_t n_ids, const uint8_t* w_pack,
+                      const void* scale_f16, const void* zero_point_f16, int nbits, int group_size,
+                      int64_t vocab, int dim, int64_t padding_idx, float embed_scale,
+                      void* out, int out_dtype, void* stream);
+
 /* ------------------------------------------------------ diagnostics ---- */
 /*
  * Memory-system ceilings for the access patterns of the kernels above (no

@@ -47,6 +47,9 @@ SIGNATURES: dict[str, list] = {
     "npamd_rvq_gemm_tile": _RVQ_LINEAR[:-1] + _WS + [_vp],
     "npamd_q_dequant": [_vp, _vp, _vp, _int, _int, _int, _int, _vp, _int, _vp],
     "npamd_q_gemv": _Q_LINEAR,
+    "npamd_rms_norm": [_vp, _i64, _vp, _vp, _i64, _int, _int, ctypes.c_float, _int, _vp],
+    "npamd_vq_embedding": [_vp, _i64, _vp, _i64, _int, _vp, _int, _int, _vp, ctypes.c_float, _vp, _int, _vp],
+    "npamd_q_embedding": [_vp, _i64, _vp, _vp, _vp, _int, _int, _i64, _int, _i64, ctypes.c_float, _vp, _int, _vp],
     "npamd_q_gemm_tile": _Q_LINEAR[:-1] + _WS + [_vp],
     "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
     "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],

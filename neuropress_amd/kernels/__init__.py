@@ -608,3 +608,102 @@ def warn_kernel_fallback(kernel: str, fallback: str, exc: BaseException) -> None
         exc,
         fallback,
     )
+
+
+# ---------------------------------------------------------------------------
+# Neighbours of the linear on a decode step: RMSNorm, embedding lookups
+# ---------------------------------------------------------------------------
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Fused RMSNorm over the last dimension of a 2-D ``x`` (reference: neuropress/kernels/__init__.py
+    ``rms_norm``, kernels/rms_norm.cu:79-118: same checks, same signature)."""
+    what = "rms_norm"
+    _check_device(what, x, weight)
+    if x.dim() != 2:
+        raise RuntimeError(f"{what}: x must be 2-D [M, H]")
+    if weight.dim() != 1 or weight.shape[0] != x.shape[1]:
+        raise RuntimeError(f"{what}: weight must be 1-D [H] matching x.size(1)")
+    if x.dtype != weight.dtype:
+        raise RuntimeError(f"{what}: x and weight must share dtype")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    weight = weight.contiguous()
+    out = torch.empty((x.shape[0], x.shape[1]), device=x.device, dtype=x.dtype)
+    _lib.call("npamd_rms_norm", x.data_ptr(), x.stride(0), weight.data_ptr(), out.data_ptr(), out.stride(0),
+              x.shape[0], x.shape[1], float(eps), _dt(x.dtype, what), _stream(x))  # fmt: skip
+    return out
+
+
+def vq_embedding(
+    input_ids: torch.Tensor,
+    all_indices: torch.Tensor,
+    centroids: torch.Tensor,
+    scale: float = 1.0,
+    inv_perm: torch.Tensor | None = None,
+    out_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    """Rows of a VQ-compressed embedding table: ``[..., groups * VL]`` for ids of any shape.
+
+    ``all_indices``: ``[vocab, groups]`` int16 (bit pattern of the unsigned index); ``centroids``:
+    fp16 ``[NC, VL]``; ``inv_perm``: optional int32 ``[groups * VL]``.  One kernel in place of the
+    gather / gather / permute / scale / cast sequence of neuropress/nn/np_vq_embedding.py:120-142.
+    """
+    what = "vq_embedding"
+    _check_device(what, input_ids, all_indices, centroids, inv_perm)
+    if all_indices.dtype != torch.int16 or all_indices.dim() != 2:
+        raise RuntimeError(f"{what}: all_indices must be int16 [vocab, groups]")
+    cb = _centroids_f16(centroids, what)
+    if cb.dtype != torch.float16:
+        raise RuntimeError(f"{what}: centroids must be float16")
+    vocab, groups = all_indices.shape
+    dim = groups * cb.shape[1]
+    if inv_perm is not None and (inv_perm.dtype != torch.int32 or inv_perm.numel() != dim):
+        raise RuntimeError(f"{what}: inv_perm must be int32 with {dim} entries")
+    ids = input_ids.reshape(-1).to(torch.int64).contiguous()
+    dtype = out_dtype or torch.float16
+    out = torch.empty((ids.numel(), dim), device=ids.device, dtype=dtype)
+    _lib.call("npamd_vq_embedding", ids.data_ptr(), ids.numel(), all_indices.contiguous().data_ptr(), vocab, groups,
+              cb.data_ptr(), cb.shape[0], cb.shape[1], _ptr(None if inv_perm is None else inv_perm.contiguous()),
+              float(scale), out.data_ptr(), _dt(dtype, what), _stream(out))  # fmt: skip
+    return out.reshape(*input_ids.shape, dim)
+
+
+def q_embedding(
+    input_ids: torch.Tensor,
+    u8_blob: torch.Tensor,
+    scale: torch.Tensor,
+    nbits: int,
+    group_size: int,
+    zero_point: torch.Tensor | None = None,
+    padding_idx: int | None = None,
+    embed_scale: float = 1.0,
+    out_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    """Rows of a group-affine n-bit embedding table, dequantized: gather, unpack, ``(q - zp) * scale``,
+    padding row, dtype cast and ``embed_scale`` of neuropress/nn/np_embedding.py:120-183, 455-473 in one kernel."""
+    what = "q_embedding"
+    _check_device(what, input_ids, u8_blob, scale, zero_point)
+    if u8_blob.dtype != torch.uint8 or u8_blob.dim() != 2:
+        raise RuntimeError(f"{what}: u8_blob must be uint8 [vocab, dim * nbits / 8]")
+    if nbits not in (1, 2, 4, 8):
+        raise RuntimeError(f"{what}: nbits must be 1, 2, 4 or 8, got {nbits}")
+    vocab = u8_blob.shape[0]
+    dim = u8_blob.shape[1] * (8 // nbits)
+    if dim % group_size:
+        raise RuntimeError(f"{what}: dim={dim} not divisible by group_size={group_size}")
+    sc = scale.reshape(-1).to(torch.float16).contiguous()
+    if sc.numel() != vocab * (dim // group_size):
+        raise RuntimeError(f"{what}: scale has {sc.numel()} entries, expected {vocab * (dim // group_size)}")
+    zp = None
+    if zero_point is not None:
+        zp = zero_point.reshape(-1).to(torch.float16).contiguous()
+        if zp.numel() != sc.numel():
+            raise RuntimeError(f"{what}: zero_point must have one entry per group")
+    ids = input_ids.reshape(-1).to(torch.int64).contiguous()
+    dtype = out_dtype or torch.float16
+    out = torch.empty((ids.numel(), dim), device=ids.device, dtype=dtype)
+    _lib.call("npamd_q_embedding", ids.data_ptr(), ids.numel(), u8_blob.contiguous().data_ptr(), sc.data_ptr(),
+              _ptr(zp), int(nbits), int(group_size), vocab, dim, -1 if padding_idx is None else int(padding_idx),
+              float(embed_scale), out.data_ptr(), _dt(dtype, what), _stream(out))  # fmt: skip
+    return out.reshape(*input_ids.shape, dim)

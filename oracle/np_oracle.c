@@ -28,6 +28,11 @@
  *       buffers written out bit by bit from the format descriptions, by the
  *       reference tests' header / byte-count assertions, and by round trips
  *       through an independent packer (tests/test_host_entropy_packing.py).
+ *   np_oracle_rms_norm    -- closed form in double precision; checked against
+ *       numpy float64 and the torch expression the reference names.
+ *   np_oracle_vq_embedding / np_oracle_q_embedding -- index arithmetic plus
+ *       IEEE roundings; checked against the torch op sequences of the
+ *       reference's modules run on the CPU (tests/test_oracle.py).
  */
 #include <stdint.h>
 #include <string.h>
@@ -467,6 +472,79 @@ int np_oracle_vq_linear_f32(const void* x, int x_dtype, const uint8_t* packed,
                (float)load_as_double(w_scratch, n * k_cols + k, x_dtype);
       if (bias) acc += bias[n];
       y[m * n_rows + n] = acc;
+    }
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* RMSNorm and embedding lookups                                       */
+/* ------------------------------------------------------------------ */
+
+/*
+ * out[m, i] = x[m, i] * rsqrt(mean_i x[m, i]^2 + eps) * w[i], returned in double
+ * (the caller rounds): the expression of neuropress/nn/np_rms_norm.py:48-50 and
+ * neuropress/kernels/rms_norm.cu:39-76 without its float summation order.
+ */
+int np_oracle_rms_norm(const void* x, const void* w, int dtype, int64_t M, int64_t H, double eps, double* out) {
+  if (M < 0 || H < 1) return -1;
+  for (int64_t m = 0; m < M; ++m) {
+    double ss = 0.0;
+    for (int64_t i = 0; i < H; ++i) { const double v = load_as_double(x, m * H + i, dtype); ss += v * v; }
+    const double scale = 1.0 / sqrt(ss / (double)H + eps);
+    for (int64_t i = 0; i < H; ++i) out[m * H + i] = load_as_double(x, m * H + i, dtype) * scale * load_as_double(w, i, dtype);
+  }
+  return 0;
+}
+
+/*
+ * VQ embedding rows (neuropress/nn/np_vq_embedding.py:120-142): gather the token's index row,
+ * gather codebook rows (fp16), optional inverse column permutation, optional scale with the
+ * product rounded to fp16 (an fp16 tensor times a Python float), cast to out_dtype.
+ * indices are 16-bit and read as unsigned.  Returns 0, -1 bad args, -2 id / index out of range.
+ */
+int np_oracle_vq_embedding(const int64_t* ids, int64_t n_ids, const uint16_t* indices, int64_t vocab,
+                           int64_t groups, const uint16_t* cb, int64_t nc, int64_t vl, const int32_t* inv_perm,
+                           float scale, int out_dtype, void* out) {
+  if (n_ids < 0 || vocab < 1 || groups < 1 || nc < 1 || vl < 1) return -1;
+  const int64_t dim = groups * vl;
+  for (int64_t t = 0; t < n_ids; ++t) {
+    if (ids[t] < 0 || ids[t] >= vocab) return -2;
+    for (int64_t j = 0; j < dim; ++j) {
+      const int64_t src = inv_perm ? inv_perm[j] : j;
+      const int64_t c = indices[ids[t] * groups + src / vl];
+      if (c >= nc) return -2;
+      float v = f16_to_f32(cb[c * vl + src % vl]);
+      if (scale != 1.0f) v = f16_to_f32(f32_to_f16(v * scale));
+      store_from_f32(out, t * dim + j, out_dtype, v);
+    }
+  }
+  return 0;
+}
+
+/*
+ * Group-affine n-bit embedding rows (neuropress/nn/np_embedding.py:120-183 for the decode,
+ * :455-473 and :497-502 for padding row, cast and embed_scale): v = f16((q - zp) * s) computed in
+ * float, zero on the padding row, cast to out_dtype, then times embed_scale rounded to out_dtype.
+ */
+int np_oracle_q_embedding(const int64_t* ids, int64_t n_ids, const uint8_t* blob, const uint16_t* scale,
+                          const uint16_t* zp, int nbits, int64_t group_size, int64_t vocab, int64_t dim,
+                          int64_t padding_idx, float embed_scale, int out_dtype, void* out) {
+  if (!(nbits == 1 || nbits == 2 || nbits == 4 || nbits == 8) || dim % group_size || n_ids < 0) return -1;
+  const int vpb = 8 / nbits;
+  const int64_t row_bytes = dim / vpb, ng = dim / group_size;
+  for (int64_t t = 0; t < n_ids; ++t) {
+    const int64_t tok = ids[t];
+    if (tok < 0 || tok >= vocab) return -2;
+    for (int64_t j = 0; j < dim; ++j) {
+      const int q = (blob[tok * row_bytes + j / vpb] >> ((j % vpb) * nbits)) & ((1 << nbits) - 1);
+      const float z = zp ? f16_to_f32(zp[tok * ng + j / group_size]) : (float)(1 << (nbits - 1));
+      float v = ((float)q - z) * f16_to_f32(scale[tok * ng + j / group_size]);
+      v = f16_to_f32(f32_to_f16(v));
+      if (tok == padding_idx) v = 0.0f;
+      if (out_dtype == NP_BF16) v = bf16_to_f32(f32_to_bf16(v));
+      if (embed_scale != 1.0f) v = v * embed_scale;
+      store_from_f32(out, t * dim + j, out_dtype, v);
     }
   }
   return 0;

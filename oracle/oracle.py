@@ -64,6 +64,12 @@ def _load() -> ctypes.CDLL:
     ]  # fmt: skip
     lib.np_oracle_q_decode.argtypes = [_u8p, _u16p, _u16p, _i64, _i64, _int, _int, _int, _vp]
     lib.np_oracle_linear.argtypes = [_vp, _int, _vp, _int, _vp, _int, _i64, _i64, _i64, _f64p]
+    _i32p = ctypes.POINTER(ctypes.c_int32)
+    lib.np_oracle_rms_norm.argtypes = [_vp, _vp, _int, _i64, _i64, ctypes.c_double, _f64p]
+    lib.np_oracle_vq_embedding.argtypes = [_i64p, _i64, _u16p, _i64, _i64, _u16p, _i64, _i64, _i32p,
+                                           ctypes.c_float, _int, _vp]  # fmt: skip
+    lib.np_oracle_q_embedding.argtypes = [_i64p, _i64, _u8p, _u16p, _u16p, _int, _i64, _i64, _i64, _i64,
+                                          ctypes.c_float, _int, _vp]  # fmt: skip
     lib.np_oracle_f32_to_f16.argtypes = [ctypes.c_float]
     lib.np_oracle_f32_to_f16.restype = ctypes.c_uint16
     lib.np_oracle_f32_to_bf16.argtypes = [ctypes.c_float]
@@ -204,6 +210,54 @@ def q_decode(
     )  # fmt: skip
     _check(rc, "q_decode")
     return out.reshape(n_rows, k_cols)
+
+
+def rms_norm_f64(x_bits: np.ndarray, w_bits: np.ndarray, dtype_code: int, eps: float) -> np.ndarray:
+    """RMSNorm of ``x`` ([M, H], given as dtype bits / float32 values) in double precision."""
+    x = _as_typed(x_bits, dtype_code)
+    w = _as_typed(w_bits, dtype_code)
+    m, h = x.shape
+    out = np.empty((m, h), dtype=np.float64)
+    rc = _load().np_oracle_rms_norm(x.ctypes.data_as(_vp), w.ctypes.data_as(_vp), dtype_code, m, h, float(eps),
+                                    _ptr(out, _f64p))  # fmt: skip
+    _check(rc, "rms_norm")
+    return out
+
+
+def vq_embedding(ids: np.ndarray, indices_u16: np.ndarray, cb_bits: np.ndarray, scale: float,
+                 inv_perm: np.ndarray | None, out_dtype_code: int) -> np.ndarray:  # fmt: skip
+    """Rows of a VQ embedding table as output-dtype bits (float32 values for code 2): ``[n_ids, groups * VL]``."""
+    ids = _c(np.asarray(ids).reshape(-1), np.int64)
+    idx = _c(indices_u16, np.uint16)
+    cb = _c(cb_bits, np.uint16)
+    perm = None if inv_perm is None else _c(np.asarray(inv_perm).reshape(-1), np.int32)
+    vocab, groups = idx.shape
+    nc, vl = cb.shape
+    out = _out_array(ids.size * groups * vl, out_dtype_code)
+    i32p = ctypes.POINTER(ctypes.c_int32)
+    rc = _load().np_oracle_vq_embedding(_ptr(ids, _i64p), ids.size, _ptr(idx, _u16p), vocab, groups, _ptr(cb, _u16p),
+                                        nc, vl, None if perm is None else perm.ctypes.data_as(i32p), float(scale),
+                                        out_dtype_code, out.ctypes.data_as(_vp))  # fmt: skip
+    _check(rc, "vq_embedding")
+    return out.reshape(ids.size, groups * vl)
+
+
+def q_embedding(ids: np.ndarray, blob: np.ndarray, scale_bits: np.ndarray, zp_bits: np.ndarray | None, nbits: int,
+                group_size: int, padding_idx: int | None, embed_scale: float, out_dtype_code: int) -> np.ndarray:  # fmt: skip
+    """Rows of a group-affine n-bit embedding table as output-dtype bits: ``[n_ids, dim]``."""
+    ids = _c(np.asarray(ids).reshape(-1), np.int64)
+    blob = _c(blob, np.uint8)
+    sc = _c(np.asarray(scale_bits).reshape(-1), np.uint16)
+    zp = None if zp_bits is None else _c(np.asarray(zp_bits).reshape(-1), np.uint16)
+    vocab = blob.shape[0]
+    dim = blob.shape[1] * (8 // nbits)
+    out = _out_array(ids.size * dim, out_dtype_code)
+    rc = _load().np_oracle_q_embedding(_ptr(ids, _i64p), ids.size, _ptr(blob, _u8p), _ptr(sc, _u16p),
+                                       _ptr(zp, _u16p), nbits, group_size, vocab, dim,
+                                       -1 if padding_idx is None else padding_idx, float(embed_scale),
+                                       out_dtype_code, out.ctypes.data_as(_vp))  # fmt: skip
+    _check(rc, "q_embedding")
+    return out.reshape(ids.size, dim)
 
 
 def _as_typed(a: np.ndarray, dtype_code: int) -> np.ndarray:
