@@ -44,7 +44,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
-    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "dequant", "q4_gemv_m1", "q4_tile_m128"],
+    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "dequant", "q4_gemv_m1", "q4_tile_m128",
+                                                    "rms_norm_m4096", "vq_embedding_m4096", "q4_embedding_m4096"],
                     help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
                          "on the config-3 / config-5 shape and print a one-line JSON with its HIP-event time")
     ap.add_argument("--ceilings", action="store_true",
@@ -146,7 +147,26 @@ def main():
         n, k = 14336, 4096
         g = gen(1003)
         n_rot = 8
-        if args.case.startswith("q4"):
+        if args.case in ("rms_norm_m4096", "vq_embedding_m4096", "q4_embedding_m4096"):
+            m, hdim, vocab, flops = 4096, 4096, 128256, 0.0
+            if args.case == "rms_norm_m4096":
+                wn = (torch.rand(hdim, generator=g) + 0.5).to(torch.bfloat16).to(dev)
+                pool = [torch.randn(m, hdim, generator=g).to(torch.bfloat16).to(dev) for _ in range(n_rot)]
+                fn = lambda i: kernels.rms_norm(pool[i], wn, 1e-6)
+                alg = 2 * m * hdim * 2 + hdim * 2
+            else:
+                pool = [torch.randint(0, vocab, (m,), generator=g).to(dev) for _ in range(n_rot)]
+                if args.case == "vq_embedding_m4096":
+                    cbe = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.float16).to(dev)
+                    tab = torch.randint(0, 65536, (vocab, hdim // 8), generator=g, dtype=torch.int32).to(torch.int16).to(dev)
+                    fn = lambda i: kernels.vq_embedding(pool[i], tab, cbe, 64.0, None, torch.bfloat16)
+                    alg = m * (8 + hdim // 8 * 2 + hdim // 8 * 16 + hdim * 2)
+                else:
+                    qblob = torch.randint(0, 256, (vocab, hdim // 2), generator=g, dtype=torch.int32).to(torch.uint8).to(dev)
+                    qsc = (torch.rand(vocab * hdim // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
+                    fn = lambda i: kernels.q_embedding(pool[i], qblob, qsc, 4, 32, None, None, 64.0, torch.bfloat16)
+                    alg = m * (8 + hdim // 2 + hdim // 32 * 2 + hdim * 2)
+        elif args.case.startswith("q4"):
             blob = BitPacking4.compress(torch.randint(0, 16, (n, k), generator=g, dtype=torch.int64).to(torch.uint8))
             sc = (torch.rand(n * k // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
             pool = [blob.to(dev).clone() for _ in range(n_rot)]
@@ -404,6 +424,27 @@ def main():
             algq = nn_ * kk // 2 + nn_ * kk // 32 * 2 + m * kk * 2 + m * nn_ * 2
             add("cfg5 int4 14336x4096 f16", "a:gemv" if m <= 16 else "b:tile-gemm", m, t, algq, 2.0 * m * nn_ * kk)
         del blobs
+        torch.cuda.empty_cache()
+        # neighbours of the linear on a decode step: RMSNorm and the embedding lookups (Llama-3-8B sizes)
+        hdim, vocab = 4096, 128256
+        wn = (torch.rand(hdim, generator=g) + 0.5).to(torch.bfloat16).to(dev)
+        for m in (1, 4096):
+            xn = [torch.randn(m, hdim, generator=gen(95 + i)).to(torch.bfloat16).to(dev) for i in range(8 if m > 1 else 2)]
+            t = time_graph(lambda i: kernels.rms_norm(xn[i % len(xn)], wn, 1e-6), len(xn), steps_s * 2, 3, dev)
+            add("rms_norm H=4096 bf16", "aux", m, t, 2 * m * hdim * 2 + hdim * 2, 0.0)
+        cbe = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.float16).to(dev)
+        tab = torch.randint(0, 65536, (vocab, hdim // 8), generator=g, dtype=torch.int32).to(torch.int16).to(dev)
+        qblob = torch.randint(0, 256, (vocab, hdim // 2), generator=g, dtype=torch.int32).to(torch.uint8).to(dev)
+        qsc = (torch.rand(vocab * hdim // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
+        for m in (1, 4096):
+            ids = [torch.randint(0, vocab, (m,), generator=gen(97 + i)).to(dev) for i in range(4)]
+            t = time_graph(lambda i: kernels.vq_embedding(ids[i % 4], tab, cbe, 64.0, None, torch.bfloat16), 4,
+                           steps_s * 2, 3, dev)
+            add("vq_embedding 128256x4096 -> bf16", "aux", m, t, m * (8 + hdim // 8 * 2 + hdim // 8 * 16 + hdim * 2), 0.0)
+            t = time_graph(lambda i: kernels.q_embedding(ids[i % 4], qblob, qsc, 4, 32, None, None, 64.0, torch.bfloat16),
+                           4, steps_s * 2, 3, dev)
+            add("int4 embedding 128256x4096 -> bf16", "aux", m, t, m * (8 + hdim // 2 + hdim // 32 * 2 + hdim * 2), 0.0)
+        del tab, qblob, qsc
         torch.cuda.empty_cache()
     result["sweep"] = sweep
 

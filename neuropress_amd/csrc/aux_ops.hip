@@ -41,12 +41,18 @@ rms_norm_wave_kernel(const uint16_t* __restrict__ x, int64_t ldx, const uint16_t
   if (row >= M) return;
   const int n_vec = H >> 3;
   const uint16_t* xr = x + (int64_t)row * ldx;
-  u32x4 v[NV];
+  u32x4 v[NV], wv[NV];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int p = lane + 64 * i;
     v[i] = p < n_vec ? *reinterpret_cast<const u32x4*>(xr + 8 * p) : u32x4{0, 0, 0, 0};
+  }
+  // the weight does not depend on the reduction: requested now, it arrives while the sum is formed
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int p = lane + 64 * i;
+    wv[i] = p < n_vec ? *reinterpret_cast<const u32x4*>(w + 8 * p) : u32x4{0, 0, 0, 0};
   }
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -64,7 +70,7 @@ rms_norm_wave_kernel(const uint16_t* __restrict__ x, int64_t ldx, const uint16_t
     if (p >= n_vec) continue;
     float f[8], g[8];
     unpack8<DT>(v[i], f);
-    unpack8<DT>(*reinterpret_cast<const u32x4*>(w + 8 * p), g);
+    unpack8<DT>(wv[i], g);
     u32x4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = pack2<DT>(f[2 * e] * scale * g[2 * e], f[2 * e + 1] * scale * g[2 * e + 1]);
@@ -257,10 +263,28 @@ q4_embedding_kernel(const int64_t* __restrict__ ids, int64_t n_ids, const uint8_
   const float s = f16_bits_to_f32(scale[grp]);
   const float z = zp ? f16_bits_to_f32(zp[grp]) : 8.0f;
   const bool pad = raw == padding_idx;
+  if constexpr (OUT == NPAMD_F32) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float q = (float)((codes >> (4 * e)) & 0xFu);
-    store_q_embedding<OUT>(out, i * 8 + e, pad ? 0.f : (q - z) * s, embed_scale, scaled);
+    for (int e = 0; e < 8; ++e) {
+      const float q = (float)((codes >> (4 * e)) & 0xFu);
+      store_q_embedding<OUT>(out, i * 8 + e, pad ? 0.f : (q - z) * s, embed_scale, scaled);
+    }
+  } else {
+    // eight 16-bit results leave as one 16-byte store; same roundings as store_q_embedding
+    uint32_t r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float q = (float)((codes >> (4 * e)) & 0xFu);
+      const uint32_t h = f32_to_f16_bits(pad ? 0.f : (q - z) * s);
+      if constexpr (OUT == NPAMD_F16) {
+        r[e] = scaled ? f32_to_f16_bits(f16_bits_to_f32(h) * embed_scale) : h;
+      } else {
+        const uint32_t b = f32_to_bf16_bits(f16_bits_to_f32(h));
+        r[e] = scaled ? f32_to_bf16_bits(bf16_bits_to_f32(b) * embed_scale) : b;
+      }
+    }
+    *reinterpret_cast<u32x4*>((uint16_t*)out + i * 8) =
+        u32x4{r[0] | (r[1] << 16), r[2] | (r[3] << 16), r[4] | (r[5] << 16), r[6] | (r[7] << 16)};
   }
 }
 
@@ -290,7 +314,8 @@ int launch_q_embedding(const int64_t* ids, int64_t n_ids, const uint8_t* w_pack,
                        const uint16_t* zp, int nbits, int group_size, int64_t vocab, int dim, int64_t padding_idx,
                        float embed_scale, void* out, hipStream_t st) {
   const bool scaled = embed_scale != 1.0f;
-  if (nbits == 4 && group_size % 8 == 0 && dim % 8 == 0 && (reinterpret_cast<uintptr_t>(w_pack) & 3) == 0) {
+  if (nbits == 4 && group_size % 8 == 0 && dim % 8 == 0 && (reinterpret_cast<uintptr_t>(w_pack) & 3) == 0 &&
+      aligned16(out)) {
     const int64_t n = n_ids * (dim / 8);
     q4_embedding_kernel<OUT><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(ids, n_ids, w_pack, scale, zp, group_size,
                                                                           vocab, dim, padding_idx, embed_scale, scaled,

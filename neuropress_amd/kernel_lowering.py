@@ -6,9 +6,9 @@ Same surface as the reference (neuropress/kernel_lowering.py:43-368):
 norm_backend).apply(model)`` / ``.from_config(src)``, ``is_lowered`` and
 ``unlower_model``.
 
-Only the two linear paths are lowered here.  ``embedding_backend`` and
-``norm_backend`` are accepted (so existing configs load) and ignored:
-quantized embeddings and RMSNorm fusion are outside this backend.
+``apply`` lowers, in the reference's order (kernel_lowering.py:200-219): scalar-quantized
+embeddings, scalar-quantized linears, VQ linears, VQ embeddings and - with ``norm_backend``
+``"auto"`` or ``"cuda"`` - the RMSNorms that live on a GPU.
 """
 
 from __future__ import annotations
@@ -106,11 +106,17 @@ class AutoKernelLowering(KernelLowering):
         )
 
     def apply(self, model: nn.Module) -> None:
+        from .nn.np_embedding import NPEmbedding, linearize_qtensor_embeddings
         from .nn.np_linear import NPLinear, linearize_qtensor_weights
+        from .nn.np_rms_norm import linearize_rms_norms
+        from .nn.np_vq_embedding import NPVQEmbedding, linearize_vq_embeddings
         from .nn.np_vq_linear import NPVQLinear, linearize_vq_weights
 
+        linearize_qtensor_embeddings(model, backend=self.embedding_backend)
         linearize_qtensor_weights(model, backend=self.linear_backend)
         linearize_vq_weights(model, backend=self.vq_backend)
+        linearize_vq_embeddings(model)
+        n_norms = linearize_rms_norms(model) if self.norm_backend in ("auto", "cuda") else 0
 
         # A lowered lm_head no longer shares storage with the embedding table:
         # keep later tie_weights() calls from trying to re-tie (kernel_lowering.py:221-227).
@@ -123,9 +129,15 @@ class AutoKernelLowering(KernelLowering):
                 key = f"NPLinear({m.backend.value})"
             elif isinstance(m, NPVQLinear):
                 key = f"NPVQLinear({m.backend.value})"
+            elif isinstance(m, NPEmbedding):
+                key = f"NPEmbedding({m.backend.value})"
+            elif isinstance(m, NPVQEmbedding):
+                key = "NPVQEmbedding"
             else:
                 continue
             counts[key] = counts.get(key, 0) + 1
+        if n_norms:
+            counts["NPRMSNorm"] = n_norms
         if counts:
             summary = ", ".join(f"{v}x {k}" for k, v in sorted(counts.items()))
             LOGGER.warning("Kernel lowering applied: %s", summary)
@@ -134,11 +146,15 @@ class AutoKernelLowering(KernelLowering):
 
 
 def is_lowered(model: nn.Module) -> bool:
-    """True if *model* contains any lowered linear module."""
+    """True if *model* contains any lowered linear, embedding or norm module (kernel_lowering.py:252-277)."""
+    from .nn.np_embedding import NPEmbedding
     from .nn.np_linear import NPLinear
+    from .nn.np_rms_norm import NPRMSNorm
+    from .nn.np_vq_embedding import NPVQEmbedding
     from .nn.np_vq_linear import NPVQLinear
 
-    return any(isinstance(m, (NPLinear, NPVQLinear)) for m in model.modules())
+    lowered = (NPLinear, NPVQLinear, NPEmbedding, NPVQEmbedding, NPRMSNorm)
+    return any(isinstance(m, lowered) for m in model.modules())
 
 
 def unlower_model(model: nn.Module) -> None:
@@ -149,12 +165,30 @@ def unlower_model(model: nn.Module) -> None:
     weight is ever materialised).  Codebook proxies registered on the model root
     are removed.
     """
+    from .nn.np_embedding import NPEmbedding
     from .nn.np_linear import NPLinear
+    from .nn.np_rms_norm import NPRMSNorm
+    from .nn.np_vq_embedding import NPVQEmbedding
     from .nn.np_vq_linear import NPVQLinear
     from .qweights import attach_quantized_weight
 
     replacements: list[tuple[str, nn.Module]] = []
     for name, module in model.named_modules():
+        if isinstance(module, NPRMSNorm):
+            source = module.to_source_module()
+            if source is not None:
+                replacements.append((name, source))
+            continue
+        if isinstance(module, (NPEmbedding, NPVQEmbedding)):
+            vocab = module.num_embeddings if isinstance(module, NPEmbedding) else module.all_indices.shape[0]
+            with torch.device("meta"):
+                emb = nn.Embedding(vocab, module.embedding_dim, padding_idx=getattr(module, "padding_idx", None))
+            attach_quantized_weight(emb, module.to_qtensor())
+            scale = module.embed_scale if isinstance(module, NPEmbedding) else module.scale
+            if scale != 1.0:
+                emb.embed_scale = scale  # read back by the next lowering (and by scaled-embedding classes)
+            replacements.append((name, emb))
+            continue
         if not isinstance(module, (NPLinear, NPVQLinear)):
             continue
         qweight = module.to_qtensor()
@@ -174,7 +208,8 @@ def unlower_model(model: nn.Module) -> None:
             parent, attr = model, name
         setattr(parent, attr, new_mod)
 
-    for pname in [n for n, _ in model.named_children() if n.startswith(("_vq_proxy_", "_vq_res_proxy_"))]:
+    for pname in [n for n, _ in model.named_children()
+                  if n.startswith(("_vq_proxy_", "_vq_res_proxy_", "_vq_emb_proxy_"))]:  # fmt: skip
         delattr(model, pname)
     LOGGER.info("unlower_model: restored %d module(s) to quantized-weight form", len(replacements))
 

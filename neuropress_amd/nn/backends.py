@@ -79,6 +79,23 @@ class LinearBackend(_StrEnum):
     GEMLITE = "gemlite"
 
 
+class EmbeddingBackend(_StrEnum):
+    """Valid backends for scalar-quantized ``nn.Embedding`` (:class:`.NPEmbedding`)."""
+
+    AUTO = "auto"
+    DEFAULT = "default"
+    COMPILE = "compile"
+    CUDA = "cuda"
+
+
+class NormBackend(_StrEnum):
+    """Valid backends for RMSNorm modules (:class:`.NPRMSNorm`)."""
+
+    AUTO = "auto"
+    DEFAULT = "default"
+    CUDA = "cuda"
+
+
 class VQBackend(_StrEnum):
     """Valid backends for vector-quantized ``nn.Linear`` (:class:`.NPVQLinear`)."""
 

@@ -33,7 +33,7 @@ residual VQ layers, components ``residual_blob`` / ``residual_centroids`` / ``ro
 ``row_bias`` with metadata ``residual_bits``.
 
 The weights handled are the containers of :mod:`neuropress_amd.qweights` (and anything with the
-same attributes), found as the ``.weight`` of ``nn.Linear`` modules.  A kernel-lowered model is
+same attributes), found as the ``.weight`` of ``nn.Linear`` and ``nn.Embedding`` modules.  A kernel-lowered model is
 unlowered for the save and lowered again afterwards, as in the reference.
 """
 
@@ -266,10 +266,10 @@ _KNOWN_TYPES = ("QTensorTractVQ", "QTensorTractScaleOnly", "QTensorScaleZp")
 
 
 def _quantized_weights(model: nn.Module) -> dict[str, Any]:
-    """``{param_path: weight}`` for every ``nn.Linear`` whose weight is a quantized container."""
+    """``{param_path: weight}`` for every ``nn.Linear`` / ``nn.Embedding`` whose weight is a quantized container."""
     found = {}
     for name, module in model.named_modules():
-        if isinstance(module, nn.Linear):
+        if isinstance(module, (nn.Linear, nn.Embedding)):
             w = module.__dict__.get("weight", None)
             if w is None:
                 w = module._parameters.get("weight")
@@ -388,8 +388,8 @@ def load_quantized_model(model: nn.Module, path: str | Path, kernel_lowering: st
             )
         module_path, _, attr = param_path.rpartition(".")
         module = model.get_submodule(module_path) if module_path else model
-        if attr != "weight" or not isinstance(module, nn.Linear):
-            raise ValueError(f"quantized parameter {param_path!r} is not the weight of an nn.Linear")
+        if attr != "weight" or not isinstance(module, (nn.Linear, nn.Embedding)):
+            raise ValueError(f"quantized parameter {param_path!r} is not the weight of an nn.Linear / nn.Embedding")
         device = next((t.device for t in list(module.parameters()) + list(module.buffers())
                        if t.device.type != "meta"), torch.device("cpu"))  # fmt: skip
         parts = {k: all_tensors[f"{param_path}{_QT_SEP}{k}"].to(device) for k in entry["tensor_keys"]}
