@@ -104,3 +104,35 @@ def test_q_dequant_in_a_graph(gpu):
     mk = lambda i: [BitPacking4.compress(
         torch.randint(0, 16, (64, 256), generator=cases.gen(600 + i), dtype=torch.int64).to(torch.uint8)).to(gpu)]
     _capture_and_replay(gpu, lambda inp: kernels.q_dequant(inp[0], sc, 4, 32, None, torch.float16), mk)
+
+
+def test_split_k_tile_gemm_and_permuted_gemv_in_a_graph(gpu):
+    """The tile GEMM with a workspace (K split over blockIdx.z plus its reduction kernel) and the GEMV
+    that gathers x[..., column_perm] itself."""
+    from neuropress_amd import kernels
+
+    L = cases.vq_layer(14, 128, 4096, 4096, bits=12, act=torch.float16, m=24, bias=True, std=0.02)
+    packed, cb, bias = L["packed"].to(gpu), L["cb"].to(gpu), L["bias"].to(gpu)
+    mk = lambda i: [torch.randn(24, 4096, generator=cases.gen(500 + i)).half().to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.vq_gemm_tile(inp[0], packed, cb, 12, 128, bias), mk)
+    perm = torch.randperm(4096, generator=cases.gen(1)).to(torch.int32).to(gpu)
+    mk2 = lambda i: [torch.randn(2, 4096, generator=cases.gen(600 + i)).half().to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.vq_linear(inp[0], packed, cb, 12, 8, bias, 128, column_perm=perm), mk2)
+
+
+def test_rms_norm_and_embedding_lookups_in_a_graph(gpu):
+    from neuropress_amd import kernels
+    from neuropress_amd.t2n.packing import BitPacking4
+
+    g = cases.gen(15)
+    w = (torch.rand(512, generator=g) + 0.5).to(torch.bfloat16).to(gpu)
+    mk = lambda i: [torch.randn(9, 512, generator=cases.gen(700 + i)).to(torch.bfloat16).to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.rms_norm(inp[0], w, 1e-6), mk)
+    cb = (torch.randn(4096, 8, generator=g) * 0.05).half().to(gpu)
+    tab = torch.randint(0, 4096, (300, 64), generator=g).to(torch.int16).to(gpu)
+    inv = torch.argsort(torch.randperm(512, generator=g)).to(torch.int32).to(gpu)
+    mk_ids = lambda i: [torch.randint(0, 300, (4, 5), generator=cases.gen(800 + i)).to(gpu)]
+    _capture_and_replay(gpu, lambda inp: kernels.vq_embedding(inp[0], tab, cb, 22.6, inv, torch.bfloat16), mk_ids)
+    blob = BitPacking4.compress(torch.randint(0, 16, (300, 512), generator=g, dtype=torch.int64).to(torch.uint8)).to(gpu)
+    sc = (torch.rand(300 * 16, generator=g) * 0.02 + 0.001).half().to(gpu)
+    _capture_and_replay(gpu, lambda inp: kernels.q_embedding(inp[0], blob, sc, 4, 32, None, 7, 22.6, torch.float16), mk_ids)
