@@ -35,7 +35,14 @@ def _dt(dtype: torch.dtype, what: str) -> int:
         raise RuntimeError(f"{what}: dtype must be bfloat16, float16 or float32, got {dtype}") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """Handle of torch's current stream on ``t``'s device (the raw query costs a few tenths of a
+    microsecond, ``torch.cuda.current_stream`` about four)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.get_device())
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
