@@ -72,3 +72,38 @@ def test_slice_lists_always_decode_to_their_input(n, groups, nc, target, seed, s
     dec, info = cases.decode_sliced_blob(blob.numpy())
     assert np.array_equal(dec, idx.reshape(n, groups).numpy())
     assert (info["hits"] == 1).all() and (info["writes"] == 1).all()
+
+
+@st.composite
+def _skewed_indices(draw):
+    """Index lists the prefix codes are meant for: mostly small values, a few anywhere in range."""
+    top_bits = draw(st.integers(9, 20))
+    n = draw(st.integers(0, 90))
+    small = st.integers(0, 300)
+    anywhere = st.integers(0, (1 << top_bits) - 1)
+    return top_bits, draw(st.lists(st.one_of(small, small, anywhere), min_size=n, max_size=n))
+
+
+@settings(max_examples=120, deadline=None)
+@given(_skewed_indices(), st.sampled_from([4, 6, 8]), st.integers(0, 2))
+def test_prefix_coded_formats_round_trip_and_agree_with_the_oracle(oracle_lib, case, hot_bits, extra_tiers):
+    """pack -> unpack is the identity for all three prefix-coded formats, on the host classes and
+    through the oracle's sequential decoders, and the per-row tier counts add up."""
+    from neuropress_amd.transforms.vq_packing import NTieredIndexPacking, TieredIndexPacking, ZeroEscapePacking
+    from oracle import oracle as orc
+
+    top_bits, idx = case
+    t = torch.tensor(idx, dtype=torch.int64)
+    tier_bits = sorted({hot_bits, *[hot_bits + 3 * (i + 1) for i in range(extra_tiers)], top_bits})
+    if len(tier_bits) < 2:
+        tier_bits = [4, top_bits]
+    for kind, buf, unpack in (
+        ("tiered", TieredIndexPacking.pack(t, top_bits, hot_bits), TieredIndexPacking.unpack),
+        ("ntier", NTieredIndexPacking.pack(t, tier_bits), NTieredIndexPacking.unpack),
+        ("zero_escape", ZeroEscapePacking.pack(t, top_bits), ZeroEscapePacking.unpack),
+    ):
+        assert unpack(buf).tolist() == idx, kind
+        assert orc.entropy_unpack(kind, buf.numpy()).tolist() == idx, kind
+    if idx:
+        offs = NTieredIndexPacking.compute_row_offsets(NTieredIndexPacking.pack(t, tier_bits), 1, len(idx))
+        assert sum(int(o[1]) for o in offs) == len(idx)
