@@ -272,6 +272,16 @@ def test_cfg3_down_proj_shape(gpu):
     ref = x.float() @ w.float().T
     _close(kernels.vq_linear(x, packed, cb, 16, 8, None, 4096), ref)
     _close(kernels.vq_gemm_tile(x, packed, cb, 16, 4096), ref)
+    # mid token counts: 64 column blocks do not fill the GPU, so the reduction is split (workspace in
+    # use); the split changes the summation order only, and rows stay independent of each other
+    from neuropress_amd import _lib
+
+    for m in (64, 384):
+        assert _lib.load().npamd_gemm_tile_workspace_bytes(m, 4096, 14336) > 0
+        xm = torch.randn(m, 14336, generator=cases.gen(m)).bfloat16().to(gpu)
+        ym = kernels.vq_gemm_tile(xm, packed, cb, 16, 4096)
+        _close(ym, xm.float() @ w.float().T)
+        assert torch.equal(kernels.vq_gemm_tile(xm[: m // 2].contiguous(), packed, cb, 16, 4096), ym[: m // 2])
 
 
 def test_cfg5_q4_full_size(gpu):
