@@ -353,6 +353,26 @@ def test_c_abi_validates_arguments_without_a_gpu():
     with pytest.raises(RuntimeError, match="exceeds the fused limit"):
         _lib.call("npamd_vq_gemv", None, 64, None, 1 << 20, 8, None, 0, 16, 8, None, None, 4, 17, 4, 64, 0, None)
     _lib.call("npamd_vq_dequant", None, 0, 8, None, 16, 8, 0, None, 0, None)  # empty: success, no launch
+    # entry points added around the path: same rule
+    with pytest.raises(RuntimeError, match="row stride smaller than the row"):
+        _lib.call("npamd_rms_norm", None, 8, None, None, 16, 2, 16, 1e-6, 0, None)
+    with pytest.raises(RuntimeError, match="bad dtype code"):
+        _lib.call("npamd_rms_norm", None, 16, None, None, 16, 2, 16, 1e-6, 7, None)
+    _lib.call("npamd_rms_norm", None, 16, None, None, 16, 0, 16, 1e-6, 0, None)  # no rows: success, no launch
+    with pytest.raises(RuntimeError, match="16-bit indices"):
+        _lib.call("npamd_vq_embedding", None, 1, None, 10, 4, None, 70000, 8, None, 1.0, None, 0, None)
+    with pytest.raises(RuntimeError, match="null pointer"):
+        _lib.call("npamd_vq_embedding", None, 1, None, 10, 4, None, 256, 8, None, 1.0, None, 0, None)
+    with pytest.raises(RuntimeError, match="nbits must be 1, 2, 4 or 8"):
+        _lib.call("npamd_q_embedding", None, 1, None, None, None, 3, 32, 10, 64, -1, 1.0, None, 0, None)
+    with pytest.raises(RuntimeError, match="bad shape"):
+        _lib.call("npamd_q_embedding", None, 1, None, None, None, 4, 48, 10, 64, -1, 1.0, None, 0, None)
+    with pytest.raises(RuntimeError, match="column_perm needs"):
+        _lib.call("npamd_vq_gemv_perm", 16, 8192, 16, 16, 1 << 20, 16, 16, 0, 65536, 8, None, 16, 64, 9, 64, 8192, 0, None)
+    lib = _lib.load()
+    assert lib.npamd_vq_gemv_perm_supported(1, 2048, 2048, 4096, 8, 12) == 1
+    assert lib.npamd_vq_gemv_perm_supported(1, 2048, 2048, 4096, 4, 12) == 0  # vector length 4
+    assert lib.npamd_vq_gemv_perm_supported(5, 2048, 4096, 4096, 8, 12) == 0  # 5 * 4096 elements > 16384
 
 
 def test_tile_band_rule_counts_reduction_splits():
