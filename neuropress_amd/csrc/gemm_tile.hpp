@@ -18,13 +18,17 @@
 //
 // Both operands are staged in LDS, rows padded to 144 bytes so 16-byte reads of
 // 32 consecutive rows are bank-conflict free:
-//   x tile  [BM][64 k], double buffered, loaded coalesced by the consumers one
-//           step ahead through registers;
-//   W tile  [64][64 k], double buffered.  Every producer decodes a quarter of
+//   x tile  [BM][64 k], double buffered.  Every consumer loads and stores only
+//           the rows it owns (coalesced, through registers, one or more steps
+//           ahead), so the x tile needs no synchronisation between waves.
+//   W tile  [64][64 k], a ring of three.  Every producer decodes a quarter of
 //           every step's tile (16 columns x 8 operands; lane = column x
 //           operand pair), keeps kDepth steps in flight in registers and
-//           writes a finished pair to LDS one iteration before its step.
-// One block barrier per macro-step, executed by all eight waves.
+//           writes a finished pair to LDS two iterations before its step.
+// One block barrier per macro-step, executed by all eight waves.  Because the
+// W tile of step t+1 is complete at the barrier that ends iteration t-1, a
+// consumer fetches the first operands of step t+1 during the last MFMAs of
+// step t: the matrix pipe does not drain across the barrier.
 //
 // Layers with few output columns (N = 4096: 64 column blocks) would leave most
 // compute units idle, and the decode rate per compute unit is the limit; for
@@ -41,6 +45,7 @@ constexpr int kStepK = 64;                      // k per macro-step (= one chunk
 constexpr int kRowBytes = kStepK * 2 + 16;      // padded LDS row stride
 constexpr int kTileCols = 64;                   // output columns per block
 constexpr int kWBufBytes = kTileCols * kRowBytes;
+constexpr int kWRing = 3;                       // W tiles in LDS: read, complete, being written
 
 struct GemmShape {
   const void* x;
@@ -77,7 +82,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   constexpr int kXBufBytes = BM * kRowBytes;
   constexpr int kPieces = BM * (kStepK / 8) / 256;  // 16-byte pieces of the x tile per consumer thread
   uint8_t* const xs = lds;                     // [2][BM][kRowBytes]
-  uint8_t* const ws = lds + 2 * kXBufBytes;    // [2][64][kRowBytes]
+  uint8_t* const ws = lds + 2 * kXBufBytes;    // [kWRing][64][kRowBytes]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -130,33 +135,39 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     auto load_raw = [&](typename Provider::PairRaw& raw, int step) {
       prov.load_pair(raw, ncol, chunk_of(min(step, steps - 1)), jp);
     };
-    auto store_w = [&](const u32x4 (&b)[2], int step) {
-      uint8_t* dst = ws + (step & 1) * kWBufBytes + col * kRowBytes + jp * 32;
+    auto store_w = [&](const u32x4 (&b)[2], int slot) {
+      uint8_t* dst = ws + slot * kWBufBytes + col * kRowBytes + jp * 32;
       *reinterpret_cast<u32x4*>(dst) = b[0];
       *reinterpret_cast<u32x4*>(dst + 16) = b[1];
     };
-    auto advance = [&](u32x4 (&b)[2], typename Provider::PairRaw& raw, int t) {
-      store_w(b, t + 1);
+    // Iteration t: the operands of step t+2 (gathered kDepth iterations ago) go to ring slot
+    // (t+2) % 3, their registers are refilled with the gathers of step t+2+kDepth, and the
+    // packed bytes of step t+2+2*kDepth are requested.
+    auto advance = [&](u32x4 (&b)[2], typename Provider::PairRaw& raw, int t, int slot) {
+      store_w(b, slot);
       prov.operand_pair(raw, b[0], b[1]);
-      load_raw(raw, t + 1 + 2 * kDepth);
+      load_raw(raw, t + 2 + 2 * kDepth);
     };
 
-    // Prologue: steps 0..kDepth-1 in flight, packed bytes of kDepth..2*kDepth-1
-    // loaded; then "iteration -1": store step 0 and refill its registers.
+    // Prologue: steps 0..kDepth-1 in flight, packed bytes of kDepth..2*kDepth-1 loaded; then
+    // "iterations -2 and -1": store steps 0 and 1 and refill their registers.
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p);
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) prov.operand_pair(raws[p], ops[p][0], ops[p][1]);
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p + kDepth);
-    advance(ops[0], raws[0], -1);
+    advance(ops[0], raws[0], -2, 0);
+    advance(ops[1], raws[1], -1, 1);
     block_sync_lds();
 
-    // Iteration t handles step t+1, which lives in register set (t+1) % kDepth.
+    // Iteration t handles step t+2, which lives in register set (t+2) % kDepth.
+    int slot = 2;
     for (int t0 = 0; t0 < total; t0 += kDepth) {
 #pragma unroll
       for (int d = 0; d < kDepth; ++d) {
-        advance(ops[(d + 1) % kDepth], raws[(d + 1) % kDepth], t0 + d);
+        advance(ops[(d + 2) % kDepth], raws[(d + 2) % kDepth], t0 + d, slot);
+        slot = slot == kWRing - 1 ? 0 : slot + 1;
         block_sync_lds();
       }
     }
@@ -167,7 +178,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   const int c = lane & 31;
   const int h = lane >> 5;
   const int wrow0 = wave * (32 * MW);              // first tile row of this wave
-  const bool wave_active = (m0 + wrow0) < s.M;     // waves past M still load x and keep the barriers
+  const bool wave_active = (m0 + wrow0) < s.M;     // waves past M compute on clamped rows and never store
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(s.x);
 
   f32x16 acc[MW][2];
@@ -178,62 +189,101 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
 
-  auto load_x = [&](u32x4 (&xr)[kPieces], int step) {
-#pragma unroll
-    for (int i = 0; i < kPieces; ++i) {
-      const int p = tid + i * 256;
-      const int row = p >> 3, col8 = p & 7;
-      const int m = min(m0 + row, s.M - 1);  // rows past M: clamped, never stored
-      xr[i] = *reinterpret_cast<const u32x4*>(xg + (int64_t)m * s.ldx + chunk_of(step) * kStepK + col8 * 8);
-      if constexpr (Provider::kPermuteA) xr[i] = permute_a_0415(xr[i]);
-    }
+  // The wave's own rows of the x tile: piece i of lane l is row wrow0 + (l >> 3) + 8 i, 16-byte
+  // column l & 7 (eight rows of 128 bytes per load instruction).
+  constexpr int kPiecesW = 4 * MW;
+  const int prow = lane >> 3, pcol8 = lane & 7;
+  auto x_src = [&](int i, int step) {
+    const int m = min(m0 + wrow0 + prow + 8 * i, s.M - 1);  // rows past M: clamped, never stored
+    return reinterpret_cast<const u32x4*>(xg + (int64_t)m * s.ldx + chunk_of(min(step, steps - 1)) * kStepK + pcol8 * 8);
   };
-  auto store_x = [&](const u32x4 (&xr)[kPieces], int buf) {
-#pragma unroll
-    for (int i = 0; i < kPieces; ++i) {
-      const int p = tid + i * 256;
-      const int row = p >> 3, col8 = p & 7;
-      *reinterpret_cast<u32x4*>(xs + buf * kXBufBytes + row * kRowBytes + col8 * 16) = xr[i];
-    }
+  auto x_dst = [&](int i, int buf) {
+    return reinterpret_cast<u32x4*>(xs + buf * kXBufBytes + (wrow0 + prow + 8 * i) * kRowBytes + pcol8 * 16);
   };
-  auto mma = [&](int step) {
-    const uint8_t* xa = xs + (step & 1) * kXBufBytes + (wrow0 + c) * kRowBytes + h * 64;
-    const uint8_t* wb = ws + (step & 1) * kWBufBytes + c * kRowBytes + h * 64;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const u32x4 b0 = *reinterpret_cast<const u32x4*>(wb + j * 16);
-      const u32x4 b1 = *reinterpret_cast<const u32x4*>(wb + 32 * kRowBytes + j * 16);
-#pragma unroll
-      for (int mt = 0; mt < MW; ++mt) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(xa + mt * 32 * kRowBytes + j * 16);
-        acc[mt][0] = mfma32<ACT>(a, b0, acc[mt][0]);
-        acc[mt][1] = mfma32<ACT>(a, b1, acc[mt][1]);
-      }
-    }
+  // A provider that wants the k order of its A operands changed gets it at the LDS store, when
+  // the loaded value has long arrived (at the load, the shuffle would wait for it on the spot).
+  auto load_piece = [&](u32x4& r, int i, int step) { r = *x_src(i, step); };
+  auto store_piece = [&](const u32x4& r, int i, int buf) {
+    if constexpr (Provider::kPermuteA) *x_dst(i, buf) = permute_a_0415(r);
+    else *x_dst(i, buf) = r;
   };
 
-  // x tile pipeline: kXDepth register sets hold the tiles of the next steps in
-  // flight (a global load takes longer than one iteration).  Step p lives in
-  // set p % kXDepth; iteration t writes tile t+1 to LDS and reloads its set
-  // with tile t+1+kXDepth.
-  constexpr int kXDepth = (MW == 1) ? 4 : 2;  // divides kDepth, so `total` suits both loops
-  u32x4 xr[kXDepth][kPieces];
-  load_x(xr[0], 0);
-  store_x(xr[0], 0);
+  // x tile pipeline: kXDepth register sets hold the tiles of the next steps in flight (a global
+  // load takes longer than one iteration).  Step p lives in set p % kXDepth; iteration t writes
+  // tile t+1 to LDS and reloads its set with tile t+1+kXDepth.
+  constexpr int kXDepth = (MW == 1) ? 4 : (MW == 2) ? 2 : 1;
+  u32x4 xr[kXDepth][kPiecesW];
 #pragma unroll
-  for (int p = 1; p <= kXDepth; ++p) load_x(xr[p % kXDepth], min(p, steps - 1));
+  for (int i = 0; i < kPiecesW; ++i) {
+    load_piece(xr[0][i], i, 0);
+    store_piece(xr[0][i], i, 0);
+  }
+#pragma unroll
+  for (int p = 1; p <= kXDepth; ++p)
+#pragma unroll
+    for (int i = 0; i < kPiecesW; ++i) load_piece(xr[p % kXDepth][i], i, p);
   block_sync_lds();
 
-  for (int t0 = 0; t0 < total; t0 += kXDepth) {
+  // Operand registers, two sets: the MFMAs of k group j read set j & 1 while the reads of the
+  // next group fill the other; group 0 of the next step takes the place of "group 4".
+  u32x4 a[2][MW], b[2][2];
+  auto read_ops = [&](int set, int step, int wslot, int j) {
+    const uint8_t* xa = xs + (step & 1) * kXBufBytes + (wrow0 + c) * kRowBytes + h * 64 + j * 16;
+    const uint8_t* wb = ws + wslot * kWBufBytes + c * kRowBytes + h * 64 + j * 16;
+    b[set][0] = *reinterpret_cast<const u32x4*>(wb);
+    b[set][1] = *reinterpret_cast<const u32x4*>(wb + 32 * kRowBytes);
+#pragma unroll
+    for (int mt = 0; mt < MW; ++mt) a[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * kRowBytes);
+  };
+  // Pieces of tile step+1 stored (and refilled with tile step+1+kXDepth) behind the MFMAs of k
+  // groups 0..2, so that all of them are in LDS before group 3 fetches the next step's operands.
+  constexpr int kPieceOfGroup[4] = {0, (kPiecesW + 2) / 3, (2 * kPiecesW + 2) / 3, kPiecesW};
+
+  auto one_step = [&](u32x4 (&set)[kPiecesW], int step, int wslot) {
+    const int wnext = wslot == kWRing - 1 ? 0 : wslot + 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (j < 3) read_ops((j + 1) & 1, step, wslot, j + 1);
+      else read_ops(0, step + 1, wnext, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < MW; ++mt) {
+        acc[mt][0] = mfma32<ACT>(a[j & 1][mt], b[j & 1][0], acc[mt][0]);
+        acc[mt][1] = mfma32<ACT>(a[j & 1][mt], b[j & 1][1], acc[mt][1]);
+      }
+      if (j < 3) {
+#pragma unroll
+        for (int i = kPieceOfGroup[j]; i < kPieceOfGroup[j + 1]; ++i) {
+          store_piece(set[i], i, (step + 1) & 1);
+          load_piece(set[i], i, step + 1 + kXDepth);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  read_ops(0, 0, 0, 0);
+  int wslot = 0;
+  const int whole = steps / kXDepth * kXDepth;
+  for (int t0 = 0; t0 < whole; t0 += kXDepth) {
 #pragma unroll
     for (int d = 0; d < kXDepth; ++d) {
-      const int step = t0 + d;
-      store_x(xr[(d + 1) % kXDepth], (step + 1) & 1);
-      load_x(xr[(d + 1) % kXDepth], min(step + 1 + kXDepth, steps - 1));
-      if (wave_active && step < steps) mma(step);
+      one_step(xr[(d + 1) % kXDepth], t0 + d, wslot);
+      wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
       block_sync_lds();
     }
   }
+  // Fewer than kXDepth real steps are left (their register sets are still indexed statically),
+  // then the padding iterations, which only keep the producers' barriers company.
+#pragma unroll
+  for (int d = 0; d < kXDepth; ++d) {
+    if (whole + d < steps) {
+      one_step(xr[(d + 1) % kXDepth], whole + d, wslot);
+      wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
+      block_sync_lds();
+    }
+  }
+  for (int t = steps; t < total; ++t) block_sync_lds();
 
   // ---- epilogue: D[m = 8*(i/4) + 4h + i%4][n = c] --------------------------
   if (!wave_active) return;
@@ -292,7 +342,7 @@ int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs
                         const char* what) {
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
-  const int lds = 2 * BM * kRowBytes + 2 * kWBufBytes;
+  const int lds = 2 * BM * kRowBytes + kWRing * kWBufBytes;
   static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
   if (!attr_set) {
     const hipError_t e = hipFuncSetAttribute(
