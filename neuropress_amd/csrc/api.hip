@@ -67,9 +67,11 @@ GemvPlan plan_gemv(int N, int chunks) {
   int jpw = (int)((jobs + target_waves - 1) / target_waves);
   if (jpw < 1) jpw = 1;
   GemvPlan p;
-  // Two row tiles per block share the x operands, but only while that still
-  // leaves at least one block per compute unit.
-  p.R = (jpw >= 2 && tiles >= 2 * cus) ? 2 : 1;
+  // Row tiles of one block share the x operands (every block reads all of x, from L2: with R
+  // tiles per block that traffic, which passes the weight bytes at a few tokens, drops R-fold)
+  // and one copy of the codebook in LDS.  The largest R that leaves blocks for at least 0.6 of
+  // the compute units wins at every token count, measured on N = 2048 ... 28672.
+  p.R = (tiles * 10 >= cus * 24) ? 4 : (tiles * 10 >= cus * 12) ? 2 : 1;
   int spw = (jpw + p.R - 1) / p.R;
   const int r_env = env_int("NPAMD_GEMV_R", 0);
   if (r_env == 1 || r_env == 2 || r_env == 4) p.R = r_env;

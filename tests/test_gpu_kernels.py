@@ -166,8 +166,11 @@ def test_vq_gemv_column_perm_limits(gpu):
     L = cases.vq_layer(41, 64, 4096, 256, bits=8, act=torch.float16, m=9)  # 9 * 4096 > 16384 elements
     perm = torch.randperm(4096, generator=cases.gen(1)).to(torch.int32).to(gpu)
     assert not kernels.vq_linear_perm_supported(9, 64, 4096, 256, 8, 8)
-    assert kernels.vq_linear_perm_supported(1, 14336, 4096, 4096, 8, 16)  # 73 KiB of LDS: two blocks per CU
-    assert not kernels.vq_linear_perm_supported(2, 14336, 4096, 4096, 8, 16)  # 82 KiB: one block per CU
+    # 28672 rows are more blocks than compute units: the permuted kernel must leave room for two per CU.
+    assert kernels.vq_linear_perm_supported(1, 28672, 4096, 4096, 8, 16)      # 74 KiB of LDS
+    assert not kernels.vq_linear_perm_supported(2, 28672, 4096, 4096, 8, 16)  # 98 KiB
+    # 14336 rows are fewer blocks (of four row tiles) than compute units: one per CU either way.
+    assert kernels.vq_linear_perm_supported(2, 14336, 4096, 4096, 8, 16)
     with pytest.raises(RuntimeError, match="column_perm needs"):
         kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), 8, 8, None, 64, column_perm=perm)
     with pytest.raises(RuntimeError, match="int32"):
@@ -294,6 +297,36 @@ def test_q4_linear_fast_path(gpu, oracle_lib, act, gs, m):
     y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
     assert y.shape == (m, 300)
     _check(y, _q_ref(oracle_lib, L, act))
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4])
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
+    """The fused GEMV shares x between 1, 2 or 4 row tiles of a block; which one a layer gets
+    depends on its row count and the device's size, so every variant is forced here (tuning
+    override NPAMD_GEMV_R) on ragged shapes: codebook in LDS, codebook gathered from memory,
+    fused column permutation, int4, residual VQ."""
+    from neuropress_amd import kernels
+
+    monkeypatch.setenv("NPAMD_GEMV_R", str(rows))
+    n, k = 200, 576  # 12.5 row tiles, 9 chunks of 64
+    for bits, nc in ((8, 256), (16, 65536)):
+        L = cases.vq_layer(900 + bits + m, n, k, nc, bits=bits, act=torch.bfloat16, m=m, bias=True, std=0.05)
+        dev = {key: L[key].to(gpu) for key in ("x", "packed", "cb", "bias")}
+        y = kernels.vq_linear(dev["x"], dev["packed"], dev["cb"], bits, 8, dev["bias"], out_features=n)
+        _check(y, _vq_ref(oracle_lib, L, torch.bfloat16))
+        if nc == 256:
+            perm = torch.randperm(k, generator=cases.gen(3 + m))
+            yp = kernels.vq_linear(dev["x"], dev["packed"], dev["cb"], bits, 8, dev["bias"], out_features=n,
+                                   column_perm=perm.to(torch.int32).to(gpu))
+            _check(yp, _vq_ref(oracle_lib, dict(L, x=L["x"][:, perm].contiguous()), torch.bfloat16))
+    Q = cases.q4_layer(950 + m, n, k, gs=32, act=torch.bfloat16, m=m, bias=True)
+    y = kernels.q_linear(Q["x"].to(gpu), Q["blob"].to(gpu), Q["scale"].to(gpu), 4, 32, None, Q["bias"].to(gpu))
+    _check(y, _q_ref(oracle_lib, Q, torch.bfloat16))
+    R = cases.rvq_layer(11 + m, 80, 256, act=torch.float16, m=m)
+    y = kernels.rvq_linear(R["x"].to(gpu), R["pm"].to(gpu), R["bm"], R["pr"].to(gpu), R["br"], R["cbm"].to(gpu),
+                           R["cbr"].to(gpu), R["scale"].to(gpu), R["wbias"].to(gpu), 80, None, tile=False)
+    _check(y, _rvq_ref(oracle_lib, R, torch.float16))
 
 
 @pytest.mark.parametrize("nbits,gs,asym", [(4, 32, True), (8, 32, False), (2, 16, True), (1, 8, False), (4, 24, False)])
