@@ -58,7 +58,7 @@ static int device_cu_count() {
 bool gemv_lds_codebook_enabled() { return env_int("NPAMD_GEMV_LDS_CB", 1) != 0; }
 bool gemv_lds_activations_forced() { return env_int("NPAMD_GEMV_LDS_X", 0) != 0; }
 
-GemvPlan plan_gemv(int N, int chunks) {
+GemvPlan plan_gemv(int N, int chunks, int max_r) {
   const int steps = (chunks + 3) / 4;
   const int tiles = (N + 15) / 16;
   const int64_t jobs = (int64_t)tiles * steps;
@@ -72,6 +72,7 @@ GemvPlan plan_gemv(int N, int chunks) {
   // and one copy of the codebook in LDS.  The largest R that leaves blocks for at least 0.6 of
   // the compute units wins at every token count, measured on N = 2048 ... 28672.
   p.R = (tiles * 10 >= cus * 24) ? 4 : (tiles * 10 >= cus * 12) ? 2 : 1;
+  if (p.R > max_r) p.R = max_r;
   int spw = (jpw + p.R - 1) / p.R;
   const int r_env = env_int("NPAMD_GEMV_R", 0);
   if (r_env == 1 || r_env == 2 || r_env == 4) p.R = r_env;
@@ -85,9 +86,9 @@ GemvPlan plan_gemv(int N, int chunks) {
 }
 
 bool gemv_perm_keeps_occupancy(int M, int N, int chunks, int cb_bytes) {
-  const GemvPlan plan = plan_gemv(N, chunks);
-  const int red = ((plan.waves * M * 16 * plan.R + 3) & ~3) * (int)sizeof(float);
   const int cbl = (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) ? cb_bytes : 0;
+  const GemvPlan plan = plan_gemv(N, chunks, cbl ? 4 : 2);
+  const int red = ((plan.waves * M * 16 * plan.R + 3) & ~3) * (int)sizeof(float);
   const int xb = M * chunks * 64 * 2;
   const int lds = red + (cbl > xb ? cbl : xb) + xb;
   const int blocks = (N + 16 * plan.R - 1) / (16 * plan.R);

@@ -204,7 +204,8 @@ struct GemvPlan {
   int steps_per_wave;
 };
 
-GemvPlan plan_gemv(int N, int chunks);
+// max_r: most row tiles per block the caller wants (4, or 2 for lookups served by L2).
+GemvPlan plan_gemv(int N, int chunks, int max_r = 4);
 
 // Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
@@ -246,11 +247,16 @@ template <int ACT, class Provider>
 int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStream_t st,
                       const char* what, int cb_bytes = 0) {
   s.steps = (s.chunks + 3) / 4;
-  const GemvPlan plan = plan_gemv(s.N, s.chunks);
+  bool cb_in_lds = false;
+  if constexpr (Provider::kLdsCodebook)
+    cb_in_lds = cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled();
+  // Lookups that go to L2 want many waves in flight more than they want shared x operands
+  // (14336 x 4096, 65536-row codebook, one token: 34.6 us with two row tiles, 37.2 with four).
+  const GemvPlan plan = plan_gemv(s.N, s.chunks, (Provider::kGathers && !cb_in_lds) ? 2 : 4);
   if constexpr (Provider::kLdsCodebook) {
     const bool x_fits = (int64_t)s.M * s.chunks * 64 <= kGemvLdsActivationsMax;
     if (s.perm || (x_fits && gemv_lds_activations_forced())) {  // with a permutation the caller has checked the size
-      if (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) {
+      if (cb_in_lds) {
         if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true, true>(s, pargs, plan, cb_bytes, st, what);
         if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true, true>(s, pargs, plan, cb_bytes, st, what);
         return launch_fused_gemv_r<ACT, Provider, 1, true, true>(s, pargs, plan, cb_bytes, st, what);
@@ -259,7 +265,7 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
       if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, false, true>(s, pargs, plan, 0, st, what);
       return launch_fused_gemv_r<ACT, Provider, 1, false, true>(s, pargs, plan, 0, st, what);
     }
-    if (cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled()) {
+    if (cb_in_lds) {
       if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true>(s, pargs, plan, cb_bytes, st, what);
       if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true>(s, pargs, plan, cb_bytes, st, what);
       return launch_fused_gemv_r<ACT, Provider, 1, true>(s, pargs, plan, cb_bytes, st, what);

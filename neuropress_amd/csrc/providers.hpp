@@ -52,6 +52,7 @@ struct VqProvider {
     u32x4 idx;
   };
   static constexpr bool kLdsCodebook = true;  // the codebook may be staged in LDS (use_codebook)
+  static constexpr bool kGathers = true;  // operands are codebook lookups, not arithmetic on the packed bytes
   const Args& a;
   const u32x4* cb;  // where operands are gathered from: global memory, or an LDS copy
   __device__ explicit VqProvider(const Args& args) : a(args), cb(args.cb) {}
@@ -108,6 +109,7 @@ struct RvqProvider {
     uint32_t s2, b2;  // scale / bias replicated in both halves
   };
   static constexpr bool kLdsCodebook = false;
+  static constexpr bool kGathers = true;  // operands are codebook lookups, not arithmetic on the packed bytes
   const Args& a;
   __device__ explicit RvqProvider(const Args& args) : a(args) {}
 
@@ -184,6 +186,7 @@ struct Q4Provider {
     uint32_t s_lo, s_hi;  // scale (replicated pair) for operands 0-3 and 4-7
   };
   static constexpr bool kLdsCodebook = false;
+  static constexpr bool kGathers = false;  // operands are codebook lookups, not arithmetic on the packed bytes
   const Args& a;
   __device__ explicit Q4Provider(const Args& args) : a(args) {}
 
