@@ -104,6 +104,37 @@ rvq_dequant_kernel(const uint8_t* __restrict__ pm, int64_t nbm, int bits_m,
     store_from_f16_bits<OUT>(out, v * vl + j, rvq_elem(cm[j], cr[j], has_s, s, has_b, b));
 }
 
+// VL = 8: two 16-byte gathers, packed fp16 arithmetic (each operation rounds per element, like
+// the scalar form), one vector store.  Grid = (row, 256 groups of the row): no division.
+template <int BITS_M, int BITS_R, int OUT>
+__global__ void __launch_bounds__(256)
+rvq_dequant_vl8_kernel(const uint8_t* __restrict__ pm, int64_t nbm, int bits_m,
+                       const uint8_t* __restrict__ pr, int64_t nbr, int bits_r,
+                       const u32x4* __restrict__ cbm, uint32_t ncm, const u32x4* __restrict__ cbr, uint32_t ncr,
+                       const uint16_t* __restrict__ row_scale, const uint16_t* __restrict__ row_bias,
+                       int groups, void* __restrict__ out) {
+  const int n = blockIdx.x;
+  const int g = blockIdx.y * 256 + threadIdx.x;
+  if (g >= groups) return;
+  const int64_t v = (int64_t)n * groups + g;
+  const uint32_t im = min(vec_index<BITS_M>(pm, nbm, v, bits_m), ncm - 1u);
+  const uint32_t ir = min(vec_index<BITS_R>(pr, nbr, v, bits_r), ncr - 1u);
+  const u32x4 a = cbm[im], r = cbr[ir];
+  const bool has_s = row_scale != nullptr, has_b = row_bias != nullptr;
+  const uint32_t s2 = has_s ? (uint32_t)row_scale[n] * 0x10001u : 0u;
+  const uint32_t b2 = has_b ? (uint32_t)row_bias[n] * 0x10001u : 0u;
+  const uint32_t am[4] = {a.x, a.y, a.z, a.w}, rr[4] = {r.x, r.y, r.z, r.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f16x2 h = __builtin_bit_cast(f16x2, am[i]) + __builtin_bit_cast(f16x2, rr[i]);
+    if (has_s) h = h * __builtin_bit_cast(f16x2, s2);
+    if (has_b) h = h + __builtin_bit_cast(f16x2, b2);
+    o[i] = __builtin_bit_cast(uint32_t, h);
+  }
+  store8<OUT>(out, v, u32x4{o[0], o[1], o[2], o[3]});
+}
+
 template <int OUT>
 static int launch_vq_dequant(const uint8_t* packed, int64_t n_bytes, int bits, const void* cb,
                              uint32_t nc, int vl, int64_t n_vectors, void* out, hipStream_t st) {
@@ -180,6 +211,33 @@ extern "C" int npamd_rvq_dequant(const uint8_t* packed_main, int64_t n_bytes_mai
                 "npamd_rvq_dequant: null pointer");
   const unsigned blocks = (unsigned)((n_vectors + 255) / 256);
   hipStream_t st = (hipStream_t)stream;
+  const bool aligned16 = ((reinterpret_cast<uintptr_t>(cb_main_f16) | reinterpret_cast<uintptr_t>(cb_res_f16) |
+                           reinterpret_cast<uintptr_t>(out)) % 16) == 0;
+  if (vl == 8 && aligned16 && (groups + 255) / 256 <= 65535) {
+    const dim3 grid((unsigned)N, (unsigned)((groups + 255) / 256));
+    const bool m16 = bits_main == 16 && (reinterpret_cast<uintptr_t>(packed_main) % 2) == 0;
+    const bool r8 = bits_res == 8;
+#define NPAMD_RVQ8_LAUNCH(BM, BR, OUT)                                                               \
+  rvq_dequant_vl8_kernel<BM, BR, OUT><<<grid, 256, 0, st>>>(                                         \
+      packed_main, n_bytes_main, bits_main, packed_res, n_bytes_res, bits_res, (const u32x4*)cb_main_f16, \
+      (uint32_t)nc_main, (const u32x4*)cb_res_f16, (uint32_t)nc_res, (const uint16_t*)row_scale_f16,  \
+      (const uint16_t*)row_bias_f16, (int)groups, out)
+#define NPAMD_RVQ8_BITS(OUT)                                \
+  do {                                                      \
+    if (m16 && r8) NPAMD_RVQ8_LAUNCH(16, 8, OUT);           \
+    else if (m16) NPAMD_RVQ8_LAUNCH(16, 0, OUT);            \
+    else NPAMD_RVQ8_LAUNCH(0, 0, OUT);                      \
+  } while (0)
+    switch (out_dtype) {
+      case NPAMD_F16: NPAMD_RVQ8_BITS(NPAMD_F16); break;
+      case NPAMD_BF16: NPAMD_RVQ8_BITS(NPAMD_BF16); break;
+      case NPAMD_F32: NPAMD_RVQ8_BITS(NPAMD_F32); break;
+      default: return fail(NPAMD_ERR_INVALID, "npamd_rvq_dequant: out_dtype must be f16, bf16 or f32");
+    }
+#undef NPAMD_RVQ8_BITS
+#undef NPAMD_RVQ8_LAUNCH
+    return check_launch("npamd_rvq_dequant");
+  }
 #define NPAMD_RVQ_LAUNCH(OUT)                                                                   \
   rvq_dequant_kernel<OUT><<<blocks, 256, 0, st>>>(                                              \
       packed_main, n_bytes_main, bits_main, packed_res, n_bytes_res, bits_res,                  \

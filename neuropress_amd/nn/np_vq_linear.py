@@ -99,6 +99,12 @@ _TILE_MIN_GRID_FRACTION: float = 0.7
 # tokens, 39 vs 36 us at 256.
 _TILE_SPLIT_MAX_TOKENS: int = 128
 _TILE_SPLIT_LONG_K: int = 8192  # from this many input features on, _TILE_MAX_TOKENS applies
+# Residual layers (two lookups and three fp16 operations per weight) decode faster in one
+# pass than inside the GEMM: 4096 x 4096, 17-384 tokens, tile 39-57 us against 30-41 us for
+# decode + GEMM; 14336 x 4096 88-119 against 74-102 us.  Only where the dense GEMM itself is
+# slow (long reductions: 4096 x 14336, 64-384 tokens, 86-119 against 90-124 us) does the
+# tile band pay.
+_RVQ_TILE_MIN_K: int = 8192
 
 # Opt-in: when a HIP kernel call fails, warn once and run torch ops instead (the
 # reference's behaviour).  Off by default so a missing or broken kernel library
@@ -643,6 +649,8 @@ class NPVQLinear(nn.Module):
         features) covers at least ``_TILE_MIN_GRID_FRACTION`` of the compute units."""
         if not x.is_cuda:
             return True
+        if self.is_residual and self.in_features < _RVQ_TILE_MIN_K:
+            return False
         cus = self._derived.get("cus")
         if cus is None:
             cus = torch.cuda.get_device_properties(x.device).multi_processor_count

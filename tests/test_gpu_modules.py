@@ -94,6 +94,7 @@ def test_nplinear_bands(gpu, act, monkeypatch):
 def test_residual_module_bands(gpu, monkeypatch):
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)  # small layers: force the tile band
+    monkeypatch.setattr(vqmod, "_RVQ_TILE_MIN_K", 0)
     L = cases.rvq_layer(12, 48, 256, nc_main=65536, nc_res=256)
     mk = lambda backend: NPVQLinear(VQProxy(L["cbm"]), L["pm"], L["bm"], 48, 256, 8, backend,
                                     residual_proxy=VQProxy(L["cbr"]), packed_residual=L["pr"],
@@ -105,6 +106,30 @@ def test_residual_module_bands(gpu, monkeypatch):
     for m in (1, 30, 100):
         x = torch.randn(m, 256, generator=cases.gen(m)).half()
         _close(layer(x.to(gpu)), x.float() @ w.T)
+
+
+def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch):
+    """A residual layer with K < 8192 goes from the fused GEMV straight to decode + GEMM; with a
+    long reduction it takes the tile GEMM like a plain layer."""
+    from neuropress_amd import kernels
+
+    calls = []
+    real = kernels.rvq_linear
+    monkeypatch.setattr(kernels, "rvq_linear",
+                        lambda *a, _real=real, **kw: (calls.append((a[0].shape[0], kw.get("tile"))), _real(*a, **kw))[1])
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
+    for k, expect in ((256, [(4, False)]), (8192, [(4, False), (40, True)])):
+        L = cases.rvq_layer(21, 32, k, nc_main=4096, nc_res=16)
+        layer = NPVQLinear(VQProxy(L["cbm"]), L["pm"], L["bm"], 32, k, 8, "cuda_wmma",
+                           residual_proxy=VQProxy(L["cbr"]), packed_residual=L["pr"], residual_bits=L["br"],
+                           row_scale=L["scale"], row_bias=L["wbias"]).to(gpu)
+        layer.proxy.to(gpu), layer.residual_proxy.to(gpu)
+        w = layer._dense_weight_torch(torch.float16).float().cpu()
+        calls.clear()
+        for m in (4, 40):
+            x = (torch.randn(m, k, generator=cases.gen(m)) * 0.3).half()
+            _close(layer(x.to(gpu)), x.float() @ w.T)
+        assert calls == expect
 
 
 def test_narrow_layers_take_the_split_tile_band(gpu, monkeypatch):
