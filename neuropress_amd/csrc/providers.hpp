@@ -166,12 +166,15 @@ struct RvqProvider {
 };
 
 // ---------------------------------------------------------------------------
-// Symmetric int4, zero point 8, group size a multiple of 32.
+// int4, group size a multiple of 32; symmetric (zero point 8) or, with ASYM, a
+// per-group fp16 zero point.
 // One dword of nibbles = one operand, emitted in k-order (0,4,1,5,2,6,3,7).
-// f16: w = f16((q-8) * s) -- exact product, one rounding: the oracle's weight.
-// bf16: w = bf16((q-8) * s) with the product taken in f32.
+// Symmetric f16: w = f16((q-8) * s) -- exact product, one rounding: the oracle's weight.
+// Otherwise w = round((f32(q) - f32(zp)) * f32(s)), the difference exact, the product
+// rounded to f32 and then to the activation type, operation for operation as the
+// element-wise decode does it.
 // ---------------------------------------------------------------------------
-template <int ACT>
+template <int ACT, bool ASYM = false>
 struct Q4Provider {
   static constexpr bool kPermuteA = true;
   struct Args {
@@ -180,10 +183,12 @@ struct Q4Provider {
     int chunks;              // K / 64
     int groups_per_row;      // K / gs
     int gs_shift_chunks;     // log2(gs/32): scale index = (2*kc + half) >> gs_shift_chunks
+    const uint16_t* zp;      // [N, K/gs] (ASYM only)
   };
   struct Raw {
     u32x4 w0, w1;
     uint32_t s_lo, s_hi;  // scale (replicated pair) for operands 0-3 and 4-7
+    uint32_t z_lo, z_hi;  // zero points (fp16 bits) of the same two groups (ASYM only)
   };
   static constexpr bool kLdsCodebook = false;
   static constexpr bool kGathers = false;  // operands are codebook lookups, not arithmetic on the packed bytes
@@ -194,48 +199,73 @@ struct Q4Provider {
     const u32x4* p = reinterpret_cast<const u32x4*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 32);
     r.w0 = p[0];
     r.w1 = p[1];
-    const uint16_t* s = a.scale + (int64_t)n * a.groups_per_row;
-    r.s_lo = (uint32_t)s[(2 * kc) >> a.gs_shift_chunks] * 0x10001u;
-    r.s_hi = (uint32_t)s[(2 * kc + 1) >> a.gs_shift_chunks] * 0x10001u;
+    const int64_t row = (int64_t)n * a.groups_per_row;
+    const int g_lo = (2 * kc) >> a.gs_shift_chunks, g_hi = (2 * kc + 1) >> a.gs_shift_chunks;
+    r.s_lo = (uint32_t)a.scale[row + g_lo] * 0x10001u;
+    r.s_hi = (uint32_t)a.scale[row + g_hi] * 0x10001u;
+    if constexpr (ASYM) {
+      r.z_lo = a.zp[row + g_lo];
+      r.z_hi = a.zp[row + g_hi];
+    }
   }
   template <int J>
   __device__ __forceinline__ u32x4 operand(const Raw& r) const {
     const u32x4& ww = (J < 4) ? r.w0 : r.w1;
     const uint32_t w = (J % 4 == 0) ? ww.x : (J % 4 == 1) ? ww.y : (J % 4 == 2) ? ww.z : ww.w;
-    return dequant8(w, (J < 4) ? r.s_lo : r.s_hi);
+    return dequant8(w, (J < 4) ? r.s_lo : r.s_hi, (J < 4) ? r.z_lo : r.z_hi);
   }
 
   struct PairRaw {
     u32x2 w;      // 16 nibbles = operands 2*jp, 2*jp+1
     uint32_t s2;  // their scale (one 32-k group), replicated
+    uint32_t z;   // their zero point, fp16 bits (ASYM only)
   };
   __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
     r.w = *reinterpret_cast<const u32x2*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 32 + jp * 8);
-    const uint16_t* s = a.scale + (int64_t)n * a.groups_per_row;
-    r.s2 = (uint32_t)s[(2 * kc + (jp >> 1)) >> a.gs_shift_chunks] * 0x10001u;
+    const int64_t g = (int64_t)n * a.groups_per_row + ((2 * kc + (jp >> 1)) >> a.gs_shift_chunks);
+    r.s2 = (uint32_t)a.scale[g] * 0x10001u;
+    if constexpr (ASYM) r.z = a.zp[g];
   }
   __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
-    b0 = dequant8(r.w.x, r.s2);
-    b1 = dequant8(r.w.y, r.s2);
+    b0 = dequant8(r.w.x, r.s2, r.z);
+    b1 = dequant8(r.w.y, r.s2, r.z);
   }
 
   // Eight nibbles of one dword -> one operand, k-order (0,4,1,5,2,6,3,7).
-  __device__ __forceinline__ u32x4 dequant8(uint32_t w, uint32_t s2) const {
+  __device__ __forceinline__ u32x4 dequant8(uint32_t w, uint32_t s2, uint32_t z) const {
 #pragma clang fp contract(off)
     uint32_t o[4];
+    const float sf = f16_bits_to_f32(s2 & 0xFFFFu);
+    const float zf = ASYM ? f16_bits_to_f32(z & 0xFFFFu) : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      // (1024 + q) as fp16 via the exponent trick, then subtract 1032 -> q - 8 exactly.
+      // (1024 + q) as fp16 via the exponent trick.
       const uint32_t pair = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-      const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, 0x64086408u);
-      if constexpr (ACT == NPAMD_F16) {
+      if constexpr (ACT == NPAMD_F16 && !ASYM) {
+        // minus 1032 -> q - 8 exactly; times the scale: one rounding.
+        const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, 0x64086408u);
         o[i] = __builtin_bit_cast(uint32_t, q * __builtin_bit_cast(f16x2, s2));
       } else {
-        const float sf = f16_bits_to_f32(s2 & 0xFFFFu);
-        bf16x2 b;
-        b.x = (__bf16)((float)q.x * sf);
-        b.y = (__bf16)((float)q.y * sf);
-        o[i] = __builtin_bit_cast(uint32_t, b);
+        // q (ASYM) or q - 8 exactly, in fp16; the rest in f32.
+        const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, ASYM ? 0x64006400u : 0x64086408u);
+        float lo = (float)q.x, hi = (float)q.y;
+        if constexpr (ASYM) {
+          lo -= zf;
+          hi -= zf;
+        }
+        lo *= sf;
+        hi *= sf;
+        if constexpr (ACT == NPAMD_F16) {
+          f16x2 h;
+          h.x = (_Float16)lo;
+          h.y = (_Float16)hi;
+          o[i] = __builtin_bit_cast(uint32_t, h);
+        } else {
+          bf16x2 b;
+          b.x = (__bf16)lo;
+          b.y = (__bf16)hi;
+          o[i] = __builtin_bit_cast(uint32_t, b);
+        }
       }
     }
     return u32x4{o[0], o[1], o[2], o[3]};

@@ -2,9 +2,9 @@
 //
 //   q = (w_pack[n, k/vpb] >> ((k%vpb)*nbits)) & mask ;  w = (float(q) - zp) * float(scale)
 //
-// Fast kernels cover the Q4_0 / GPTQ layout the benchmark uses (4 bits, symmetric,
-// group size a power-of-two multiple of 32, K % 64 == 0); every other valid
-// combination (1/2/8 bits, zero points, odd K) runs the element-wise fallback.
+// Fast kernels cover the Q4_0 / GPTQ layouts (4 bits, symmetric or with per-group fp16
+// zero points, group size a power-of-two multiple of 32, K % 64 == 0); every other valid
+// combination (1/2/8 bits, odd group sizes, odd K) runs the element-wise fallback.
 #include <stdlib.h>
 
 #include "gemm_tile.hpp"
@@ -31,23 +31,26 @@ q_dequant_generic_kernel(const uint8_t* __restrict__ w_pack, const uint16_t* __r
   store_from_f32<OUT>(out, e, d * f16_bits_to_f32(scale[sidx]));
 }
 
-// Decode, 4-bit symmetric: one thread per dword of nibbles = 8 weights, one
-// 16-byte (32-byte for f32) store.  group_size % 8 == 0 so the 8 share a scale.
-template <int OUT>
+// Decode, 4-bit (symmetric, or ASYM with per-group zero points): one thread per dword of
+// nibbles = 8 weights, one 16-byte (32-byte for f32) store.  group_size % 8 == 0 so the 8
+// share a scale.
+template <int OUT, bool ASYM>
 __global__ void __launch_bounds__(256)
 q4_dequant_kernel(const uint32_t* __restrict__ w_pack, const uint16_t* __restrict__ scale,
-                  int64_t n_words, int words_per_row, int groups_per_row, int words_per_group,
-                  void* __restrict__ out) {
+                  const uint16_t* __restrict__ zero_point, int64_t n_words, int words_per_row,
+                  int groups_per_row, int words_per_group, void* __restrict__ out) {
 #pragma clang fp contract(off)
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n_words) return;
   const int64_t n = i / words_per_row;
   const int wr = (int)(i - n * words_per_row);
-  const float sc = f16_bits_to_f32(scale[n * groups_per_row + wr / words_per_group]);
+  const int64_t sidx = n * groups_per_row + wr / words_per_group;
+  const float sc = f16_bits_to_f32(scale[sidx]);
+  const float zp = ASYM ? f16_bits_to_f32(zero_point[sidx]) : 8.0f;
   const uint32_t w = w_pack[i];
   float v[8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = ((float)((w >> (4 * j)) & 0xFu) - 8.0f) * sc;
+  for (int j = 0; j < 8; ++j) v[j] = ((float)((w >> (4 * j)) & 0xFu) - zp) * sc;
   if constexpr (OUT == NPAMD_F32) {
     reinterpret_cast<f32x4*>(out)[2 * i] = f32x4{v[0], v[1], v[2], v[3]};
     reinterpret_cast<f32x4*>(out)[2 * i + 1] = f32x4{v[4], v[5], v[6], v[7]};
@@ -69,7 +72,7 @@ q4_dequant_kernel(const uint32_t* __restrict__ w_pack, const uint16_t* __restric
 }
 
 // ---------------------------------------------------------------------------
-// Row-wise GEMV for 4-bit symmetric weights, one token.
+// Row-wise GEMV for 4-bit weights, one token (written out for the symmetric case, zero point 8).
 //
 // A lane takes 16 bytes of one weight row = 32 nibbles = one 32-k group, so the
 // weight stream is read with plain coalesced 16-byte loads and the kernel is
@@ -90,6 +93,7 @@ struct Q4RowArgs {
   const uint16_t* x; int64_t ldx;
   const uint8_t* w_pack;   // [N, K/2]
   const uint16_t* scale;   // [N, K/gs]
+  const uint16_t* zp;      // [N, K/gs] or null (zero point 8)
   const float* bias; uint16_t* y; int64_t ldy;
   int N, K;
   int groups32;            // K / 32
@@ -120,9 +124,10 @@ template <int R>
 struct Q4RowItem {   // one pass (64 groups of 32 k) of R rows
   u32x4 w[R];
   uint16_t sc[R];
+  uint16_t zp[R];    // ASYM only
 };
 
-template <int R>
+template <int R, bool ASYM>
 __device__ __forceinline__ void q4_row_load(Q4RowItem<R>& it, const Q4RowArgs& a, int r0, int p, int lane) {
   const int g = min(p * 64 + lane, a.groups32 - 1);
 #pragma unroll
@@ -130,29 +135,38 @@ __device__ __forceinline__ void q4_row_load(Q4RowItem<R>& it, const Q4RowArgs& a
     const int n = min(r0 + i, a.N - 1);
     it.w[i] = *reinterpret_cast<const u32x4*>(a.w_pack + (int64_t)n * (a.K / 2) + (int64_t)g * 16);
     it.sc[i] = a.scale[(int64_t)n * a.scales_per_row + (g >> a.gs_shift)];
+    if constexpr (ASYM) it.zp[i] = a.zp[(int64_t)n * a.scales_per_row + (g >> a.gs_shift)];
   }
 }
 
-template <int ACT, int M, int R>
+// With a zero point z instead of 8 the part that depends on x only becomes
+// sum_k (b[k] + z) * x[k] = off + (z - 8) * sum_k x[k]: a second table (the plain sum of the
+// group's activations) and one more multiply-add per row and group.
+template <int ACT, int M, int R, bool ASYM>
 __device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4RowArgs& a, const u32x4* xs,
-                                               const float* off, int p, int lane, float (&acc)[R][M]) {
+                                               const float* off, const float* sumx, int p, int lane,
+                                               float (&acc)[R][M]) {
   const bool live = p * 64 + lane < a.groups32;
   // fp16: 1024 + q (nibble in mantissa bits 0..3) and 64 + q (bits 4..7).
   // bf16 has 7 mantissa bits: only 128 + q (bits 0..3 of 0x4300), so three shifts.
   const uint32_t magic_lo = ACT == NPAMD_BF16 ? 0x43004300u : 0x64006400u, magic_hi = 0x54005400u;
   u32x4 xv[M][4];
-  float of[M];
+  float of[M], sx[M];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) xv[m][j] = xs[((size_t)m * a.passes * 4 + (size_t)p * 4 + j) * 64 + lane];
     of[m] = off[(m * a.passes + p) * 64 + lane];
+    if constexpr (ASYM) sx[m] = sumx[(m * a.passes + p) * 64 + lane];
   }
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     float g_acc[M];
 #pragma unroll
-    for (int m = 0; m < M; ++m) g_acc[m] = -of[m];
+    for (int m = 0; m < M; ++m) {
+      g_acc[m] = -of[m];
+      if constexpr (ASYM) g_acc[m] = __builtin_fmaf(8.0f - f16_bits_to_f32(it.zp[i]), sx[m], g_acc[m]);
+    }
     const uint32_t wd[4] = {it.w[i].x, it.w[i].y, it.w[i].z, it.w[i].w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -184,12 +198,14 @@ __device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4R
   }
 }
 
-template <int ACT, int M, int R>
+template <int ACT, int M, int R, bool ASYM>
 __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4RowArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  // xs[m][pass][piece 0..3][lane] (16-byte vectors), then off[m][pass][lane] (floats).
+  // xs[m][pass][piece 0..3][lane] (16-byte vectors), then off[m][pass][lane] (floats), then
+  // (ASYM) sumx[m][pass][lane].
   u32x4* xs = reinterpret_cast<u32x4*>(smem);
   float* off = reinterpret_cast<float*>(smem + (size_t)M * a.passes * 4 * 64 * 16);
+  float* sumx = off + (size_t)M * a.passes * 64;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r0 = (blockIdx.x * kQ4RowWaves + wave) * R;
@@ -197,7 +213,7 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
   // The first pass of weights is requested before x is staged (requesting two here is
   // slower: 11.5 vs 9.2 us on 14336 x 4096).
   Q4RowItem<R> cur, nxt;
-  q4_row_load<R>(cur, a, r0, 0, lane);
+  q4_row_load<R, ASYM>(cur, a, r0, 0, lane);
 
   // Stage x: one thread per (token, 32-k group): its four vectors go to the lane-major
   // layout in (k, k+4) pair order, sum (b[k] + 8) * x[k] to the offset table.
@@ -217,6 +233,7 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
       xs[((size_t)m * a.passes * 4 + (size_t)(g >> 6) * 4 + j) * 64 + (g & 63)] = v;
     }
     off[i] = ACT == NPAMD_BF16 ? 136.f * (sum_even + sum_odd) : 1032.f * sum_even + 72.f * sum_odd;
+    if constexpr (ASYM) sumx[i] = sum_even + sum_odd;
   }
   __syncthreads();
   if (r0 >= a.N) return;
@@ -229,12 +246,12 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
   // Two passes in flight: the next one is requested before the current one is used.
   int p = 0;
   for (; p + 2 <= a.passes; p += 2) {
-    q4_row_load<R>(nxt, a, r0, p + 1, lane);
-    q4_row_compute<ACT, M, R>(cur, a, xs, off, p, lane, acc);
-    q4_row_load<R>(cur, a, r0, min(p + 2, a.passes - 1), lane);
-    q4_row_compute<ACT, M, R>(nxt, a, xs, off, p + 1, lane, acc);
+    q4_row_load<R, ASYM>(nxt, a, r0, p + 1, lane);
+    q4_row_compute<ACT, M, R, ASYM>(cur, a, xs, off, sumx, p, lane, acc);
+    q4_row_load<R, ASYM>(cur, a, r0, min(p + 2, a.passes - 1), lane);
+    q4_row_compute<ACT, M, R, ASYM>(nxt, a, xs, off, sumx, p + 1, lane, acc);
   }
-  if (p < a.passes) q4_row_compute<ACT, M, R>(cur, a, xs, off, p, lane, acc);
+  if (p < a.passes) q4_row_compute<ACT, M, R, ASYM>(cur, a, xs, off, sumx, p, lane, acc);
 
 #pragma unroll
   for (int i = 0; i < R; ++i)
@@ -272,7 +289,7 @@ static int validate_q(const char* what, int N, int K, int nbits, int gs) {
 }
 
 static bool q_fast_ok(const QCall& c) {
-  return c.nbits == 4 && c.zp == nullptr && c.gs % 32 == 0 && is_pow2(c.gs / 32) && c.K % 64 == 0 &&
+  return c.nbits == 4 && c.gs % 32 == 0 && is_pow2(c.gs / 32) && c.K % 64 == 0 &&
          c.K > 0 && c.ldx % 8 == 0 && ptr_aligned(c.x, 16) && ptr_aligned(c.w_pack, 16);
 }
 
@@ -286,8 +303,9 @@ template <int ACT, int M, int R>
 static int launch_q4_rowwise_r(const Q4RowArgs& a, hipStream_t st, const char* what) {
   const int rows_per_block = R * kQ4RowWaves;
   const int blocks = (a.N + rows_per_block - 1) / rows_per_block;
-  const int lds = M * a.passes * (4 * 64 * 16 + 64 * 4);
-  q4_rowwise_gemv_kernel<ACT, M, R><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
+  const int lds = M * a.passes * (4 * 64 * 16 + 64 * 4 * 2);
+  if (a.zp) q4_rowwise_gemv_kernel<ACT, M, R, true><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
+  else q4_rowwise_gemv_kernel<ACT, M, R, false><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
   return check_launch(what);
 }
 
@@ -295,7 +313,7 @@ template <int ACT, int M>
 static int launch_q4_rowwise(const QCall& c) {
   Q4RowArgs a;
   a.x = (const uint16_t*)c.x; a.ldx = c.ldx;
-  a.w_pack = c.w_pack; a.scale = (const uint16_t*)c.scale;
+  a.w_pack = c.w_pack; a.scale = (const uint16_t*)c.scale; a.zp = (const uint16_t*)c.zp;
   a.bias = c.bias; a.y = (uint16_t*)c.y; a.ldy = c.ldy;
   a.N = c.N; a.K = c.K;
   a.groups32 = c.K / 32;
@@ -326,22 +344,27 @@ static int launch_q4_rowwise(const QCall& c) {
 // 13.5 vs 13.8 us on 14336 x 4096), x staged in at most 64 KiB of LDS.
 static bool q4_rowwise_ok(const QCall& c) {
   const int passes = (c.K / 32 + 63) / 64;
-  return (c.act == NPAMD_F16 || env_flag("NPAMD_Q4_ROWWISE_BF16", 0) != 0) && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4) <= 64 * 1024 &&
+  return (c.act == NPAMD_F16 || env_flag("NPAMD_Q4_ROWWISE_BF16", 0) != 0) && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4 * 2) <= 64 * 1024 &&
          ptr_aligned(c.scale, 2) && env_flag("NPAMD_Q4_ROWWISE", 1) != 0;
+}
+
+template <int ACT, bool ASYM>
+static int q4_fused(const QCall& c, bool gemv) {
+  using P = Q4Provider<ACT, ASYM>;
+  typename P::Args a{c.w_pack, (const uint16_t*)c.scale, c.K / 64, c.K / c.gs, log2i(c.gs / 32), (const uint16_t*)c.zp};
+  if (gemv) {
+    GemvShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K / 64, 0, 0};
+    return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+  }
+  GemmShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, c.K / 64, 0};
+  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
 template <int ACT>
 static int q_dispatch(const QCall& c, bool gemv) {
   if (q_fast_ok(c)) {
     if (gemv && q4_rowwise_ok(c)) return launch_q4_rowwise<ACT, 1>(c);
-    using P = Q4Provider<ACT>;
-    typename P::Args a{c.w_pack, (const uint16_t*)c.scale, c.K / 64, c.K / c.gs, log2i(c.gs / 32)};
-    if (gemv) {
-      GemvShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K / 64, 0, 0};
-      return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
-    }
-    GemmShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, c.K / 64, 0};
-    return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
+    return c.zp ? q4_fused<ACT, true>(c, gemv) : q4_fused<ACT, false>(c, gemv);
   }
   const QElem e{c.w_pack, (const uint16_t*)c.scale, (const uint16_t*)c.zp, c.K, c.nbits, c.gs, c.act};
   if (gemv) return launch_generic_gemv<ACT>(c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, e, c.st, c.what);
@@ -377,15 +400,22 @@ extern "C" int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, con
   if (total == 0) return NPAMD_OK;
   NPAMD_REQUIRE(w_pack && scale_f16 && out, "npamd_q_dequant: null pointer");
   hipStream_t st = (hipStream_t)stream;
-  const bool fast = nbits == 4 && !zero_point_f16 && K % 8 == 0 && group_size % 8 == 0 &&
+  const bool fast = nbits == 4 && K % 8 == 0 && group_size % 8 == 0 &&
                     ptr_aligned(w_pack, 4) && ptr_aligned(out, 16);
   if (fast) {
     const int64_t n_words = total / 8;
     const unsigned blocks = (unsigned)((n_words + 255) / 256);
-#define NPAMD_Q4_LAUNCH(OUT)                                                                 \
-  q4_dequant_kernel<OUT><<<blocks, 256, 0, st>>>((const uint32_t*)w_pack,                    \
-                                                 (const uint16_t*)scale_f16, n_words, K / 8, \
-                                                 K / group_size, group_size / 8, out)
+#define NPAMD_Q4_LAUNCH(OUT)                                                                              \
+  do {                                                                                                    \
+    if (zero_point_f16)                                                                                   \
+      q4_dequant_kernel<OUT, true><<<blocks, 256, 0, st>>>(                                               \
+          (const uint32_t*)w_pack, (const uint16_t*)scale_f16, (const uint16_t*)zero_point_f16, n_words,  \
+          K / 8, K / group_size, group_size / 8, out);                                                    \
+    else                                                                                                  \
+      q4_dequant_kernel<OUT, false><<<blocks, 256, 0, st>>>(                                              \
+          (const uint32_t*)w_pack, (const uint16_t*)scale_f16, nullptr, n_words, K / 8, K / group_size,   \
+          group_size / 8, out);                                                                           \
+  } while (0)
     if (out_dtype == NPAMD_F16) NPAMD_Q4_LAUNCH(NPAMD_F16);
     else if (out_dtype == NPAMD_BF16) NPAMD_Q4_LAUNCH(NPAMD_BF16);
     else NPAMD_Q4_LAUNCH(NPAMD_F32);

@@ -258,32 +258,37 @@ def _q_ref(oracle_lib, L, act):
 @pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 128), (4200, 256)])
 @pytest.mark.parametrize("gs", [32, 128])
 @pytest.mark.parametrize("m", [1, 2])
-def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m):
+@pytest.mark.parametrize("asym", [False, True])
+def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m, asym):
     """One fp16 token takes the row-wise kernel (nibbles read as base + q, group offsets folded
     out), two tokens and bf16 the MFMA GEMV.  Row counts that are not a multiple of the rows per wave
     (and enough rows for two per wave), K of one partial pass, of several passes and of a
     partial last pass."""
     from neuropress_amd import kernels
 
-    L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=act, m=m, bias=True)
-    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
+    L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=act, m=m, bias=True, asym=asym)
+    zp = None if L["zp"] is None else L["zp"].to(gpu)
+    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, zp, L["bias"].to(gpu))
     assert y.shape == (m, n) and y.dtype == act
     _check(y, _q_ref(oracle_lib, L, act))
 
 
-def test_q4_rowwise_gemv_large_activations(gpu):
+@pytest.mark.parametrize("asym", [False, True])
+def test_q4_rowwise_gemv_large_activations(gpu, asym):
     """Activations of a few hundred: the folded-out offset (72 * sum x) is then far larger than
-    the result.  Checked against the contraction with the unrounded weight (q - 8) * s in
+    the result.  Checked against the contraction with the unrounded weight (q - zp) * s in
     float64 (what the reference's fused kernel computes, kernels/q4_linear.cu:113-122): the
     only error left must be the fp16 rounding of the output."""
     from neuropress_amd import kernels
 
-    L = cases.q4_layer(731, 96, 4096, gs=32, act=torch.float16, m=1)
+    L = cases.q4_layer(731, 96, 4096, gs=32, act=torch.float16, m=1, asym=asym)
     x = (L["x"].float() * 300).to(torch.float16)
-    q = torch.stack([L["blob"] & 0xF, L["blob"] >> 4], dim=-1).reshape(96, 4096).double() - 8
+    zp = L["zp"].double().reshape(96, 128).repeat_interleave(32, dim=1) if asym else 8
+    q = torch.stack([L["blob"] & 0xF, L["blob"] >> 4], dim=-1).reshape(96, 4096).double() - zp
     w = q * L["scale"].double().reshape(96, 128).repeat_interleave(32, dim=1)
     ref = x.double() @ w.T
-    y = kernels.q_linear(x.to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, 32).cpu().double()
+    y = kernels.q_linear(x.to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, 32,
+                         L["zp"].to(gpu) if asym else None).cpu().double()
     assert ((y - ref).abs() <= 2.0 ** -10 * ref.abs() + 1e-2).all()
 
 
@@ -327,6 +332,48 @@ def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
     y = kernels.rvq_linear(R["x"].to(gpu), R["pm"].to(gpu), R["bm"], R["pr"].to(gpu), R["br"], R["cbm"].to(gpu),
                            R["cbr"].to(gpu), R["scale"].to(gpu), R["wbias"].to(gpu), 80, None, tile=False)
     _check(y, _rvq_ref(oracle_lib, R, torch.float16))
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["vq12", "vq16", "rvq", "q4", "q4_asym", "q4_asym_gs128"])
+def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
+    """One-hot activations read the decoded weight back through the contraction kernels: with
+    x = rows of the identity, y[m, n] is the single product 1 * W[n, k_m], which f32 accumulation
+    and the final rounding leave untouched.  So the MFMA GEMV (16 rows at a time) and the tile
+    GEMM (all K rows at once, with and without a reduction split) must reproduce the one-pass
+    decode, itself checked bit for bit against the oracle, exactly."""
+    from neuropress_amd import kernels
+
+    n, k = 200, 512
+    if kind.startswith("vq"):
+        bits = int(kind[2:])
+        L = cases.vq_layer(61 + bits, n, k, 1 << bits, bits=bits, act=act, m=1, std=0.05)
+        pk, cb = L["packed"].to(gpu), L["cb"].to(gpu)
+        w = kernels.vq_dequant(pk, cb, bits, n, k, act)
+        gemv = lambda x: kernels.vq_linear(x, pk, cb, bits, 8, None, n)
+        tile = lambda x: kernels.vq_gemm_tile(x, pk, cb, bits, n, None)
+    elif kind == "rvq":
+        L = cases.rvq_layer(62, n, k, act=act, m=1)
+        d = {key: (v.to(gpu) if torch.is_tensor(v) else v) for key, v in L.items()}
+        args = (d["pm"], L["bm"], d["pr"], L["br"], d["cbm"], d["cbr"], d["scale"], d["wbias"], n)
+        w = kernels.rvq_dequant(*args, k, act)
+        gemv = lambda x: kernels.rvq_linear(x, *args, None, tile=False)
+        tile = lambda x: kernels.rvq_linear(x, *args, None, tile=True)
+    else:
+        gs = 128 if kind.endswith("gs128") else 32
+        L = cases.q4_layer(63, n, k, gs=gs, act=act, m=1, asym=kind.startswith("q4_asym"))
+        blob, sc = L["blob"].to(gpu), L["scale"].to(gpu)
+        zp = None if L["zp"] is None else L["zp"].to(gpu)
+        w = kernels.q_dequant(blob, sc, 4, gs, zp, act)
+        gemv = lambda x: kernels.q_linear(x, blob, sc, 4, gs, zp)
+        tile = lambda x: kernels.q_gemm_tile(x, blob, sc, 4, gs, zp)
+    eye = torch.eye(k, dtype=act, device=gpu)
+    wt = w.t().contiguous()  # [K, N]: row k is what token "one-hot k" must produce
+    for k0 in (0, 48, k - 16):
+        assert torch.equal(gemv(eye[k0:k0 + 16]), wt[k0:k0 + 16]), f"GEMV, rows {k0}.."
+    assert torch.equal(gemv(eye[7:9]), wt[7:9])   # two tokens (int4: still the MFMA kernel)
+    assert torch.equal(tile(eye), wt), "tile GEMM, 512 tokens"
+    assert torch.equal(tile(eye[100:330]), wt[100:330]), "tile GEMM, 230 tokens"
 
 
 @pytest.mark.parametrize("nbits,gs,asym", [(4, 32, True), (8, 32, False), (2, 16, True), (1, 8, False), (4, 24, False)])
