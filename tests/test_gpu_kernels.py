@@ -42,6 +42,21 @@ def test_vq_dequant_bit_exact(gpu, oracle_lib, bits, dtype, vl):
     _bits_equal(out, ref)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nc,bits", [(4096, 12), (3000, 12), (4096, 16), (2049, 13)])
+def test_vq_dequant_lds_codebook_bit_exact(gpu, oracle_lib, dtype, nc, bits):
+    """Layers of at least 2^20 vectors with a 2049..4096-row codebook decode from an LDS copy of the
+    table (512 blocks, each a contiguous run of vectors).  2050 rows of 4096 columns: the last
+    block's run is ragged.  Checked bit for bit against the oracle."""
+    from neuropress_amd import kernels
+
+    n, k = 2050, 4096
+    L = cases.vq_layer(300 + nc + bits, n, k, nc, bits=bits, std=1.0)
+    ref = oracle_lib.vq_decode(L["packed"].numpy(), bits, orc.to_bits(L["cb"]), n, k, orc.torch_dtype_code(dtype))
+    out = kernels.vq_dequant(L["packed"].to(gpu), L["cb"].to(gpu), bits, n, k, dtype)
+    _bits_equal(out, ref)
+
+
 def test_vq_dequant_special_values(gpu, oracle_lib):
     """Codebook holding inf, subnormals, the largest finite half and signed zeros."""
     from neuropress_amd import kernels
