@@ -93,6 +93,14 @@ int npamd_vq_gemv_perm(const void* x, int64_t ldx, const int32_t* column_perm,
  * 0 otherwise: gather x yourself and call npamd_vq_gemv.  Host-only arithmetic. */
 int npamd_vq_gemv_perm_supported(int M, int N, int K, int nc, int vl, int bits);
 
+/* 1 when the MFMA kernels behind npamd_vq_gemv / npamd_vq_gemm_tile (and the residual forms) take
+ * a layer of this shape (VL = 8, K % 64 == 0, index width 4 / 8 / 12 / 16), pointer alignment
+ * aside; 0 when they would run their element-wise fallback, which decodes the weight once per 16
+ * tokens: beyond 16 tokens decode once (npamd_vq_dequant) and use a dense GEMM instead, as the
+ * reference does for shapes its kernels do not take (neuropress/nn/np_vq_linear.py:1127-1148).
+ * Host-only arithmetic. */
+int npamd_vq_fused_supported(int K, int vl, int bits);
+
 /*
  * Tile-decode MFMA GEMM, any M >= 1: same contraction, weight tiles decoded
  * inside the kernel, dense weight never written.
@@ -239,6 +247,13 @@ int npamd_rvq_gemm_tile(const void* x, int64_t ldx,
 int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, const void* zero_point_f16,
                     int N, int K, int nbits, int group_size, void* out, int out_dtype,
                     void* stream);
+
+/* 1 when the MFMA kernels behind npamd_q_gemv / npamd_q_gemm_tile take the layer (4 bits, with or
+ * without zero points, group size 32 * 2^j, K % 64 == 0), pointer alignment aside; 0 when they would
+ * run the element-wise fallback (1 / 2 / 8 bits, other group sizes), which decodes the weight once per
+ * 16 tokens: beyond 16 tokens use npamd_q_dequant and a dense GEMM.  The reference runs its one GEMV
+ * kernel at every token count (neuropress/kernels/q4_linear.cu:137-139).  Host-only arithmetic. */
+int npamd_q_fused_supported(int K, int nbits, int group_size);
 
 /*
  * Fused dequant GEMV, M <= NPAMD_GEMV_MAX_M.

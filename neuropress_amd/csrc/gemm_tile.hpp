@@ -40,6 +40,7 @@
 // bias, and rounds.
 #pragma once
 
+#include "gemv.hpp"
 #include "providers.hpp"
 
 namespace npamd {
@@ -521,29 +522,14 @@ int launch_tile_gemm(GemmShape s, const typename Provider::Args& pargs, hipStrea
 }
 
 // ---------------------------------------------------------------------------
-// Fallback for shapes the MFMA kernel does not take: one thread per output
-// element.  Slow by design; exists so every valid input has a HIP path.
+// Fallback for shapes the MFMA kernel does not take: the element-wise GEMV kernel
+// over blocks of 16 tokens (the weight is decoded once per block).  Slow; exists so
+// every valid input has a HIP path.  The modules send such layers to decode + GEMM.
 // ---------------------------------------------------------------------------
-template <int ACT, class Elem>
-__global__ void __launch_bounds__(256)
-generic_gemm_kernel(const void* __restrict__ x, int64_t ldx, const float* __restrict__ bias,
-                    void* __restrict__ y, int64_t ldy, int M, int N, int K, const Elem elem) {
-  const int n = blockIdx.x * 64 + (threadIdx.x & 63);
-  const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
-  if (n >= N || m >= M) return;
-  float acc = 0.f;
-  for (int k = 0; k < K; ++k)
-    acc = __builtin_fmaf(load_as_f32<ACT>(x, (int64_t)m * ldx + k), elem.get(n, k), acc);
-  if (bias) acc += bias[n];
-  store_from_f32<ACT>(y, (int64_t)m * ldy + n, acc);
-}
-
 template <int ACT, class Elem>
 int launch_generic_gemm(const void* x, int64_t ldx, const float* bias, void* y, int64_t ldy,
                         int M, int N, int K, const Elem& elem, hipStream_t st, const char* what) {
-  const dim3 grid((N + 63) / 64, (M + 3) / 4);
-  generic_gemm_kernel<ACT, Elem><<<grid, 256, 0, st>>>(x, ldx, bias, y, ldy, M, N, K, elem);
-  return check_launch(what);
+  return launch_generic_gemv<ACT, Elem>(x, ldx, bias, y, ldy, M, N, K, elem, st, what);
 }
 
 }  // namespace npamd

@@ -64,7 +64,7 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   const int red_floats = (n_waves * s.M * 16 * R + 3) & ~3;
   uint8_t* const lds0 = reinterpret_cast<uint8_t*>(red) + red_floats * (int)sizeof(float);
   int cb_lds_bytes = 0;
-  if constexpr (CB_LDS) cb_lds_bytes = prov.codebook_rows() * 16;
+  if constexpr (CB_LDS) cb_lds_bytes = prov.codebook_vec16() * 16;
   const uint16_t* x_lds = nullptr;
   if constexpr (X_LDS) {
     // Rows of x: a coalesced copy into LDS, then (with a permutation) a second LDS buffer filled
@@ -105,7 +105,7 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   if constexpr (CB_LDS) {
     u32x4* cb_lds = reinterpret_cast<u32x4*>(lds0);
     const u32x4* src = prov.global_codebook();
-    for (int i = threadIdx.x; i < prov.codebook_rows(); i += blockDim.x) cb_lds[i] = src[i];
+    for (int i = threadIdx.x; i < prov.codebook_vec16(); i += blockDim.x) cb_lds[i] = src[i];
     prov.use_codebook(cb_lds);
   }
   if constexpr (CB_LDS || X_LDS) __syncthreads();
@@ -283,29 +283,44 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
 // Slow by design; exists so that every valid input has a HIP path.
 //   Elem::get(n, k) -> float weight value in the activation dtype's rounding.
 // ---------------------------------------------------------------------------
-template <int ACT, class Elem>
+template <int ACT, class Elem, int MT>
 __global__ void __launch_bounds__(256)
-generic_gemv_kernel(const void* __restrict__ x, int64_t ldx, const float* __restrict__ bias,
+generic_rows_kernel(const void* __restrict__ x, int64_t ldx, const float* __restrict__ bias,
                     void* __restrict__ y, int64_t ldy, int M, int N, int K, const Elem elem) {
+  // One wave per output row and block of up to MT tokens (blockIdx.y): a weight element is
+  // decoded once per MT tokens, each lane summing its k = lane, lane + 64, ... in order.
   const int lane = threadIdx.x & 63;
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int m = blockIdx.y;
-  if (n >= N || m >= M) return;
-  float acc = 0.f;
-  for (int k = lane; k < K; k += 64)
-    acc = __builtin_fmaf(load_as_f32<ACT>(x, (int64_t)m * ldx + k), elem.get(n, k), acc);
-  acc = wave_reduce_sum(acc);
-  if (lane == 0) {
-    if (bias) acc += bias[n];
-    store_from_f32<ACT>(y, (int64_t)m * ldy + n, acc);
+  const int m0 = blockIdx.y * MT;
+  const int mt = min(MT, M - m0);
+  if (n >= N) return;
+  float acc[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) acc[j] = 0.f;
+  for (int k = lane; k < K; k += 64) {
+    const float w = elem.get(n, k);
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+      if (j < mt) acc[j] = __builtin_fmaf(load_as_f32<ACT>(x, (int64_t)(m0 + j) * ldx + k), w, acc[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    if (j >= mt) break;
+    float total = wave_reduce_sum(acc[j]);
+    if (lane == 0) {
+      if (bias) total += bias[n];
+      store_from_f32<ACT>(y, (int64_t)(m0 + j) * ldy + n, total);
+    }
   }
 }
 
 template <int ACT, class Elem>
 int launch_generic_gemv(const void* x, int64_t ldx, const float* bias, void* y, int64_t ldy,
                         int M, int N, int K, const Elem& elem, hipStream_t st, const char* what) {
-  const dim3 grid((N + 3) / 4, M);
-  generic_gemv_kernel<ACT, Elem><<<grid, 256, 0, st>>>(x, ldx, bias, y, ldy, M, N, K, elem);
+  const unsigned rows = (unsigned)((N + 3) / 4);
+  if (M == 1) generic_rows_kernel<ACT, Elem, 1><<<dim3(rows, 1), 256, 0, st>>>(x, ldx, bias, y, ldy, M, N, K, elem);
+  else if (M <= 4) generic_rows_kernel<ACT, Elem, 4><<<dim3(rows, 1), 256, 0, st>>>(x, ldx, bias, y, ldy, M, N, K, elem);
+  else generic_rows_kernel<ACT, Elem, 16><<<dim3(rows, (unsigned)((M + 15) / 16)), 256, 0, st>>>(x, ldx, bias, y, ldy, M, N, K, elem);
   return check_launch(what);
 }
 

@@ -19,7 +19,7 @@
 //   operand_pair(raw, b0, b1)     -- the two operands
 //
 // A B-operand of a VQ weight with VL = 8 is exactly one codebook row, so the
-// 16-byte gather lands in MFMA layout with no shuffling.  For int4 the eight
+// 16-byte gather lands in MFMA layout with no shuffling (VL = 4: two rows, two 8-byte gathers).  For int4 the eight
 // nibbles of one dword are one operand, produced in the k-order
 // (0,4,1,5,2,6,3,7); the A-operand is permuted the same way (kPermuteA).
 #pragma once
@@ -36,20 +36,25 @@ __device__ __forceinline__ uint32_t select_dword(const u32x4& v, int jp) {
 }
 
 // ---------------------------------------------------------------------------
-// Single-codebook VQ, VL = 8, fast index widths.
+// Single-codebook VQ, fast index widths, VL = 8 or 4.
 //   CONV : codebook is fp16 but activations are bf16 -> convert per gather.
+// VL = 8: a codebook row is one operand (one 16-byte gather).  VL = 4 (the reference's default
+// vector length): an operand is two rows, two 8-byte gathers; a 64-k chunk holds 16 indices.
 // ---------------------------------------------------------------------------
-template <int ACT, int BITS, bool CONV>
+template <int ACT, int BITS, bool CONV, int VL = 8>
 struct VqProvider {
+  static_assert(VL == 8 || VL == 4, "vector length 8 or 4");
   static constexpr bool kPermuteA = false;
+  static constexpr int kIdxPerChunk = 64 / VL;
   struct Args {
     const uint8_t* packed;
-    const u32x4* cb;
+    const u32x4* cb;   // VL = 4: rows of 8 bytes behind this pointer
     uint32_t nc_minus_1;
     int chunks;  // K / 64
   };
   struct Raw {
-    u32x4 idx;
+    u32x4 idx;     // indices 0..7 of the chunk, 16 bits each
+    u32x4 idx_hi;  // indices 8..15 (VL = 4 only)
   };
   static constexpr bool kLdsCodebook = true;  // the codebook may be staged in LDS (use_codebook)
   static constexpr bool kGathers = true;  // operands are codebook lookups, not arithmetic on the packed bytes
@@ -58,28 +63,59 @@ struct VqProvider {
   __device__ explicit VqProvider(const Args& args) : a(args), cb(args.cb) {}
   __device__ __forceinline__ void use_codebook(const u32x4* p) { cb = p; }
   __device__ __forceinline__ const u32x4* global_codebook() const { return a.cb; }
-  __device__ __forceinline__ int codebook_rows() const { return (int)a.nc_minus_1 + 1; }
+  // Size of the table in 16-byte units (VL = 4: callers stage it in LDS only when it has an even number of rows).
+  __device__ __forceinline__ int codebook_vec16() const {
+    return VL == 8 ? (int)a.nc_minus_1 + 1 : ((int)a.nc_minus_1 + 1) / 2;
+  }
+
+  __device__ __forceinline__ u32x4 row_pair(uint32_t i0, uint32_t i1) const {  // VL = 4: two rows = one operand
+    const u32x2* c2 = reinterpret_cast<const u32x2*>(cb);
+    const u32x2 lo = c2[min(i0, a.nc_minus_1)], hi = c2[min(i1, a.nc_minus_1)];
+    return u32x4{lo.x, lo.y, hi.x, hi.y};
+  }
 
   __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
-    r.idx = load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8);
+    const int64_t i0 = ((int64_t)n * a.chunks + kc) * kIdxPerChunk;
+    r.idx = load_idx8<BITS>(a.packed, i0);
+    if constexpr (VL == 4) r.idx_hi = load_idx8<BITS>(a.packed, i0 + 8);
   }
   template <int J>
   __device__ __forceinline__ u32x4 operand(const Raw& r) const {
-    u32x4 c = cb[min(idx8_get(r.idx, J), a.nc_minus_1)];
+    u32x4 c;
+    if constexpr (VL == 8) {
+      c = cb[min(idx8_get(r.idx, J), a.nc_minus_1)];
+    } else {
+      const u32x4& v = (J < 4) ? r.idx : r.idx_hi;
+      c = row_pair(idx8_get(v, (2 * J) % 8), idx8_get(v, (2 * J + 1) % 8));
+    }
     if constexpr (CONV) c = cb_to_act<ACT>(c);
     return c;
   }
 
   struct PairRaw {
-    uint32_t pair;  // indices of operands 2*jp (low half) and 2*jp+1 (high half)
+    uint32_t pair;   // VL = 8: indices of operands 2*jp (low half) and 2*jp+1 (high half)
+    uint32_t pair1;  // VL = 4: `pair` holds the two rows of operand 2*jp, `pair1` those of 2*jp+1
   };
   __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
-    // the four lane-groups of a column read the same 8-index group: one request
-    r.pair = select_dword(load_idx8<BITS>(a.packed, ((int64_t)n * a.chunks + kc) * 8), jp);
+    const int64_t i0 = ((int64_t)n * a.chunks + kc) * kIdxPerChunk;
+    if constexpr (VL == 8) {
+      // the four lane-groups of a column read the same 8-index group: one request
+      r.pair = select_dword(load_idx8<BITS>(a.packed, i0), jp);
+    } else {
+      // operands 2jp, 2jp+1 = indices 4jp .. 4jp+3: dwords 2(jp&1), 2(jp&1)+1 of index group jp>>1
+      const u32x4 v = load_idx8<BITS>(a.packed, i0 + 8 * (jp >> 1));
+      r.pair = (jp & 1) ? v.z : v.x;
+      r.pair1 = (jp & 1) ? v.w : v.y;
+    }
   }
   __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
-    b0 = cb[min(r.pair & 0xFFFFu, a.nc_minus_1)];
-    b1 = cb[min(r.pair >> 16, a.nc_minus_1)];
+    if constexpr (VL == 8) {
+      b0 = cb[min(r.pair & 0xFFFFu, a.nc_minus_1)];
+      b1 = cb[min(r.pair >> 16, a.nc_minus_1)];
+    } else {
+      b0 = row_pair(r.pair & 0xFFFFu, r.pair >> 16);
+      b1 = row_pair(r.pair1 & 0xFFFFu, r.pair1 >> 16);
+    }
     if constexpr (CONV) {
       b0 = cb_to_act<ACT>(b0);
       b1 = cb_to_act<ACT>(b1);

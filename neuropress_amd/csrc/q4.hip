@@ -71,6 +71,44 @@ q4_dequant_kernel(const uint32_t* __restrict__ w_pack, const uint16_t* __restric
   }
 }
 
+// Decode, 1 / 2 / 8 bits: one thread per eight weights (NBITS bytes of codes), same arithmetic
+// as the element-wise kernel, one 16-byte (32-byte for f32) store.
+template <int NBITS, int OUT>
+__global__ void __launch_bounds__(256)
+qn_dequant_kernel(const uint8_t* __restrict__ w_pack, const uint16_t* __restrict__ scale,
+                  const uint16_t* __restrict__ zero_point, int64_t n_octets, int octets_per_row,
+                  int groups_per_row, int octets_per_group, void* __restrict__ out) {
+#pragma clang fp contract(off)
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_octets) return;
+  const int64_t n = i / octets_per_row;
+  const int o = (int)(i - n * octets_per_row);
+  const int64_t sidx = n * groups_per_row + o / octets_per_group;
+  const float sc = f16_bits_to_f32(scale[sidx]);
+  const float zp = zero_point ? f16_bits_to_f32(zero_point[sidx]) : (float)(1 << (NBITS - 1));
+  uint64_t bits;
+  if constexpr (NBITS == 8) {
+    const u32x2 t = *reinterpret_cast<const u32x2*>(w_pack + i * 8);
+    bits = (uint64_t)t.x | ((uint64_t)t.y << 32);
+  } else if constexpr (NBITS == 2) {
+    bits = *reinterpret_cast<const uint16_t*>(w_pack + i * 2);
+  } else {
+    bits = w_pack[i];
+  }
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = ((float)(uint32_t)((bits >> (NBITS * j)) & ((1u << NBITS) - 1u)) - zp) * sc;
+  if constexpr (OUT == NPAMD_F32) {
+    reinterpret_cast<f32x4*>(out)[2 * i] = f32x4{v[0], v[1], v[2], v[3]};
+    reinterpret_cast<f32x4*>(out)[2 * i + 1] = f32x4{v[4], v[5], v[6], v[7]};
+  } else {
+    uint32_t h[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) h[j] = OUT == NPAMD_F16 ? f32_to_f16_bits(v[j]) : f32_to_bf16_bits(v[j]);
+    reinterpret_cast<u32x4*>(out)[i] = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Row-wise GEMV for 4-bit weights, one token (written out for the symmetric case, zero point 8).
 //
@@ -420,6 +458,25 @@ extern "C" int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, con
     else if (out_dtype == NPAMD_BF16) NPAMD_Q4_LAUNCH(NPAMD_BF16);
     else NPAMD_Q4_LAUNCH(NPAMD_F32);
 #undef NPAMD_Q4_LAUNCH
+  } else if ((nbits == 8 || nbits == 2 || nbits == 1) && K % 8 == 0 && group_size % 8 == 0 &&
+             ptr_aligned(w_pack, nbits) && ptr_aligned(out, 16)) {
+    const int64_t n_octets = total / 8;
+    const unsigned blocks = (unsigned)((n_octets + 255) / 256);
+#define NPAMD_QN_LAUNCH(NB, OUT)                                                                       \
+  qn_dequant_kernel<NB, OUT><<<blocks, 256, 0, st>>>(w_pack, (const uint16_t*)scale_f16,               \
+                                                     (const uint16_t*)zero_point_f16, n_octets, K / 8, \
+                                                     K / group_size, group_size / 8, out)
+#define NPAMD_QN_OUT(NB)                                         \
+  do {                                                           \
+    if (out_dtype == NPAMD_F16) NPAMD_QN_LAUNCH(NB, NPAMD_F16);  \
+    else if (out_dtype == NPAMD_BF16) NPAMD_QN_LAUNCH(NB, NPAMD_BF16); \
+    else NPAMD_QN_LAUNCH(NB, NPAMD_F32);                         \
+  } while (0)
+    if (nbits == 8) NPAMD_QN_OUT(8);
+    else if (nbits == 2) NPAMD_QN_OUT(2);
+    else NPAMD_QN_OUT(1);
+#undef NPAMD_QN_OUT
+#undef NPAMD_QN_LAUNCH
   } else {
     const unsigned blocks = (unsigned)((total + 255) / 256);
 #define NPAMD_QG_LAUNCH(OUT)                                                                   \
@@ -432,6 +489,13 @@ extern "C" int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, con
 #undef NPAMD_QG_LAUNCH
   }
   return check_launch("npamd_q_dequant");
+}
+
+extern "C" int npamd_q_fused_supported(int K, int nbits, int group_size) {
+  return nbits == 4 && group_size > 0 && group_size % 32 == 0 && is_pow2(group_size / 32) && K > 0 && K % 64 == 0 &&
+                 K % group_size == 0
+             ? 1
+             : 0;
 }
 
 extern "C" int npamd_q_gemv(const void* x, int64_t ldx, const uint8_t* w_pack, const void* scale_f16,

@@ -61,7 +61,7 @@ inline VqElem make_elem(const VqCall& c) {
 
 inline bool fast_ok(const VqCall& c) {
   const bool bits_ok = c.bits == 4 || c.bits == 8 || c.bits == 12 || c.bits == 16;
-  return c.vl == 8 && bits_ok && c.K % 64 == 0 && c.K > 0 && c.ldx % 8 == 0 && aligned(c.x, 16) &&
+  return (c.vl == 8 || (c.vl == 4 && !c.packed_r)) && bits_ok && c.K % 64 == 0 && c.K > 0 && c.ldx % 8 == 0 && aligned(c.x, 16) &&
          aligned(c.packed, 16) && aligned(c.cb, 16);
 }
 

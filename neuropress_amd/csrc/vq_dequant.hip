@@ -52,23 +52,71 @@ vq_dequant_vl8_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int b
   store8<OUT>(out, v, codebook[idx]);
 }
 
-// VL = 8, codebook of up to 4096 rows copied into LDS first.  A 64 KiB table does not fit the
-// 32 KiB vector L1, so gathers from memory run at the L1-miss rate (36 us for a 14336 x 4096
-// layer, the same as a 65536-row table); from LDS the kernel is bound by the store stream.
-// Two blocks of 1024 threads per compute unit, each decoding a contiguous run of vectors.
+// VL = 4: two vectors per thread -- two 8-byte gathers, one 16-byte (f32: 32-byte) store.
+template <int OUT>
+__device__ __forceinline__ void store4x2(void* out, int64_t v0, u32x2 c0, u32x2 c1, bool both) {
+  if (both) {
+    store8<OUT>(out, v0 >> 1, u32x4{c0.x, c0.y, c1.x, c1.y});  // v0 is even: 8 values = one store8 unit
+  } else if constexpr (OUT == NPAMD_F16) {
+    reinterpret_cast<u32x2*>(out)[v0] = c0;
+  } else if constexpr (OUT == NPAMD_BF16) {
+    reinterpret_cast<u32x2*>(out)[v0] = u32x2{f16x2_to_bf16x2(c0.x), f16x2_to_bf16x2(c0.y)};
+  } else {
+    reinterpret_cast<f32x4*>(out)[v0] = f32x4{f16_bits_to_f32(c0.x & 0xFFFFu), f16_bits_to_f32(c0.x >> 16),
+                                              f16_bits_to_f32(c0.y & 0xFFFFu), f16_bits_to_f32(c0.y >> 16)};
+  }
+}
+
 template <int BITS, int OUT>
+__global__ void __launch_bounds__(256)
+vq_dequant_vl4_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int bits,
+                      const u32x2* __restrict__ codebook, uint32_t nc, void* __restrict__ out,
+                      int64_t n_vectors) {
+  const int64_t v0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (v0 >= n_vectors) return;
+  const bool both = v0 + 1 < n_vectors;
+  const u32x2 c0 = codebook[min(vec_index<BITS>(packed, n_bytes, v0, bits), nc - 1u)];
+  const u32x2 c1 = codebook[min(vec_index<BITS>(packed, n_bytes, both ? v0 + 1 : v0, bits), nc - 1u)];
+  store4x2<OUT>(out, v0, c0, c1, both);
+}
+
+// VL = 8 or 4, a table of 16 to 64 KiB copied into LDS first.  Such a table overflows or fills
+// the 32 KiB vector L1, so gathers from memory run at the L1-miss rate (36 us for a
+// 14336 x 4096 layer with 4096 rows of 16 bytes, the same as a 65536-row table); from LDS the
+// kernel is bound by the store stream.  Two blocks of 1024 threads per compute unit, each
+// decoding a contiguous run of vectors.
+template <int BITS, int OUT, int VL>
 __global__ void __launch_bounds__(1024)
-vq_dequant_vl8_lds_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int bits,
-                          const u32x4* __restrict__ codebook, uint32_t nc, void* __restrict__ out,
-                          int64_t n_vectors, int64_t vectors_per_block) {
+vq_dequant_lds_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int bits,
+                      const u32x4* __restrict__ codebook, uint32_t nc, void* __restrict__ out,
+                      int64_t n_vectors, int64_t vectors_per_block) {
   extern __shared__ __attribute__((aligned(16))) u32x4 cb_lds[];
-  for (uint32_t i = threadIdx.x; i < nc; i += 1024) cb_lds[i] = codebook[i];
+  const uint32_t vec16 = VL == 8 ? nc : (nc + 1) / 2;  // the allocation behind an odd VL = 4 table is not read past:
+  for (uint32_t i = threadIdx.x; i < vec16; i += 1024) {  // its last half-filled unit is fetched as 8 bytes
+    if (VL == 4 && (nc & 1) && i == vec16 - 1) {
+      const u32x2 t = reinterpret_cast<const u32x2*>(codebook)[nc - 1];
+      cb_lds[i] = u32x4{t.x, t.y, 0u, 0u};
+    } else {
+      cb_lds[i] = codebook[i];
+    }
+  }
   __syncthreads();
   const int64_t begin = (int64_t)blockIdx.x * vectors_per_block;
   const int64_t end = min(begin + vectors_per_block, n_vectors);
-  for (int64_t v = begin + threadIdx.x; v < end; v += 1024) {
-    const uint32_t idx = min(vec_index<BITS>(packed, n_bytes, v, bits), nc - 1u);
-    store8<OUT>(out, v, cb_lds[idx]);
+  if constexpr (VL == 8) {
+    for (int64_t v = begin + threadIdx.x; v < end; v += 1024) {
+      const uint32_t idx = min(vec_index<BITS>(packed, n_bytes, v, bits), nc - 1u);
+      store8<OUT>(out, v, cb_lds[idx]);
+    }
+  } else {
+    // two vectors per thread (a run starts at an even vector: vectors_per_block is a multiple of 1024)
+    const u32x2* cb2 = reinterpret_cast<const u32x2*>(cb_lds);
+    for (int64_t v0 = begin + 2 * threadIdx.x; v0 < end; v0 += 2048) {
+      const bool both = v0 + 1 < end;
+      const u32x2 c0 = cb2[min(vec_index<BITS>(packed, n_bytes, v0, bits), nc - 1u)];
+      const u32x2 c1 = cb2[min(vec_index<BITS>(packed, n_bytes, both ? v0 + 1 : v0, bits), nc - 1u)];
+      store4x2<OUT>(out, v0, c0, c1, both);
+    }
   }
 }
 
@@ -161,25 +209,44 @@ static int launch_vq_dequant(const uint8_t* packed, int64_t n_bytes, int bits, c
   const unsigned blocks = (unsigned)((n_vectors + 255) / 256);
   const bool cb_aligned = (reinterpret_cast<uintptr_t>(cb) % 16) == 0;
   const bool out_aligned = (reinterpret_cast<uintptr_t>(out) % 16) == 0;
+  // Tables of 16 to 64 KiB on layers large enough to pay for one copy per block.
+  const int64_t table_bytes = (int64_t)nc * vl * 2;
+  if ((vl == 8 || vl == 4) && cb_aligned && out_aligned && table_bytes > 16 * 1024 && table_bytes <= 64 * 1024 &&
+      n_vectors >= (1 << 20)) {
+    const u32x4* c = reinterpret_cast<const u32x4*>(cb);
+    const int lds = (int)((table_bytes + 15) / 16 * 16);
+    const int64_t per_block = ((n_vectors + 511) / 512 + 1023) / 1024 * 1024;
+    const unsigned grid = (unsigned)((n_vectors + per_block - 1) / per_block);
+    const bool b16 = bits == 16 && (reinterpret_cast<uintptr_t>(packed) % 2) == 0;
+#define NPAMD_VQ_LDS(B, V) \
+  vq_dequant_lds_kernel<B, OUT, V><<<grid, 1024, lds, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors, per_block)
+    if (vl == 8) {
+      if (b16) NPAMD_VQ_LDS(16, 8);
+      else NPAMD_VQ_LDS(0, 8);
+    } else {
+      if (b16) NPAMD_VQ_LDS(16, 4);
+      else NPAMD_VQ_LDS(0, 4);
+    }
+#undef NPAMD_VQ_LDS
+    return check_launch("npamd_vq_dequant");
+  }
   if (vl == 8 && cb_aligned && out_aligned) {
     const u32x4* c = reinterpret_cast<const u32x4*>(cb);
-    // Tables of 32 to 64 KiB on layers large enough to pay for one copy per block.
-    if (nc > 2048 && nc <= 4096 && n_vectors >= (1 << 20)) {
-      const int lds = (int)nc * 16;
-      const int64_t per_block = ((n_vectors + 511) / 512 + 1023) / 1024 * 1024;
-      const unsigned grid = (unsigned)((n_vectors + per_block - 1) / per_block);
-      if (bits == 16 && (reinterpret_cast<uintptr_t>(packed) % 2) == 0)
-        vq_dequant_vl8_lds_kernel<16, OUT><<<grid, 1024, lds, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors, per_block);
-      else
-        vq_dequant_vl8_lds_kernel<0, OUT><<<grid, 1024, lds, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors, per_block);
-      return check_launch("npamd_vq_dequant");
-    }
     if (bits == 16 && (reinterpret_cast<uintptr_t>(packed) % 2) == 0)
       vq_dequant_vl8_kernel<16, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
     else if (bits == 8)
       vq_dequant_vl8_kernel<8, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
     else
       vq_dequant_vl8_kernel<0, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
+  } else if (vl == 4 && (reinterpret_cast<uintptr_t>(cb) % 8) == 0 && out_aligned) {
+    const u32x2* c = reinterpret_cast<const u32x2*>(cb);
+    const unsigned blocks = (unsigned)(((n_vectors + 1) / 2 + 255) / 256);  // two vectors per thread
+    if (bits == 16 && (reinterpret_cast<uintptr_t>(packed) % 2) == 0)
+      vq_dequant_vl4_kernel<16, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
+    else if (bits == 8)
+      vq_dequant_vl4_kernel<8, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
+    else
+      vq_dequant_vl4_kernel<0, OUT><<<blocks, 256, 0, st>>>(packed, n_bytes, bits, c, nc, out, n_vectors);
   } else {
     vq_dequant_generic_kernel<OUT><<<blocks, 256, 0, st>>>(
         packed, n_bytes, bits, reinterpret_cast<const uint16_t*>(cb), nc, out, n_vectors, vl);

@@ -6,28 +6,33 @@ using namespace npamd;
 
 namespace {
 
-template <int ACT, int BITS>
+template <int ACT, int BITS, int VL>
 int run_vq(const VqCall& c, const GemmShape& s) {
   if constexpr (ACT == NPAMD_BF16) {
     if (c.cb_dtype == NPAMD_F16) {
-      using P = VqProvider<ACT, BITS, true>;
+      using P = VqProvider<ACT, BITS, true, VL>;
       typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
       return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
     }
   }
-  using P = VqProvider<ACT, BITS, false>;
+  using P = VqProvider<ACT, BITS, false, VL>;
   typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
   return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
+template <int ACT, int VL>
+int run_vq_bits_vl(const VqCall& c, const GemmShape& s) {
+  switch (c.bits) {
+    case 4: return run_vq<ACT, 4, VL>(c, s);
+    case 8: return run_vq<ACT, 8, VL>(c, s);
+    case 12: return run_vq<ACT, 12, VL>(c, s);
+    default: return run_vq<ACT, 16, VL>(c, s);
+  }
+}
+
 template <int ACT>
 int run_vq_bits(const VqCall& c, const GemmShape& s) {
-  switch (c.bits) {
-    case 4: return run_vq<ACT, 4>(c, s);
-    case 8: return run_vq<ACT, 8>(c, s);
-    case 12: return run_vq<ACT, 12>(c, s);
-    default: return run_vq<ACT, 16>(c, s);
-  }
+  return c.vl == 4 ? run_vq_bits_vl<ACT, 4>(c, s) : run_vq_bits_vl<ACT, 8>(c, s);
 }
 
 template <int ACT, int BM_, int BR_>

@@ -5,28 +5,33 @@ using namespace npamd;
 
 namespace {
 
-template <int ACT, int BITS>
+template <int ACT, int BITS, int VL>
 int run_vq(const VqCall& c, const GemvShape& s) {
   if constexpr (ACT == NPAMD_BF16) {
     if (c.cb_dtype == NPAMD_F16) {
-      using P = VqProvider<ACT, BITS, true>;
+      using P = VqProvider<ACT, BITS, true, VL>;
       typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-      return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, c.nc * 16);
+      return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, (VL == 8 ? c.nc * 16 : (c.nc % 2 == 0 ? c.nc * 8 : 0)));
     }
   }
-  using P = VqProvider<ACT, BITS, false>;
+  using P = VqProvider<ACT, BITS, false, VL>;
   typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, c.nc * 16);
+  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, (VL == 8 ? c.nc * 16 : (c.nc % 2 == 0 ? c.nc * 8 : 0)));
+}
+
+template <int ACT, int VL>
+int run_vq_bits_vl(const VqCall& c, const GemvShape& s) {
+  switch (c.bits) {
+    case 4: return run_vq<ACT, 4, VL>(c, s);
+    case 8: return run_vq<ACT, 8, VL>(c, s);
+    case 12: return run_vq<ACT, 12, VL>(c, s);
+    default: return run_vq<ACT, 16, VL>(c, s);
+  }
 }
 
 template <int ACT>
 int run_vq_bits(const VqCall& c, const GemvShape& s) {
-  switch (c.bits) {
-    case 4: return run_vq<ACT, 4>(c, s);
-    case 8: return run_vq<ACT, 8>(c, s);
-    case 12: return run_vq<ACT, 12>(c, s);
-    default: return run_vq<ACT, 16>(c, s);
-  }
+  return c.vl == 4 ? run_vq_bits_vl<ACT, 4>(c, s) : run_vq_bits_vl<ACT, 8>(c, s);
 }
 
 template <int ACT, int BM_, int BR_>
@@ -45,7 +50,7 @@ int dispatch(const VqCall& c) {
     // The gather is done while x is copied to LDS, which only the MFMA kernel for plain VQ does.
     if (!(fast_ok(c) && !c.packed_r && (int64_t)c.M * c.K <= kGemvLdsActivationsMax && aligned(c.perm, 16)))
       return fail(NPAMD_ERR_UNSUPPORTED,
-                  "%s: column_perm needs VL = 8, 4/8/12/16-bit indices, K %% 64 == 0, 16-byte aligned "
+                  "%s: column_perm needs VL = 8 or 4, 4/8/12/16-bit indices, K %% 64 == 0, 16-byte aligned "
                   "buffers and M * K <= %d (got M=%d K=%d)", c.what, kGemvLdsActivationsMax, c.M, c.K);
     s.perm = c.perm;
   }
@@ -91,11 +96,16 @@ extern "C" int npamd_vq_gemv_perm(const void* x, int64_t ldx, const int32_t* col
   return run(c);
 }
 
+extern "C" int npamd_vq_fused_supported(int K, int vl, int bits) {
+  const bool bits_ok = bits == 4 || bits == 8 || bits == 12 || bits == 16;
+  return (vl == 8 || vl == 4) && bits_ok && K > 0 && K % 64 == 0 ? 1 : 0;
+}
+
 extern "C" int npamd_vq_gemv_perm_supported(int M, int N, int K, int nc, int vl, int bits) {
   const bool bits_ok = bits == 4 || bits == 8 || bits == 12 || bits == 16;
-  if (!(vl == 8 && bits_ok && K > 0 && K % 64 == 0 && M >= 1 && M <= NPAMD_GEMV_MAX_M && N >= 1 && nc >= 1)) return 0;
+  if (!((vl == 8 || vl == 4) && bits_ok && K > 0 && K % 64 == 0 && M >= 1 && M <= NPAMD_GEMV_MAX_M && N >= 1 && nc >= 1)) return 0;
   if ((int64_t)M * K > kGemvLdsActivationsMax) return 0;
-  return gemv_perm_keeps_occupancy(M, N, K / 64, nc * 16) ? 1 : 0;
+  return gemv_perm_keeps_occupancy(M, N, K / 64, vl == 8 ? nc * 16 : (nc % 2 == 0 ? nc * 8 : 0)) ? 1 : 0;
 }
 
 extern "C" int npamd_rvq_gemv(const void* x, int64_t ldx,

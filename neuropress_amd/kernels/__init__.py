@@ -251,6 +251,17 @@ def vq_linear_perm_supported(m: int, n: int, k: int, num_centroids: int, vector_
                                                          int(vector_len), int(bits)))  # fmt: skip
 
 
+def vq_fused_supported(in_features: int, vector_len: int, bits: int) -> bool:
+    """Whether the MFMA GEMV / tile GEMM take a VQ layer of this shape (``npamd_vq_fused_supported``).
+    Other shapes run an element-wise kernel that decodes the weight once per 16 tokens."""
+    return bool(_lib.load().npamd_vq_fused_supported(int(in_features), int(vector_len), int(bits)))
+
+
+def q_fused_supported(in_features: int, nbits: int, group_size: int) -> bool:
+    """The same question for group-quantized layers (``npamd_q_fused_supported``)."""
+    return bool(_lib.load().npamd_q_fused_supported(int(in_features), int(nbits), int(group_size)))
+
+
 class SlicedIndices:
     """Slice-list form of one layer's indices: the blob on the GPU plus a host copy of its header.
 

@@ -268,6 +268,15 @@ class NPLinear(nn.Module):
             self._bias_as(x.dtype),
         )
 
+    def _mfma_layer(self) -> bool:
+        ok = self._derived.get("mfma_layer")
+        if ok is None:
+            from .. import kernels
+
+            ok = kernels.q_fused_supported(self.in_features, self.nbits, self.group_size)
+            self._derived["mfma_layer"] = ok
+        return ok
+
     def _tile_grid_fills_gpu(self, x: torch.Tensor, m: int) -> bool:
         cus = self._derived.get("cus")
         if cus is None:
@@ -288,7 +297,13 @@ class NPLinear(nn.Module):
         try:
             fused_ok = x.dtype in (torch.float16, torch.bfloat16)
             if fused_ok and m > _Q_FUSED_MAX_TOKENS:
-                fused_ok = m <= _Q_TILE_MAX_TOKENS and self._tile_grid_fills_gpu(x, m)
+                # Layers the MFMA kernels do not take (1 / 2 / 8 bits, odd group sizes) would run
+                # an element-wise kernel there: decode once and use the dense GEMM instead.
+                fused_ok = (
+                    m <= _Q_TILE_MAX_TOKENS
+                    and self._mfma_layer()
+                    and self._tile_grid_fills_gpu(x, m)
+                )
             if fused_ok:
                 if m <= _Q_FUSED_MAX_TOKENS:
                     return kernels.q_linear(

@@ -643,6 +643,17 @@ class NPVQLinear(nn.Module):
             return self._forward_dequant_gemm(x)
         return y.reshape(*leading, self.out_features)
 
+    def _mfma_layer(self) -> bool:
+        """Whether the MFMA kernels take this layer's shape (vector length 8, K a multiple of 64)."""
+        ok = self._derived.get("mfma_layer")
+        if ok is None:
+            from .. import kernels
+
+            bits = self.bits if (self.bits in _FAST_BITS or self.bits > 16) else 16  # as _kernel_stream
+            ok = kernels.vq_fused_supported(self.in_features, self.vector_len, bits)
+            self._derived["mfma_layer"] = ok
+        return ok
+
     def _tile_band_ok(self, x: torch.Tensor, m: int) -> bool:
         """True when the tile GEMM's grid (64 columns x up to 384 rows per workgroup,
         times the reduction splits the kernel adds for layers with few output
@@ -651,6 +662,8 @@ class NPVQLinear(nn.Module):
             return True
         if self.is_residual and self.in_features < _RVQ_TILE_MIN_K:
             return False
+        if not self._mfma_layer():
+            return False  # the tile entry point would run its element-wise fallback
         cus = self._derived.get("cus")
         if cus is None:
             cus = torch.cuda.get_device_properties(x.device).multi_processor_count

@@ -43,15 +43,30 @@ def test_vq_dequant_bit_exact(gpu, oracle_lib, bits, dtype, vl):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nc,bits", [(4096, 12), (3000, 12), (4096, 16), (2049, 13)])
-def test_vq_dequant_lds_codebook_bit_exact(gpu, oracle_lib, dtype, nc, bits):
-    """Layers of at least 2^20 vectors with a 2049..4096-row codebook decode from an LDS copy of the
-    table (512 blocks, each a contiguous run of vectors).  2050 rows of 4096 columns: the last
-    block's run is ragged.  Checked bit for bit against the oracle."""
+@pytest.mark.parametrize("bits", [8, 11, 16])
+def test_vq_dequant_vl4_odd_vector_count(gpu, oracle_lib, dtype, bits):
+    """Vector length 4 decodes two vectors per thread; 37 rows of 3 vectors leave a single one at
+    the end."""
+    from neuropress_amd import kernels
+
+    n, k = 37, 12
+    L = cases.vq_layer(170 + bits, n, k, min(1 << bits, 2048), vl=4, bits=bits, std=1.0)
+    ref = oracle_lib.vq_decode(L["packed"].numpy(), bits, orc.to_bits(L["cb"]), n, k, orc.torch_dtype_code(dtype))
+    _bits_equal(kernels.vq_dequant(L["packed"].to(gpu), L["cb"].to(gpu), bits, n, k, dtype), ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nc,bits,vl", [(4096, 12, 8), (3000, 12, 8), (4096, 16, 8), (1025, 11, 8),
+                                        (4096, 12, 4), (8192, 13, 4), (3001, 16, 4)])
+def test_vq_dequant_lds_codebook_bit_exact(gpu, oracle_lib, dtype, nc, bits, vl):
+    """Layers of at least 2^20 vectors with a table of 16 to 64 KiB decode from an LDS copy of it
+    (512 blocks, each a contiguous run of vectors), for vector length 8 and 4 (an odd row count
+    with VL = 4 ends in half a 16-byte unit).  2050 rows of 4096 columns: the last block's run
+    is ragged.  Checked bit for bit against the oracle."""
     from neuropress_amd import kernels
 
     n, k = 2050, 4096
-    L = cases.vq_layer(300 + nc + bits, n, k, nc, bits=bits, std=1.0)
+    L = cases.vq_layer(300 + nc + bits, n, k, nc, vl=vl, bits=bits, std=1.0)
     ref = oracle_lib.vq_decode(L["packed"].numpy(), bits, orc.to_bits(L["cb"]), n, k, orc.torch_dtype_code(dtype))
     out = kernels.vq_dequant(L["packed"].to(gpu), L["cb"].to(gpu), bits, n, k, dtype)
     _bits_equal(out, ref)
@@ -137,12 +152,14 @@ def _check(y: torch.Tensor, ref: np.ndarray):
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,nc", [(4, 16), (8, 256), (12, 4096), (16, 65536)])
 @pytest.mark.parametrize("m", [1, 2, 5, 16])
-def test_vq_gemv_fast_path(gpu, oracle_lib, act, bits, nc, m):
+@pytest.mark.parametrize("vl", [8, 4])
+def test_vq_gemv_fast_path(gpu, oracle_lib, act, bits, nc, m, vl):
     from neuropress_amd import kernels
 
     # N not a multiple of 16, K = 5 chunks of 64 (not a multiple of the 256-k step).
-    L = cases.vq_layer(200 + bits + m, 100, 320, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
-    y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 8,
+    # Vector length 4 (the reference's default, np_vq_linear.py:109): two codebook rows per operand.
+    L = cases.vq_layer(200 + bits + m, 100, 320, nc, vl=vl, bits=bits, act=act, m=m, bias=True, std=0.05)
+    y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, vl,
                           L["bias"].to(gpu), out_features=100)
     assert y.shape == (m, 100) and y.dtype == act
     _check(y, _vq_ref(oracle_lib, L, act))
@@ -151,25 +168,26 @@ def test_vq_gemv_fast_path(gpu, oracle_lib, act, bits, nc, m):
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,nc", [(4, 16), (8, 256), (12, 4096), (16, 65536)])
 @pytest.mark.parametrize("m", [1, 2, 5, 16])
-def test_vq_gemv_column_perm(gpu, oracle_lib, act, bits, nc, m):
+@pytest.mark.parametrize("vl", [8, 4])
+def test_vq_gemv_column_perm(gpu, oracle_lib, act, bits, nc, m, vl):
     """npamd_vq_gemv_perm == the plain GEMV fed with x[:, column_perm] (reference:
     np_vq_linear.py:1027-1028), checked against the oracle on the permuted activations.  x has a
     row stride larger than K, so a kernel that ignored the permutation or the stride would fail."""
     from neuropress_amd import kernels
 
     n, k = 100, 320
-    L = cases.vq_layer(700 + bits + m, n, k, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
+    L = cases.vq_layer(700 + bits + m, n, k, nc, vl=vl, bits=bits, act=act, m=m, bias=True, std=0.05)
     perm = torch.randperm(k, generator=cases.gen(9 + m))
     xw = torch.zeros(m, k + 64, dtype=act)
     xw[:, :k] = L["x"]
     x_gpu = xw.to(gpu)[:, :k]  # stride k + 64
-    assert kernels.vq_linear_perm_supported(m, n, k, nc, 8, bits)
-    y = kernels.vq_linear(x_gpu, L["packed"].to(gpu), L["cb"].to(gpu), bits, 8, L["bias"].to(gpu),
+    assert kernels.vq_linear_perm_supported(m, n, k, nc, vl, bits)
+    y = kernels.vq_linear(x_gpu, L["packed"].to(gpu), L["cb"].to(gpu), bits, vl, L["bias"].to(gpu),
                           out_features=n, column_perm=perm.to(torch.int32).to(gpu))
     assert y.shape == (m, n) and y.dtype == act
     _check(y, _vq_ref(oracle_lib, dict(L, x=L["x"][:, perm].contiguous()), act))
     # bit-identical to the unpermuted kernel on pre-gathered activations
-    y2 = kernels.vq_linear(L["x"][:, perm].contiguous().to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 8,
+    y2 = kernels.vq_linear(L["x"][:, perm].contiguous().to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, vl,
                            L["bias"].to(gpu), out_features=n)
     assert torch.equal(y, y2)
 
@@ -233,11 +251,12 @@ def test_vq_gemm_tile_reference_shapes(gpu, oracle_lib, bits, m):
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,nc", [(8, 256), (12, 4096), (16, 65536)])
 @pytest.mark.parametrize("m", [1, 17, 96, 130, 300])
-def test_vq_gemm_tile_fast_path(gpu, oracle_lib, act, bits, nc, m):
+@pytest.mark.parametrize("vl", [8, 4])
+def test_vq_gemm_tile_fast_path(gpu, oracle_lib, act, bits, nc, m, vl):
     from neuropress_amd import kernels
 
     # N = 300 spans two 256-column blocks with a ragged tail; K = 448 = 3.5 macro-steps.
-    L = cases.vq_layer(500 + bits + m, 300, 448, nc, bits=bits, act=act, m=m, bias=True, std=0.05)
+    L = cases.vq_layer(500 + bits + m, 300, 448, nc, vl=vl, bits=bits, act=act, m=m, bias=True, std=0.05)
     y = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 300, L["bias"].to(gpu))
     _check(y, _vq_ref(oracle_lib, L, act))
 
@@ -350,7 +369,7 @@ def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("kind", ["vq12", "vq16", "rvq", "q4", "q4_asym", "q4_asym_gs128"])
+@pytest.mark.parametrize("kind", ["vq12", "vq16", "vq12_vl4", "vq16_vl4", "vq10_vl4", "rvq", "q4", "q4_asym", "q4_asym_gs128", "q8", "q2_asym"])
 def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
     """One-hot activations read the decoded weight back through the contraction kernels: with
     x = rows of the identity, y[m, n] is the single product 1 * W[n, k_m], which f32 accumulation
@@ -361,11 +380,12 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
 
     n, k = 200, 512
     if kind.startswith("vq"):
-        bits = int(kind[2:])
-        L = cases.vq_layer(61 + bits, n, k, 1 << bits, bits=bits, act=act, m=1, std=0.05)
+        bits = int(kind[2:4])
+        vl = 4 if kind.endswith("vl4") else 8  # 10-bit stream: the element-wise kernels
+        L = cases.vq_layer(61 + bits, n, k, 1 << bits, vl=vl, bits=bits, act=act, m=1, std=0.05)
         pk, cb = L["packed"].to(gpu), L["cb"].to(gpu)
         w = kernels.vq_dequant(pk, cb, bits, n, k, act)
-        gemv = lambda x: kernels.vq_linear(x, pk, cb, bits, 8, None, n)
+        gemv = lambda x: kernels.vq_linear(x, pk, cb, bits, vl, None, n)
         tile = lambda x: kernels.vq_gemm_tile(x, pk, cb, bits, n, None)
     elif kind == "rvq":
         L = cases.rvq_layer(62, n, k, act=act, m=1)
@@ -375,13 +395,14 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
         gemv = lambda x: kernels.rvq_linear(x, *args, None, tile=False)
         tile = lambda x: kernels.rvq_linear(x, *args, None, tile=True)
     else:
+        nbits = int(kind[1])  # 8 and 2 bits: the element-wise kernels
         gs = 128 if kind.endswith("gs128") else 32
-        L = cases.q4_layer(63, n, k, gs=gs, act=act, m=1, asym=kind.startswith("q4_asym"))
+        L = cases.q4_layer(63, n, k, nbits=nbits, gs=gs, act=act, m=1, asym="asym" in kind)
         blob, sc = L["blob"].to(gpu), L["scale"].to(gpu)
         zp = None if L["zp"] is None else L["zp"].to(gpu)
-        w = kernels.q_dequant(blob, sc, 4, gs, zp, act)
-        gemv = lambda x: kernels.q_linear(x, blob, sc, 4, gs, zp)
-        tile = lambda x: kernels.q_gemm_tile(x, blob, sc, 4, gs, zp)
+        w = kernels.q_dequant(blob, sc, nbits, gs, zp, act)
+        gemv = lambda x: kernels.q_linear(x, blob, sc, nbits, gs, zp)
+        tile = lambda x: kernels.q_gemm_tile(x, blob, sc, nbits, gs, zp)
     eye = torch.eye(k, dtype=act, device=gpu)
     wt = w.t().contiguous()  # [K, N]: row k is what token "one-hot k" must produce
     for k0 in (0, 48, k - 16):

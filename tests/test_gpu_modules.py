@@ -132,6 +132,32 @@ def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch
         assert calls == expect
 
 
+def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch):
+    """8-bit group quantization and vector length 2 have no MFMA kernel: up to 16 tokens they run
+    the element-wise GEMV, beyond that the modules decode once and call the dense GEMM instead of
+    the tile entry points (which would decode the weight once per 16 tokens)."""
+    import neuropress_amd.nn.np_linear as qmod
+    from neuropress_amd import kernels
+
+    calls = []
+    for name in ("vq_gemm_tile", "q_gemm_tile", "vq_dequant", "q_dequant"):
+        real = getattr(kernels, name)
+        monkeypatch.setattr(kernels, name, lambda *a, _real=real, _name=name, **kw: (calls.append(_name), _real(*a, **kw))[1])
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
+    monkeypatch.setattr(qmod, "_Q_TILE_MIN_GRID_FRACTION", 0.0)
+    Q = cases.q4_layer(81, 96, 256, nbits=8, bias=True)
+    qlayer = NPLinear(Q["blob"], Q["scale"], 96, 256, 32, 8, "sym", "cuda", bias=Q["bias"].float()).to(gpu)
+    wq = ((Q["codes"].float() - 128).reshape(96, 8, 32) * Q["scale"].float().reshape(96, 8, 1)).reshape(96, 256)
+    L = cases.vq_layer(82, 96, 256, 1024, vl=2, bits=10, bias=True, std=0.05)
+    layer = NPVQLinear(VQProxy(L["cb"]).to(gpu), L["packed"], 10, 96, 256, 2, "cuda_wmma", bias=L["bias"].float()).to(gpu)
+    w = L["cb"][L["idx"]].reshape(96, 256).half().float()
+    for m in (3, 40):
+        x = (torch.randn(m, 256, generator=cases.gen(m)) * 0.5).half()
+        _close(qlayer(x.to(gpu)), torch.nn.functional.linear(x.float(), wq.half().float(), Q["bias"].float()))
+        _close(layer(x.to(gpu)), torch.nn.functional.linear(x.float(), w, L["bias"].float()))
+    assert calls == ["q_dequant", "vq_dequant"]  # 40 tokens only; nothing went to a tile entry point
+
+
 def test_narrow_layers_take_the_split_tile_band(gpu, monkeypatch):
     """A 2048 x 4096 layer has 32 column tiles: the module still routes 17..128 tokens
     to the tile GEMM (which splits the reduction), and more tokens to decode + GEMM."""

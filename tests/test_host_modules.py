@@ -371,8 +371,19 @@ def test_c_abi_validates_arguments_without_a_gpu():
         _lib.call("npamd_vq_gemv_perm", 16, 8192, 16, 16, 1 << 20, 16, 16, 0, 65536, 8, None, 16, 64, 9, 64, 8192, 0, None)
     lib = _lib.load()
     assert lib.npamd_vq_gemv_perm_supported(1, 2048, 2048, 4096, 8, 12) == 1
-    assert lib.npamd_vq_gemv_perm_supported(1, 2048, 2048, 4096, 4, 12) == 0  # vector length 4
+    assert lib.npamd_vq_gemv_perm_supported(1, 2048, 2048, 4096, 4, 12) == 1  # vector length 4
+    assert lib.npamd_vq_gemv_perm_supported(1, 2048, 2048, 4096, 6, 12) == 0  # vector length 6
     assert lib.npamd_vq_gemv_perm_supported(5, 2048, 4096, 4096, 8, 12) == 0  # 5 * 4096 elements > 16384
+    # which layers the MFMA kernels take (the rest run element-wise kernels; the modules send
+    # them to decode + GEMM beyond 16 tokens)
+    assert lib.npamd_vq_fused_supported(4096, 8, 12) == 1 and lib.npamd_vq_fused_supported(4096, 8, 16) == 1
+    assert lib.npamd_vq_fused_supported(4096, 4, 12) == 1  # vector length 4: two rows per operand
+    assert lib.npamd_vq_fused_supported(4096, 2, 12) == 0 and lib.npamd_vq_fused_supported(4096, 16, 12) == 0
+    assert lib.npamd_vq_fused_supported(4096, 8, 10) == 0  # 10-bit stream (the module widens it to 16 first)
+    assert lib.npamd_vq_fused_supported(4096 + 32, 8, 12) == 0  # K not a multiple of 64
+    assert lib.npamd_q_fused_supported(4096, 4, 32) == 1 and lib.npamd_q_fused_supported(4096, 4, 128) == 1
+    assert lib.npamd_q_fused_supported(4096, 8, 32) == 0 and lib.npamd_q_fused_supported(4096, 4, 96) == 0
+    assert lib.npamd_q_fused_supported(4096, 4, 16) == 0 and lib.npamd_q_fused_supported(4096 + 32, 4, 32) == 0
 
 
 def test_tile_band_rule_counts_reduction_splits():
