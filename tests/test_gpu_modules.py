@@ -28,14 +28,17 @@ def _close(y_gpu, y_ref):
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("bits,nc", [(8, 256), (10, 1024), (12, 4096), (16, 65536)])
-def test_npvqlinear_all_bands_match_default(gpu, act, bits, nc, monkeypatch):
+@pytest.mark.parametrize("vl", [8, 4])
+def test_npvqlinear_all_bands_match_default(gpu, act, bits, nc, vl, monkeypatch):
+    """Vector length 8 (the benchmark configurations) and 4 (the reference's default)."""
     monkeypatch.setattr(vqmod, "_FUSED_MAX_TOKENS", 16)
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)  # small layers: force the tile band
-    L = cases.vq_layer(40 + bits, 96, 256, nc, bits=bits, bias=True, std=0.05)
-    ref_layer = NPVQLinear(VQProxy(L["cb"]), L["packed"], bits, 96, 256, 8, "default", bias=L["bias"].float())
+    L = cases.vq_layer(40 + bits, 96, 256, nc, vl=vl, bits=bits, bias=True, std=0.05)
+    ref_layer = NPVQLinear(VQProxy(L["cb"]), L["packed"], bits, 96, 256, vl, "default", bias=L["bias"].float())
     proxy = VQProxy(L["cb"]).to(gpu)
-    layer = NPVQLinear(proxy, L["packed"], bits, 96, 256, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
+    layer = NPVQLinear(proxy, L["packed"], bits, 96, 256, vl, "cuda_wmma", bias=L["bias"].float()).to(gpu)
+    assert layer._mfma_layer()
     for shape in [(1, 256), (2, 8, 256), (40, 256), (3, 50, 256)]:  # fused, fused(16), tile, dense
         x = torch.randn(*shape, generator=cases.gen(1)).to(act)
         y = layer(x.to(gpu))
