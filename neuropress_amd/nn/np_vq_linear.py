@@ -546,6 +546,11 @@ class NPVQLinear(nn.Module):
         if self.backend in _FUSED_BACKENDS:
             if x.dtype not in (torch.float16, torch.bfloat16):
                 return self._forward_dequant_gemm(x)  # fp32 activations: decode + GEMM
+            if x.is_cuda and not self._mfma_layer():
+                # Shapes without an MFMA kernel (vector lengths other than 8 and 4, K not a
+                # multiple of 64): the element-wise GEMV is slower than decoding once and calling
+                # the dense GEMM at every token count (14336 x 4096: 99 us against 57 us at one token).
+                return self._forward_dequant_gemm(x)
             m = x.numel() // self.in_features
             if m > _fused_max_tokens(self.backend):
                 if (

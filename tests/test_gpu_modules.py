@@ -136,14 +136,14 @@ def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch
 
 
 def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch):
-    """8-bit group quantization and vector length 2 have no MFMA kernel: up to 16 tokens they run
-    the element-wise GEMV, beyond that the modules decode once and call the dense GEMM instead of
-    the tile entry points (which would decode the weight once per 16 tokens)."""
+    """8-bit group quantization and vector length 2 have no MFMA kernel: the modules decode once and
+    call the dense GEMM at every token count instead of the fused entry points (whose element-wise
+    kernels decode the weight once per 16 tokens)."""
     import neuropress_amd.nn.np_linear as qmod
     from neuropress_amd import kernels
 
     calls = []
-    for name in ("vq_gemm_tile", "q_gemm_tile", "vq_dequant", "q_dequant"):
+    for name in ("vq_gemm_tile", "q_gemm_tile", "vq_linear", "q_linear", "vq_dequant", "q_dequant"):
         real = getattr(kernels, name)
         monkeypatch.setattr(kernels, name, lambda *a, _real=real, _name=name, **kw: (calls.append(_name), _real(*a, **kw))[1])
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
@@ -158,7 +158,7 @@ def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch)
         x = (torch.randn(m, 256, generator=cases.gen(m)) * 0.5).half()
         _close(qlayer(x.to(gpu)), torch.nn.functional.linear(x.float(), wq.half().float(), Q["bias"].float()))
         _close(layer(x.to(gpu)), torch.nn.functional.linear(x.float(), w, L["bias"].float()))
-    assert calls == ["q_dequant", "vq_dequant"]  # 40 tokens only; nothing went to a tile entry point
+    assert calls == ["q_dequant", "vq_dequant"] * 2  # nothing went to a fused entry point
 
 
 def test_narrow_layers_take_the_split_tile_band(gpu, monkeypatch):
