@@ -248,9 +248,9 @@ int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, const void* ze
                     int N, int K, int nbits, int group_size, void* out, int out_dtype,
                     void* stream);
 
-/* 1 when the MFMA kernels behind npamd_q_gemv / npamd_q_gemm_tile take the layer (4 bits, with or
+/* 1 when the MFMA kernels behind npamd_q_gemv / npamd_q_gemm_tile take the layer (4 or 8 bits, with or
  * without zero points, group size 32 * 2^j, K % 64 == 0), pointer alignment aside; 0 when they would
- * run the element-wise fallback (1 / 2 / 8 bits, other group sizes), which decodes the weight once per
+ * run the element-wise fallback (1 / 2 bits, other group sizes), which decodes the weight once per
  * 16 tokens: beyond 16 tokens use npamd_q_dequant and a dense GEMM.  The reference runs its one GEMV
  * kernel at every token count (neuropress/kernels/q4_linear.cu:137-139).  Host-only arithmetic. */
 int npamd_q_fused_supported(int K, int nbits, int group_size);

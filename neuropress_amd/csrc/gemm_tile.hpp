@@ -21,9 +21,7 @@
 //   x tile  [BM][64 k], two or three buffers.  Every consumer fetches only the
 //           rows it owns, one or more steps ahead, so the x tile needs no
 //           synchronisation between waves.  The bytes go from memory straight
-//           into LDS (swizzled 128-byte rows) unless the provider reorders
-//           them on the way (then through registers, rows padded to 144 bytes);
-//           see XStage.
+//           into LDS (swizzled 128-byte rows); see XStage.
 //   W tile  [64][64 k], rows padded to 144 bytes, a ring of three.  Every
 //           producer decodes a quarter of every step's tile (16 columns x 8 operands; lane = column x
 //           operand pair), keeps kDepth steps in flight in registers and
@@ -78,22 +76,18 @@ __device__ __forceinline__ void block_sync_lds() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// How the x tile reaches LDS.
-//   Direct (providers that take x as it lies in memory): `global_load_lds_dwordx4` writes the
-//   loaded bytes straight into LDS, 64 lanes x 16 bytes = 1 KiB contiguous per instruction, with
-//   no register, no LDS store instruction and nothing for the issuing wave to wait for until the
-//   tile is read.  Rows are 128 bytes, unpadded (the transfer fills a contiguous KiB), and the
-//   16-byte piece p of row r lies in slot p ^ ((r >> 1) & 7) of its row: a 16-byte read of 32
-//   consecutive rows then touches every 16-byte bank group twice, as with padded rows.  A lane may
-//   fetch any source address, so the swizzle costs nothing at the load.  kBufs tiles are in LDS,
-//   requested kBufs - 1 steps ahead.
-//   Through registers (int4, whose A operands change their k order on the way): padded rows,
-//   two tiles.
-template <class Provider, int MW>
+// How the x tile reaches LDS: `global_load_lds_dwordx4` writes the loaded bytes straight into
+// LDS, 64 lanes x 16 bytes = 1 KiB contiguous per instruction, with no register, no LDS store
+// instruction and nothing for the issuing wave to wait for until the tile is read.  Rows are
+// 128 bytes, unpadded (the transfer fills a contiguous KiB), and the 16-byte piece p of row r
+// lies in slot p ^ ((r >> 1) & 7) of its row: a 16-byte read of 32 consecutive rows then touches
+// every 16-byte bank group twice, as with padded rows.  A lane may fetch any source address, so
+// the swizzle costs nothing at the load.  kBufs tiles are in LDS.  (Every provider takes x as
+// it lies in memory; one that reordered k inside an operand would have to go through registers.)
+template <int MW>
 struct XStage {
-  static constexpr bool kDirect = !Provider::kPermuteA;
-  static constexpr int kBufs = kDirect ? (MW == 3 ? 2 : 3) : 2;
-  static constexpr int kXRowBytes = kDirect ? kStepK * 2 : kRowBytes;
+  static constexpr int kBufs = MW == 3 ? 2 : 3;
+  static constexpr int kXRowBytes = kStepK * 2;
   static constexpr int kBufBytes = 128 * MW * kXRowBytes;
   static constexpr int kLdsBytes = kBufs * kBufBytes + kWRing * kWBufBytes;
 };
@@ -102,7 +96,7 @@ template <int ACT, class Provider, int MW>
 __global__ void __launch_bounds__(512)
 tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  using XS = XStage<Provider, MW>;
+  using XS = XStage<MW>;
   constexpr int BM = 128 * MW;
   constexpr int kXBufBytes = XS::kBufBytes;
   uint8_t* const xs = lds;                             // [XS::kBufs][BM][XS::kXRowBytes]
@@ -213,218 +207,119 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
 
-  if constexpr (XS::kDirect) {
-    // ---- x tile by LDS-direct loads --------------------------------------------------------
-    // Instruction i of a tile covers the wave's rows 8i .. 8i+7: lane l fills slot l & 7 of row
-    // 8i + (l >> 3), i.e. fetches piece (l & 7) ^ ((row >> 1) & 7) of that row.  The address is
-    // a scalar base (the wave's first row, this step's chunk) plus a 32-bit lane offset.
-    constexpr int kPiecesW = 4 * MW;
-    constexpr int kBufs = XS::kBufs;
-    const int base_row = min(m0 + wrow0, s.M - 1);          // waves past M re-read the last row
-    const uint8_t* const xbase = reinterpret_cast<const uint8_t*>(xg + (int64_t)base_row * s.ldx);
-    uint32_t voff[kPiecesW];
+  // ---- x tile by LDS-direct loads --------------------------------------------------------
+  // Instruction i of a tile covers the wave's rows 8i .. 8i+7: lane l fills slot l & 7 of row
+  // 8i + (l >> 3), i.e. fetches piece (l & 7) ^ ((row >> 1) & 7) of that row.  The address is
+  // a scalar base (the wave's first row, this step's chunk) plus a 32-bit lane offset.
+  constexpr int kPiecesW = 4 * MW;
+  constexpr int kBufs = XS::kBufs;
+  const int base_row = min(m0 + wrow0, s.M - 1);          // waves past M re-read the last row
+  const uint8_t* const xbase = reinterpret_cast<const uint8_t*>(xg + (int64_t)base_row * s.ldx);
+  uint32_t voff[kPiecesW];
 #pragma unroll
-    for (int i = 0; i < kPiecesW; ++i) {
-      const int r = 8 * i + (lane >> 3);
-      const int piece = (lane & 7) ^ ((r >> 1) & 7);
-      voff[i] = (uint32_t)(((int64_t)min(r, s.M - 1 - base_row) * s.ldx + piece * 8) * 2);
-    }
-    const uint32_t xs_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)xs;
-    const uint32_t wave_lds = xs_lds + (uint32_t)(wrow0 * XS::kXRowBytes);
-    auto fetch_piece = [&](int i, int buf, const uint8_t* src) {
-      const uint32_t dst = __builtin_amdgcn_readfirstlane(wave_lds + (uint32_t)(buf * kXBufBytes + i * 1024));
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(dst), "v"(voff[i]), "s"(src) : "memory");
-    };
-    auto tile_src = [&](int step) { return xbase + (int64_t)chunk_of(min(step, steps - 1)) * (kStepK * 2); };
-    // The consumers issue no other vector memory instruction in the loop, so the in-order
-    // counter counts tiles: with tiles up to step + kBufs - 1 requested, tile step + 1 has
-    // landed once at most (kBufs - 2) tiles' worth of loads are outstanding.
-    constexpr int kOutstandingOk = (kBufs - 2) * kPiecesW;
+  for (int i = 0; i < kPiecesW; ++i) {
+    const int r = 8 * i + (lane >> 3);
+    const int piece = (lane & 7) ^ ((r >> 1) & 7);
+    voff[i] = (uint32_t)(((int64_t)min(r, s.M - 1 - base_row) * s.ldx + piece * 8) * 2);
+  }
+  const uint32_t xs_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)xs;
+  const uint32_t wave_lds = xs_lds + (uint32_t)(wrow0 * XS::kXRowBytes);
+  auto fetch_piece = [&](int i, int buf, const uint8_t* src) {
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(wave_lds + (uint32_t)(buf * kXBufBytes + i * 1024));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(dst), "v"(voff[i]), "s"(src) : "memory");
+  };
+  auto tile_src = [&](int step) { return xbase + (int64_t)chunk_of(min(step, steps - 1)) * (kStepK * 2); };
+  // The consumers issue no other vector memory instruction in the loop, so the in-order
+  // counter counts tiles: with tiles up to step + kBufs - 1 requested, tile step + 1 has
+  // landed once at most (kBufs - 2) tiles' worth of loads are outstanding.
+  constexpr int kOutstandingOk = (kBufs - 2) * kPiecesW;
 
-    // With three tiles in LDS, tile step + 2 is requested behind the MFMAs of k groups 0..2 of
-    // step `step` (its buffer held tile step - 1).  With two, there is no such slack: tile
-    // step + 2 goes into the buffer of tile `step` itself, as soon as that tile's last operands
-    // have been read (behind the MFMAs of group 3), which leaves it almost two steps to arrive.
-    constexpr bool kIssueAtEnd = kBufs == 2;
-    constexpr int kPrologueTiles = kIssueAtEnd ? kBufs : kBufs - 1;
+  // With three tiles in LDS, tile step + 2 is requested behind the MFMAs of k groups 0..2 of
+  // step `step` (its buffer held tile step - 1).  With two, there is no such slack: tile
+  // step + 2 goes into the buffer of tile `step` itself, as soon as that tile's last operands
+  // have been read (behind the MFMAs of group 3), which leaves it almost two steps to arrive.
+  constexpr bool kIssueAtEnd = kBufs == 2;
+  constexpr int kPrologueTiles = kIssueAtEnd ? kBufs : kBufs - 1;
 #pragma unroll
-    for (int p = 0; p < kPrologueTiles; ++p) {
-      const uint8_t* src = tile_src(p);
+  for (int p = 0; p < kPrologueTiles; ++p) {
+    const uint8_t* src = tile_src(p);
 #pragma unroll
-      for (int i = 0; i < kPiecesW; ++i) fetch_piece(i, p, src);
-    }
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kPrologueTiles - 1) * kPiecesW) : "memory");
-    block_sync_lds();
+    for (int i = 0; i < kPiecesW; ++i) fetch_piece(i, p, src);
+  }
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kPrologueTiles - 1) * kPiecesW) : "memory");
+  block_sync_lds();
 
-    u32x4 a[2][MW], b[2][2];
-    const uint32_t row_off = (uint32_t)((wrow0 + c) * XS::kXRowBytes);
-    uint32_t slot_off[4];
+  u32x4 a[2][MW], b[2][2];
+  const uint32_t row_off = (uint32_t)((wrow0 + c) * XS::kXRowBytes);
+  uint32_t slot_off[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) slot_off[j] = (uint32_t)((((h << 2) | j) ^ ((c >> 1) & 7)) << 4);
-    auto read_ops = [&](int set, int buf, int wslot, int j) {
-      const uint8_t* xa = xs + buf * kXBufBytes + row_off + slot_off[j];
-      const uint8_t* wb = ws + wslot * kWBufBytes + c * kRowBytes + h * 64 + j * 16;
-      b[set][0] = *reinterpret_cast<const u32x4*>(wb);
-      b[set][1] = *reinterpret_cast<const u32x4*>(wb + 32 * kRowBytes);
+  for (int j = 0; j < 4; ++j) slot_off[j] = (uint32_t)((((h << 2) | j) ^ ((c >> 1) & 7)) << 4);
+  auto read_ops = [&](int set, int buf, int wslot, int j) {
+    const uint8_t* xa = xs + buf * kXBufBytes + row_off + slot_off[j];
+    const uint8_t* wb = ws + wslot * kWBufBytes + c * kRowBytes + h * 64 + j * 16;
+    b[set][0] = *reinterpret_cast<const u32x4*>(wb);
+    b[set][1] = *reinterpret_cast<const u32x4*>(wb + 32 * kRowBytes);
 #pragma unroll
-      for (int mt = 0; mt < MW; ++mt)
-        a[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * XS::kXRowBytes);
-    };
-    constexpr int kPieceOfGroup[4] = {0, (kPiecesW + 2) / 3, (2 * kPiecesW + 2) / 3, kPiecesW};
+    for (int mt = 0; mt < MW; ++mt)
+      a[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * XS::kXRowBytes);
+  };
+  constexpr int kPieceOfGroup[4] = {0, (kPiecesW + 2) / 3, (2 * kPiecesW + 2) / 3, kPiecesW};
 
-    // buf = step % kBufs (compile-time through the unrolled loops below).
-    auto one_step = [&](int buf, int step, int wslot) {
-      const int wnext = wslot == kWRing - 1 ? 0 : wslot + 1;
-      const int nbuf = buf == kBufs - 1 ? 0 : buf + 1;
-      const int fbuf = kIssueAtEnd ? buf : (buf == 0 ? kBufs - 1 : buf - 1);  // where the requested tile goes
-      const uint8_t* src = tile_src(kIssueAtEnd ? step + kBufs : step + kBufs - 1);
+  // buf = step % kBufs (compile-time through the unrolled loops below).
+  auto one_step = [&](int buf, int step, int wslot) {
+    const int wnext = wslot == kWRing - 1 ? 0 : wslot + 1;
+    const int nbuf = buf == kBufs - 1 ? 0 : buf + 1;
+    const int fbuf = kIssueAtEnd ? buf : (buf == 0 ? kBufs - 1 : buf - 1);  // where the requested tile goes
+    const uint8_t* src = tile_src(kIssueAtEnd ? step + kBufs : step + kBufs - 1);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (j < 3) {
-          read_ops((j + 1) & 1, buf, wslot, j + 1);
-        } else {
-          asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kOutstandingOk) : "memory");
-          read_ops(0, nbuf, wnext, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int mt = 0; mt < MW; ++mt) {
-          acc[mt][0] = mfma32<ACT>(a[j & 1][mt], b[j & 1][0], acc[mt][0]);
-          acc[mt][1] = mfma32<ACT>(a[j & 1][mt], b[j & 1][1], acc[mt][1]);
-        }
-        if (!kIssueAtEnd && j < 3) {
-#pragma unroll
-          for (int i = kPieceOfGroup[j]; i < kPieceOfGroup[j + 1]; ++i) fetch_piece(i, fbuf, src);
-        }
-        if (kIssueAtEnd && j == 3) {
-#pragma unroll
-          for (int i = 0; i < kPiecesW; ++i) fetch_piece(i, fbuf, src);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int j = 0; j < 4; ++j) {
+      if (j < 3) {
+        read_ops((j + 1) & 1, buf, wslot, j + 1);
+      } else {
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kOutstandingOk) : "memory");
+        read_ops(0, nbuf, wnext, 0);
       }
-    };
-
-    read_ops(0, 0, 0, 0);
-    int wslot = 0;
-    const int whole = steps / kBufs * kBufs;
-    for (int t0 = 0; t0 < whole; t0 += kBufs) {
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int d = 0; d < kBufs; ++d) {
-        one_step(d, t0 + d, wslot);
-        wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
-        block_sync_lds();
+      for (int mt = 0; mt < MW; ++mt) {
+        acc[mt][0] = mfma32<ACT>(a[j & 1][mt], b[j & 1][0], acc[mt][0]);
+        acc[mt][1] = mfma32<ACT>(a[j & 1][mt], b[j & 1][1], acc[mt][1]);
       }
+      if (!kIssueAtEnd && j < 3) {
+#pragma unroll
+        for (int i = kPieceOfGroup[j]; i < kPieceOfGroup[j + 1]; ++i) fetch_piece(i, fbuf, src);
+      }
+      if (kIssueAtEnd && j == 3) {
+#pragma unroll
+        for (int i = 0; i < kPiecesW; ++i) fetch_piece(i, fbuf, src);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
+
+  read_ops(0, 0, 0, 0);
+  int wslot = 0;
+  const int whole = steps / kBufs * kBufs;
+  for (int t0 = 0; t0 < whole; t0 += kBufs) {
 #pragma unroll
     for (int d = 0; d < kBufs; ++d) {
-      if (whole + d < steps) {
-        one_step(d, whole + d, wslot);
-        wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
-        block_sync_lds();
-      }
+      one_step(d, t0 + d, wslot);
+      wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
+      block_sync_lds();
     }
-    for (int t = steps; t < total; ++t) block_sync_lds();
-    // Nothing may still be on its way into LDS when the wave ends (the block's LDS is handed on).
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  } else {
-    // The wave's own rows of the x tile: piece i of lane l is row wrow0 + (l >> 3) + 8 i, 16-byte
-    // column l & 7 (eight rows of 128 bytes per load instruction).
-    constexpr int kPiecesW = 4 * MW;
-    const int prow = lane >> 3, pcol8 = lane & 7;
-    auto x_src = [&](int i, int step) {
-      const int m = min(m0 + wrow0 + prow + 8 * i, s.M - 1);  // rows past M: clamped, never stored
-      return reinterpret_cast<const u32x4*>(xg + (int64_t)m * s.ldx + chunk_of(min(step, steps - 1)) * kStepK + pcol8 * 8);
-    };
-    auto x_dst = [&](int i, int buf) {
-      return reinterpret_cast<u32x4*>(xs + buf * kXBufBytes + (wrow0 + prow + 8 * i) * kRowBytes + pcol8 * 16);
-    };
-    // A provider that wants the k order of its A operands changed gets it at the LDS store, when
-    // the loaded value has long arrived (at the load, the shuffle would wait for it on the spot).
-    auto load_piece = [&](u32x4& r, int i, int step) { r = *x_src(i, step); };
-    auto store_piece = [&](const u32x4& r, int i, int buf) {
-      if constexpr (Provider::kPermuteA) *x_dst(i, buf) = permute_a_0415(r);
-      else *x_dst(i, buf) = r;
-    };
-
-    // x tile pipeline: kXDepth register sets hold the tiles of the next steps in flight (a global
-    // load takes longer than one iteration).  Step p lives in set p % kXDepth; iteration t writes
-    // tile t+1 to LDS and reloads its set with tile t+1+kXDepth.
-    constexpr int kXDepth = (MW == 1) ? 4 : (MW == 2) ? 2 : 1;
-    u32x4 xr[kXDepth][kPiecesW];
-  #pragma unroll
-    for (int i = 0; i < kPiecesW; ++i) {
-      load_piece(xr[0][i], i, 0);
-      store_piece(xr[0][i], i, 0);
-    }
-  #pragma unroll
-    for (int p = 1; p <= kXDepth; ++p)
-  #pragma unroll
-      for (int i = 0; i < kPiecesW; ++i) load_piece(xr[p % kXDepth][i], i, p);
-    block_sync_lds();
-
-    // Operand registers, two sets: the MFMAs of k group j read set j & 1 while the reads of the
-    // next group fill the other; group 0 of the next step takes the place of "group 4".
-    u32x4 a[2][MW], b[2][2];
-    auto read_ops = [&](int set, int step, int wslot, int j) {
-      const uint8_t* xa = xs + (step & 1) * kXBufBytes + (wrow0 + c) * kRowBytes + h * 64 + j * 16;
-      const uint8_t* wb = ws + wslot * kWBufBytes + c * kRowBytes + h * 64 + j * 16;
-      b[set][0] = *reinterpret_cast<const u32x4*>(wb);
-      b[set][1] = *reinterpret_cast<const u32x4*>(wb + 32 * kRowBytes);
-  #pragma unroll
-      for (int mt = 0; mt < MW; ++mt) a[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * kRowBytes);
-    };
-    // Pieces of tile step+1 stored (and refilled with tile step+1+kXDepth) behind the MFMAs of k
-    // groups 0..2, so that all of them are in LDS before group 3 fetches the next step's operands.
-    constexpr int kPieceOfGroup[4] = {0, (kPiecesW + 2) / 3, (2 * kPiecesW + 2) / 3, kPiecesW};
-
-    auto one_step = [&](u32x4 (&set)[kPiecesW], int step, int wslot) {
-      const int wnext = wslot == kWRing - 1 ? 0 : wslot + 1;
-  #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (j < 3) read_ops((j + 1) & 1, step, wslot, j + 1);
-        else read_ops(0, step + 1, wnext, 0);
-        __builtin_amdgcn_sched_barrier(0);
-  #pragma unroll
-        for (int mt = 0; mt < MW; ++mt) {
-          acc[mt][0] = mfma32<ACT>(a[j & 1][mt], b[j & 1][0], acc[mt][0]);
-          acc[mt][1] = mfma32<ACT>(a[j & 1][mt], b[j & 1][1], acc[mt][1]);
-        }
-        if (j < 3) {
-  #pragma unroll
-          for (int i = kPieceOfGroup[j]; i < kPieceOfGroup[j + 1]; ++i) {
-            store_piece(set[i], i, (step + 1) & 1);
-            load_piece(set[i], i, step + 1 + kXDepth);
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-
-    read_ops(0, 0, 0, 0);
-    int wslot = 0;
-    const int whole = steps / kXDepth * kXDepth;
-    for (int t0 = 0; t0 < whole; t0 += kXDepth) {
-  #pragma unroll
-      for (int d = 0; d < kXDepth; ++d) {
-        one_step(xr[(d + 1) % kXDepth], t0 + d, wslot);
-        wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
-        block_sync_lds();
-      }
-    }
-    // Fewer than kXDepth real steps are left (their register sets are still indexed statically),
-    // then the padding iterations, which only keep the producers' barriers company.
-  #pragma unroll
-    for (int d = 0; d < kXDepth; ++d) {
-      if (whole + d < steps) {
-        one_step(xr[(d + 1) % kXDepth], whole + d, wslot);
-        wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
-        block_sync_lds();
-      }
-    }
-    for (int t = steps; t < total; ++t) block_sync_lds();
-
   }
+#pragma unroll
+  for (int d = 0; d < kBufs; ++d) {
+    if (whole + d < steps) {
+      one_step(d, whole + d, wslot);
+      wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
+      block_sync_lds();
+    }
+  }
+  for (int t = steps; t < total; ++t) block_sync_lds();
+  // Nothing may still be on its way into LDS when the wave ends (the block's LDS is handed on).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: D[m = 8*(i/4) + 4h + i%4][n = c] --------------------------
   if (!wave_active) return;
@@ -483,7 +378,7 @@ int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs
                         const char* what) {
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
-  const int lds = XStage<Provider, MW>::kLdsBytes;
+  const int lds = XStage<MW>::kLdsBytes;
   static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
   if (!attr_set) {
     const hipError_t e = hipFuncSetAttribute(

@@ -141,7 +141,6 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       xa[j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)kc * 64 + j * 8);
-      if constexpr (Provider::kPermuteA) xa[j] = permute_a_0415(xa[j]);
       xa[j] = (x_lane && kvalid) ? xa[j] : zero4;
     }
 

@@ -20,8 +20,7 @@
 //
 // A B-operand of a VQ weight with VL = 8 is exactly one codebook row, so the
 // 16-byte gather lands in MFMA layout with no shuffling (VL = 4: two rows, two 8-byte gathers).  For int4 the eight
-// nibbles of one dword are one operand, produced in the k-order
-// (0,4,1,5,2,6,3,7); the A-operand is permuted the same way (kPermuteA).
+// nibbles of one dword are one operand, for int8 eight bytes.
 #pragma once
 
 #include "common.hpp"
@@ -44,7 +43,6 @@ __device__ __forceinline__ uint32_t select_dword(const u32x4& v, int jp) {
 template <int ACT, int BITS, bool CONV, int VL = 8>
 struct VqProvider {
   static_assert(VL == 8 || VL == 4, "vector length 8 or 4");
-  static constexpr bool kPermuteA = false;
   static constexpr int kIdxPerChunk = 64 / VL;
   struct Args {
     const uint8_t* packed;
@@ -129,7 +127,6 @@ struct VqProvider {
 // ---------------------------------------------------------------------------
 template <int ACT, int BITS_M, int BITS_R>
 struct RvqProvider {
-  static constexpr bool kPermuteA = false;
   struct Args {
     const uint8_t* packed_m;
     const uint8_t* packed_r;
@@ -204,15 +201,18 @@ struct RvqProvider {
 // ---------------------------------------------------------------------------
 // int4, group size a multiple of 32; symmetric (zero point 8) or, with ASYM, a
 // per-group fp16 zero point.
-// One dword of nibbles = one operand, emitted in k-order (0,4,1,5,2,6,3,7).
-// Symmetric f16: w = f16((q-8) * s) -- exact product, one rounding: the oracle's weight.
+// One dword of nibbles = one operand, in natural k order: byte i of the dword (nibbles 2i and
+// 2i+1) is copied under both halves of a pair (v_perm_b32); masked with 0x00F0000F and or-ed
+// with 0x54006400, the low half reads as fp16 1024 + q[2i] (nibble in mantissa bits 0..3 of
+// 0x6400) and the high half as 64 + q[2i+1] (bits 4..7 of 0x5400), both exact.
+// Symmetric f16: minus (1032, 72) -> q - 8 exactly, times the scale -- exact product, one
+// rounding: the oracle's weight.
 // Otherwise w = round((f32(q) - f32(zp)) * f32(s)), the difference exact, the product
 // rounded to f32 and then to the activation type, operation for operation as the
 // element-wise decode does it.
 // ---------------------------------------------------------------------------
 template <int ACT, bool ASYM = false>
 struct Q4Provider {
-  static constexpr bool kPermuteA = true;
   struct Args {
     const uint8_t* w_pack;   // [N, K/2]
     const uint16_t* scale;   // [N, K/gs]
@@ -267,23 +267,25 @@ struct Q4Provider {
     b1 = dequant8(r.w.y, r.s2, r.z);
   }
 
-  // Eight nibbles of one dword -> one operand, k-order (0,4,1,5,2,6,3,7).
+  // Eight nibbles of one dword -> one operand, natural k order.
   __device__ __forceinline__ u32x4 dequant8(uint32_t w, uint32_t s2, uint32_t z) const {
 #pragma clang fp contract(off)
     uint32_t o[4];
     const float sf = f16_bits_to_f32(s2 & 0xFFFFu);
     const float zf = ASYM ? f16_bits_to_f32(z & 0xFFFFu) : 0.f;
+    // byte i of w into bytes 0 and 2 (bytes 1 and 3: zero)
+    const uint32_t spread[4] = {__builtin_amdgcn_perm(0u, w, 0x0c000c00u), __builtin_amdgcn_perm(0u, w, 0x0c010c01u),
+                                __builtin_amdgcn_perm(0u, w, 0x0c020c02u), __builtin_amdgcn_perm(0u, w, 0x0c030c03u)};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      // (1024 + q) as fp16 via the exponent trick.
-      const uint32_t pair = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+      const uint32_t pair = (spread[i] & 0x00F0000Fu) | 0x54006400u;  // (1024 + q[2i], 64 + q[2i+1])
       if constexpr (ACT == NPAMD_F16 && !ASYM) {
-        // minus 1032 -> q - 8 exactly; times the scale: one rounding.
-        const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, 0x64086408u);
+        // minus (1032, 72) -> q - 8 exactly; times the scale: one rounding.
+        const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, 0x54806408u);
         o[i] = __builtin_bit_cast(uint32_t, q * __builtin_bit_cast(f16x2, s2));
       } else {
         // q (ASYM) or q - 8 exactly, in fp16; the rest in f32.
-        const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, ASYM ? 0x64006400u : 0x64086408u);
+        const f16x2 q = __builtin_bit_cast(f16x2, pair) - __builtin_bit_cast(f16x2, ASYM ? 0x54006400u : 0x54806408u);
         float lo = (float)q.x, hi = (float)q.y;
         if constexpr (ASYM) {
           lo -= zf;
@@ -308,7 +310,112 @@ struct Q4Provider {
   }
 };
 
-// A-operand (x) permutation matching Q4Provider's k-order.
+// ---------------------------------------------------------------------------
+// int8, group size a multiple of 32; symmetric (zero point 128) or, with ASYM, a per-group
+// fp16 zero point.  Eight bytes = one operand, in natural k order (no A permutation).
+// A byte b placed under the exponent byte 0x64 reads as fp16 1024 + b exactly (v_perm_b32,
+// two weights per instruction).  Symmetric f16: minus 1152 -> q - 128 exactly, times the
+// scale: one rounding of an exact product, the oracle's weight.  Otherwise as Q4Provider:
+// difference and product in f32, then rounded to the activation type.
+// ---------------------------------------------------------------------------
+template <int ACT, bool ASYM = false>
+struct Q8Provider {
+  struct Args {
+    const uint8_t* w_pack;   // [N, K]
+    const uint16_t* scale;   // [N, K/gs]
+    int chunks;              // K / 64
+    int groups_per_row;      // K / gs
+    int gs_shift_chunks;     // log2(gs/32)
+    const uint16_t* zp;      // [N, K/gs] (ASYM only)
+  };
+  struct Raw {
+    u32x4 w[4];           // 64 bytes = operands 0..7
+    uint32_t s_lo, s_hi;  // scale (replicated pair) for operands 0-3 and 4-7
+    uint32_t z_lo, z_hi;  // zero points (fp16 bits), ASYM only
+  };
+  static constexpr bool kLdsCodebook = false;
+  static constexpr bool kGathers = false;  // operands are arithmetic on the packed bytes
+  const Args& a;
+  __device__ explicit Q8Provider(const Args& args) : a(args) {}
+
+  __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
+    const u32x4* p = reinterpret_cast<const u32x4*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.w[i] = p[i];
+    const int64_t row = (int64_t)n * a.groups_per_row;
+    const int g_lo = (2 * kc) >> a.gs_shift_chunks, g_hi = (2 * kc + 1) >> a.gs_shift_chunks;
+    r.s_lo = (uint32_t)a.scale[row + g_lo] * 0x10001u;
+    r.s_hi = (uint32_t)a.scale[row + g_hi] * 0x10001u;
+    if constexpr (ASYM) {
+      r.z_lo = a.zp[row + g_lo];
+      r.z_hi = a.zp[row + g_hi];
+    }
+  }
+  template <int J>
+  __device__ __forceinline__ u32x4 operand(const Raw& r) const {
+    const u32x4& ww = r.w[J / 2];
+    return dequant8((J & 1) ? ww.z : ww.x, (J & 1) ? ww.w : ww.y, (J < 4) ? r.s_lo : r.s_hi, (J < 4) ? r.z_lo : r.z_hi);
+  }
+
+  struct PairRaw {
+    u32x4 w;      // 16 bytes = operands 2*jp, 2*jp+1
+    uint32_t s2;  // their scale (one 32-k group), replicated
+    uint32_t z;   // their zero point, fp16 bits (ASYM only)
+  };
+  __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
+    r.w = *reinterpret_cast<const u32x4*>(a.w_pack + ((int64_t)n * a.chunks + kc) * 64 + jp * 16);
+    const int64_t g = (int64_t)n * a.groups_per_row + ((2 * kc + (jp >> 1)) >> a.gs_shift_chunks);
+    r.s2 = (uint32_t)a.scale[g] * 0x10001u;
+    if constexpr (ASYM) r.z = a.zp[g];
+  }
+  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
+    b0 = dequant8(r.w.x, r.w.y, r.s2, r.z);
+    b1 = dequant8(r.w.z, r.w.w, r.s2, r.z);
+  }
+
+  // Eight bytes (two dwords) -> one operand.
+  __device__ __forceinline__ u32x4 dequant8(uint32_t d0, uint32_t d1, uint32_t s2, uint32_t z) const {
+#pragma clang fp contract(off)
+    const float sf = f16_bits_to_f32(s2 & 0xFFFFu);
+    const float zf = ASYM ? f16_bits_to_f32(z & 0xFFFFu) : 0.f;
+    const uint32_t pairs[4] = {__builtin_amdgcn_perm(0x64646464u, d0, 0x04010400u),   // (1024 + b0, 1024 + b1)
+                               __builtin_amdgcn_perm(0x64646464u, d0, 0x04030402u),   // (1024 + b2, 1024 + b3)
+                               __builtin_amdgcn_perm(0x64646464u, d1, 0x04010400u),
+                               __builtin_amdgcn_perm(0x64646464u, d1, 0x04030402u)};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (ACT == NPAMD_F16 && !ASYM) {
+        const f16x2 q = __builtin_bit_cast(f16x2, pairs[i]) - __builtin_bit_cast(f16x2, 0x64806480u);  // 1152
+        o[i] = __builtin_bit_cast(uint32_t, q * __builtin_bit_cast(f16x2, s2));
+      } else {
+        const f16x2 q = __builtin_bit_cast(f16x2, pairs[i]) - __builtin_bit_cast(f16x2, ASYM ? 0x64006400u : 0x64806480u);
+        float lo = (float)q.x, hi = (float)q.y;
+        if constexpr (ASYM) {
+          lo -= zf;
+          hi -= zf;
+        }
+        lo *= sf;
+        hi *= sf;
+        if constexpr (ACT == NPAMD_F16) {
+          f16x2 h;
+          h.x = (_Float16)lo;
+          h.y = (_Float16)hi;
+          o[i] = __builtin_bit_cast(uint32_t, h);
+        } else {
+          bf16x2 b;
+          b.x = (__bf16)lo;
+          b.y = (__bf16)hi;
+          o[i] = __builtin_bit_cast(uint32_t, b);
+        }
+      }
+    }
+    return u32x4{o[0], o[1], o[2], o[3]};
+  }
+};
+
+// Eight 16-bit values reordered (0,4,1,5,2,6,3,7): the (k, k+4) pair order in which the row-wise
+// int4 GEMV stages its activations.
 __device__ __forceinline__ u32x4 permute_a_0415(u32x4 x) {
   u32x4 r;
   r.x = (x.x & 0xFFFFu) | (x.z << 16);

@@ -2,9 +2,9 @@
 //
 //   q = (w_pack[n, k/vpb] >> ((k%vpb)*nbits)) & mask ;  w = (float(q) - zp) * float(scale)
 //
-// Fast kernels cover the Q4_0 / GPTQ layouts (4 bits, symmetric or with per-group fp16
-// zero points, group size a power-of-two multiple of 32, K % 64 == 0); every other valid
-// combination (1/2/8 bits, odd group sizes, odd K) runs the element-wise fallback.
+// Fast kernels cover the Q4_0 / Q8_0 / GPTQ layouts (4 or 8 bits, symmetric or with per-group
+// fp16 zero points, group size a power-of-two multiple of 32, K % 64 == 0); every other valid
+// combination (1/2 bits, odd group sizes, odd K) runs the element-wise fallback.
 #include <stdlib.h>
 
 #include "gemm_tile.hpp"
@@ -327,7 +327,7 @@ static int validate_q(const char* what, int N, int K, int nbits, int gs) {
 }
 
 static bool q_fast_ok(const QCall& c) {
-  return c.nbits == 4 && c.gs % 32 == 0 && is_pow2(c.gs / 32) && c.K % 64 == 0 &&
+  return (c.nbits == 4 || c.nbits == 8) && c.gs % 32 == 0 && is_pow2(c.gs / 32) && c.K % 64 == 0 &&
          c.K > 0 && c.ldx % 8 == 0 && ptr_aligned(c.x, 16) && ptr_aligned(c.w_pack, 16);
 }
 
@@ -398,9 +398,22 @@ static int q4_fused(const QCall& c, bool gemv) {
   return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
+template <int ACT, bool ASYM>
+static int q8_fused(const QCall& c, bool gemv) {
+  using P = Q8Provider<ACT, ASYM>;
+  typename P::Args a{c.w_pack, (const uint16_t*)c.scale, c.K / 64, c.K / c.gs, log2i(c.gs / 32), (const uint16_t*)c.zp};
+  if (gemv) {
+    GemvShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K / 64, 0, 0};
+    return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+  }
+  GemmShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, c.K / 64, 0};
+  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
+}
+
 template <int ACT>
 static int q_dispatch(const QCall& c, bool gemv) {
   if (q_fast_ok(c)) {
+    if (c.nbits == 8) return c.zp ? q8_fused<ACT, true>(c, gemv) : q8_fused<ACT, false>(c, gemv);
     if (gemv && q4_rowwise_ok(c)) return launch_q4_rowwise<ACT, 1>(c);
     return c.zp ? q4_fused<ACT, true>(c, gemv) : q4_fused<ACT, false>(c, gemv);
   }
@@ -492,7 +505,7 @@ extern "C" int npamd_q_dequant(const uint8_t* w_pack, const void* scale_f16, con
 }
 
 extern "C" int npamd_q_fused_supported(int K, int nbits, int group_size) {
-  return nbits == 4 && group_size > 0 && group_size % 32 == 0 && is_pow2(group_size / 32) && K > 0 && K % 64 == 0 &&
+  return (nbits == 4 || nbits == 8) && group_size > 0 && group_size % 32 == 0 && is_pow2(group_size / 32) && K > 0 && K % 64 == 0 &&
                  K % group_size == 0
              ? 1
              : 0;

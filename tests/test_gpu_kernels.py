@@ -329,11 +329,14 @@ def test_q4_rowwise_gemv_large_activations(gpu, asym):
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("gs", [32, 64, 128])
 @pytest.mark.parametrize("m", [1, 16, 17, 200])
-def test_q4_linear_fast_path(gpu, oracle_lib, act, gs, m):
+@pytest.mark.parametrize("nbits,asym", [(4, False), (4, True), (8, False), (8, True)])
+def test_q4_linear_fast_path(gpu, oracle_lib, act, gs, m, nbits, asym):
+    """4 and 8 bits, with and without zero points, on the MFMA GEMV (<= 16 tokens) and tile GEMM."""
     from neuropress_amd import kernels
 
-    L = cases.q4_layer(600 + gs + m, 300, 384, gs=gs, act=act, m=m, bias=True)
-    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, None, L["bias"].to(gpu))
+    L = cases.q4_layer(600 + gs + m, 300, 384, nbits=nbits, gs=gs, act=act, m=m, bias=True, asym=asym)
+    zp = None if L["zp"] is None else L["zp"].to(gpu)
+    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), nbits, gs, zp, L["bias"].to(gpu))
     assert y.shape == (m, 300)
     _check(y, _q_ref(oracle_lib, L, act))
 
@@ -369,7 +372,7 @@ def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("kind", ["vq12", "vq16", "vq12_vl4", "vq16_vl4", "vq10_vl4", "rvq", "q4", "q4_asym", "q4_asym_gs128", "q8", "q2_asym"])
+@pytest.mark.parametrize("kind", ["vq12", "vq16", "vq12_vl4", "vq16_vl4", "vq10_vl4", "rvq", "q4", "q4_asym", "q4_asym_gs128", "q8", "q8_asym", "q8_gs128", "q2_asym"])
 def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
     """One-hot activations read the decoded weight back through the contraction kernels: with
     x = rows of the identity, y[m, n] is the single product 1 * W[n, k_m], which f32 accumulation
@@ -395,7 +398,7 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
         gemv = lambda x: kernels.rvq_linear(x, *args, None, tile=False)
         tile = lambda x: kernels.rvq_linear(x, *args, None, tile=True)
     else:
-        nbits = int(kind[1])  # 8 and 2 bits: the element-wise kernels
+        nbits = int(kind[1])  # 2 bits: the element-wise kernels
         gs = 128 if kind.endswith("gs128") else 32
         L = cases.q4_layer(63, n, k, nbits=nbits, gs=gs, act=act, m=1, asym="asym" in kind)
         blob, sc = L["blob"].to(gpu), L["scale"].to(gpu)

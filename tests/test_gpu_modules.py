@@ -136,7 +136,7 @@ def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch
 
 
 def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch):
-    """8-bit group quantization and vector length 2 have no MFMA kernel: the modules decode once and
+    """2-bit group quantization and vector length 2 have no MFMA kernel: the modules decode once and
     call the dense GEMM at every token count instead of the fused entry points (whose element-wise
     kernels decode the weight once per 16 tokens)."""
     import neuropress_amd.nn.np_linear as qmod
@@ -148,9 +148,9 @@ def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch)
         monkeypatch.setattr(kernels, name, lambda *a, _real=real, _name=name, **kw: (calls.append(_name), _real(*a, **kw))[1])
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
     monkeypatch.setattr(qmod, "_Q_TILE_MIN_GRID_FRACTION", 0.0)
-    Q = cases.q4_layer(81, 96, 256, nbits=8, bias=True)
-    qlayer = NPLinear(Q["blob"], Q["scale"], 96, 256, 32, 8, "sym", "cuda", bias=Q["bias"].float()).to(gpu)
-    wq = ((Q["codes"].float() - 128).reshape(96, 8, 32) * Q["scale"].float().reshape(96, 8, 1)).reshape(96, 256)
+    Q = cases.q4_layer(81, 96, 256, nbits=2, bias=True)
+    qlayer = NPLinear(Q["blob"], Q["scale"], 96, 256, 32, 2, "sym", "cuda", bias=Q["bias"].float()).to(gpu)
+    wq = ((Q["codes"].float() - 2).reshape(96, 8, 32) * Q["scale"].float().reshape(96, 8, 1)).reshape(96, 256)
     L = cases.vq_layer(82, 96, 256, 1024, vl=2, bits=10, bias=True, std=0.05)
     layer = NPVQLinear(VQProxy(L["cb"]).to(gpu), L["packed"], 10, 96, 256, 2, "cuda_wmma", bias=L["bias"].float()).to(gpu)
     w = L["cb"][L["idx"]].reshape(96, 256).half().float()

@@ -382,7 +382,8 @@ def test_c_abi_validates_arguments_without_a_gpu():
     assert lib.npamd_vq_fused_supported(4096, 8, 10) == 0  # 10-bit stream (the module widens it to 16 first)
     assert lib.npamd_vq_fused_supported(4096 + 32, 8, 12) == 0  # K not a multiple of 64
     assert lib.npamd_q_fused_supported(4096, 4, 32) == 1 and lib.npamd_q_fused_supported(4096, 4, 128) == 1
-    assert lib.npamd_q_fused_supported(4096, 8, 32) == 0 and lib.npamd_q_fused_supported(4096, 4, 96) == 0
+    assert lib.npamd_q_fused_supported(4096, 8, 32) == 1 and lib.npamd_q_fused_supported(4096, 8, 64) == 1
+    assert lib.npamd_q_fused_supported(4096, 2, 32) == 0 and lib.npamd_q_fused_supported(4096, 4, 96) == 0
     assert lib.npamd_q_fused_supported(4096, 4, 16) == 0 and lib.npamd_q_fused_supported(4096 + 32, 4, 32) == 0
 
 
