@@ -34,16 +34,20 @@ from .backends import Backend, LinearBackend, is_hip_backend_available, tile_ban
 log = logging.getLogger(__name__)
 
 # Upper end of the fused-GEMM band for the int4 path; above it decode + GEMM.
-# Measured on one MI355X (14336 x 4096, group 32): fused GEMM 38-42 us up to 128
-# tokens and 72 us at 256 against 56-62 / 78 us for decode + GEMM; 104 vs 84 us at 384.
+# Measured on one MI355X (14336 x 4096, group 32): fused GEMM 35-40 us up to 128
+# tokens and 56 us at 256 against 56-64 / 80 us for decode + GEMM; 83-84 vs 78-84 us at
+# 320-384, 158 vs 93 us at 512.
 _Q_TILE_MAX_TOKENS: int = int(os.environ.get("NEUROPRESS_Q_TILE_MAX_TOKENS", "256"))
+# Long reductions (K >= _Q_TILE_SPLIT_LONG_K), where the dense GEMM is slow, keep the fused
+# GEMM up to this many tokens: 4096 x 14336 80 vs 105-109 us at 320-384, 148 vs 120 us at 512.
+_Q_TILE_LONG_K_MAX_TOKENS: int = 384
 # As for the VQ path: the fused GEMM splits the reduction when the layer has few
 # output features; a layer that still leaves most compute units idle takes decode +
-# GEMM.  Measured (fused vs decode + GEMM): 4096 x 14336 39-46 vs 58-93 us up to 128
-# tokens, 75 vs 91 us at 256; 4096 x 4096 20-25 vs 32-41 us up to 128, 36 vs 37 us
-# at 256; 1024 x 4096 (not enough workgroups even when split) 17-19 vs 16-20 us.
+# GEMM.  Measured (fused vs decode + GEMM): 4096 x 14336 41-57 vs 93-115 us from 128 to
+# 256 tokens; 4096 x 4096 24-31 vs 37-45 us from 128 to 256, 39-41 vs 39-40 us at
+# 320-384; 1024 x 4096 (not enough workgroups even when split) 17-19 vs 16-20 us.
 _Q_TILE_MIN_GRID_FRACTION: float = 0.7
-_Q_TILE_SPLIT_MAX_TOKENS: int = 128
+_Q_TILE_SPLIT_MAX_TOKENS: int = 256
 _Q_TILE_SPLIT_LONG_K: int = 8192
 _Q_FUSED_MAX_TOKENS: int = 16
 
@@ -300,7 +304,10 @@ class NPLinear(nn.Module):
             # dense GEMM (14336 x 4096, 8 bits: 99 us against 57 us at one token, 452 against 57 at 16).
             fused_ok = x.dtype in (torch.float16, torch.bfloat16) and self._mfma_layer()
             if fused_ok and m > _Q_FUSED_MAX_TOKENS:
-                fused_ok = m <= _Q_TILE_MAX_TOKENS and self._tile_grid_fills_gpu(x, m)
+                limit = _Q_TILE_MAX_TOKENS
+                if self.in_features >= _Q_TILE_SPLIT_LONG_K:
+                    limit = max(limit, _Q_TILE_LONG_K_MAX_TOKENS)
+                fused_ok = m <= limit and self._tile_grid_fills_gpu(x, m)
             if fused_ok:
                 if m <= _Q_FUSED_MAX_TOKENS:
                     return kernels.q_linear(
