@@ -56,6 +56,7 @@ static int device_cu_count() {
 // as soon as the grid starts: jobs per wave is kept near jobs / (16 waves * CUs).
 // NPAMD_GEMV_R / NPAMD_GEMV_SPW override the choice (tuning aid).
 bool gemv_lds_codebook_enabled() { return env_int("NPAMD_GEMV_LDS_CB", 1) != 0; }
+bool tile_lds_codebook_enabled() { return env_int("NPAMD_TILE_LDS_CB", 1) != 0; }
 bool gemv_lds_activations_forced() { return env_int("NPAMD_GEMV_LDS_X", 0) != 0; }
 
 GemvPlan plan_gemv(int N, int chunks, int max_r) {

@@ -84,23 +84,36 @@ __device__ __forceinline__ void block_sync_lds() {
 // every 16-byte bank group twice, as with padded rows.  A lane may fetch any source address, so
 // the swizzle costs nothing at the load.  kBufs tiles are in LDS.  (Every provider takes x as
 // it lies in memory; one that reordered k inside an operand would have to go through registers.)
-template <int MW>
+// CB_LDS (codebooks of up to 64 KiB): the block copies the table into LDS behind the tiles and
+// the producers look operands up there; to make room, two x tiles instead of three at 129..256
+// tokens.  Larger tables and 257..384 tokens (LDS is full) gather from memory.
+template <int MW, bool CB_LDS = false>
 struct XStage {
-  static constexpr int kBufs = MW == 3 ? 2 : 3;
+  static constexpr int kBufs = (MW == 3 || (MW == 2 && CB_LDS)) ? 2 : 3;
   static constexpr int kXRowBytes = kStepK * 2;
   static constexpr int kBufBytes = 128 * MW * kXRowBytes;
-  static constexpr int kLdsBytes = kBufs * kBufBytes + kWRing * kWBufBytes;
+  static constexpr int kLdsBytes = kBufs * kBufBytes + kWRing * kWBufBytes;  // the codebook copy follows
 };
+constexpr int kTileLdsCodebookMax = 64 * 1024;
+constexpr int kLdsPerBlockMax = 160 * 1024;
 
-template <int ACT, class Provider, int MW>
+template <int ACT, class Provider, int MW, bool CB_LDS = false>
 __global__ void __launch_bounds__(512)
 tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  using XS = XStage<MW>;
+  using XS = XStage<MW, CB_LDS>;
   constexpr int BM = 128 * MW;
   constexpr int kXBufBytes = XS::kBufBytes;
   uint8_t* const xs = lds;                             // [XS::kBufs][BM][XS::kXRowBytes]
   uint8_t* const ws = lds + XS::kBufs * kXBufBytes;    // [kWRing][64][kRowBytes]
+  Provider prov(pargs);
+  if constexpr (CB_LDS) {
+    u32x4* cb_lds = reinterpret_cast<u32x4*>(lds + XS::kLdsBytes);
+    const u32x4* src = prov.global_codebook();
+    for (int i = threadIdx.x; i < prov.codebook_vec16(); i += 512) cb_lds[i] = src[i];
+    prov.use_codebook(cb_lds);
+    __syncthreads();
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -141,7 +154,6 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     //   3. loads the packed bytes of step t+1+2*kDepth.
     // Loads are consumed in the order they were issued, so waiting for the
     // oldest never drains the younger ones.
-    const Provider prov(pargs);
     const int q = wave - 4;
     const int col = 16 * q + (lane & 15);
     const int jp = lane >> 4;
@@ -373,22 +385,24 @@ int plan_tile_splits(int M, int N, int chunks, int mw);
 // NPAMD_TILE_MW overrides the choice (tuning aid).
 int plan_tile_mw(int M);
 
-template <int ACT, class Provider, int MW>
-int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs, hipStream_t st,
-                        const char* what) {
+bool tile_lds_codebook_enabled();  // NPAMD_TILE_LDS_CB=0 switches the LDS copy off (tuning aid)
+
+template <int ACT, class Provider, int MW, bool CB_LDS>
+int launch_tile_gemm_mw_cb(const GemmShape& s, const typename Provider::Args& pargs, int cb_bytes, hipStream_t st,
+                           const char* what) {
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
-  const int lds = XStage<MW>::kLdsBytes;
-  static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
-  if (!attr_set) {
+  const int lds = XStage<MW, CB_LDS>::kLdsBytes + (CB_LDS ? cb_bytes : 0);
+  static int reserved = 0;  // per instantiation: largest dynamic-LDS size enabled so far
+  if (lds > reserved) {
     const hipError_t e = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&tile_gemm_kernel<ACT, Provider, MW>),
+        reinterpret_cast<const void*>(&tile_gemm_kernel<ACT, Provider, MW, CB_LDS>),
         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds,
                                      hipGetErrorString(e));
-    attr_set = true;
+    reserved = lds;
   }
-  tile_gemm_kernel<ACT, Provider, MW><<<grid, 512, lds, st>>>(s, pargs);
+  tile_gemm_kernel<ACT, Provider, MW, CB_LDS><<<grid, 512, lds, st>>>(s, pargs);
   if (s.splits > 1) {
     const int64_t quads = (int64_t)s.M * ((s.N + 3) / 4);
     splitk_reduce_kernel<ACT><<<(unsigned)((quads + 255) / 256), 256, 0, st>>>(s.partials, s.splits, s.M, s.N,
@@ -397,10 +411,25 @@ int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs
   return check_launch(what);
 }
 
+// cb_bytes: size of the (single) codebook for providers that can look it up in LDS, else 0.
+template <int ACT, class Provider, int MW>
+int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs, int cb_bytes, hipStream_t st,
+                        const char* what) {
+  if constexpr (Provider::kLdsCodebook && MW < 3) {
+    // At 129..256 tokens the copy costs the third x tile: worth it only for tables the vector L1
+    // does not hold anyway (14336 x 4096 at 256 tokens: 4096 rows 64 -> 57 us, 256 rows 49 -> 53 us).
+    const bool pays = MW == 1 || cb_bytes > 16 * 1024;
+    if (pays && cb_bytes > 0 && cb_bytes <= kTileLdsCodebookMax && cb_bytes % 16 == 0 &&
+        XStage<MW, true>::kLdsBytes + cb_bytes <= kLdsPerBlockMax && tile_lds_codebook_enabled())
+      return launch_tile_gemm_mw_cb<ACT, Provider, MW, true>(s, pargs, cb_bytes, st, what);
+  }
+  return launch_tile_gemm_mw_cb<ACT, Provider, MW, false>(s, pargs, 0, st, what);
+}
+
 // `workspace` (f32, may be null) decides whether K may be split: it must hold splits * M * N floats.
 template <int ACT, class Provider>
 int launch_tile_gemm(GemmShape s, const typename Provider::Args& pargs, hipStream_t st,
-                     const char* what, void* workspace = nullptr, int64_t workspace_bytes = 0) {
+                     const char* what, void* workspace = nullptr, int64_t workspace_bytes = 0, int cb_bytes = 0) {
   s.steps = s.chunks;
   const int mw = plan_tile_mw(s.M);
   int splits = workspace ? plan_tile_splits(s.M, s.N, s.chunks, mw) : 1;
@@ -410,9 +439,9 @@ int launch_tile_gemm(GemmShape s, const typename Provider::Args& pargs, hipStrea
   s.splits = (s.chunks + s.split_chunks - 1) / s.split_chunks;  // no empty split
   s.partials = (float*)workspace;
   switch (mw) {
-    case 1: return launch_tile_gemm_mw<ACT, Provider, 1>(s, pargs, st, what);
-    case 2: return launch_tile_gemm_mw<ACT, Provider, 2>(s, pargs, st, what);
-    default: return launch_tile_gemm_mw<ACT, Provider, 3>(s, pargs, st, what);
+    case 1: return launch_tile_gemm_mw<ACT, Provider, 1>(s, pargs, cb_bytes, st, what);
+    case 2: return launch_tile_gemm_mw<ACT, Provider, 2>(s, pargs, cb_bytes, st, what);
+    default: return launch_tile_gemm_mw<ACT, Provider, 3>(s, pargs, cb_bytes, st, what);
   }
 }
 

@@ -12,12 +12,12 @@ int run_vq(const VqCall& c, const GemmShape& s) {
     if (c.cb_dtype == NPAMD_F16) {
       using P = VqProvider<ACT, BITS, true, VL>;
       typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-      return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
+      return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes, (VL == 8 ? c.nc * 16 : (c.nc % 2 == 0 ? c.nc * 8 : 0)));
     }
   }
   using P = VqProvider<ACT, BITS, false, VL>;
   typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
-  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
+  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes, (VL == 8 ? c.nc * 16 : (c.nc % 2 == 0 ? c.nc * 8 : 0)));
 }
 
 template <int ACT, int VL>
