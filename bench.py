@@ -375,6 +375,18 @@ def main():
                     t = time_graph(lambda i: kernels.vq_linear(xm[i % 2][:, perm], cc["pool"][i], cc["d_cb"], bits, 8, None,
                                                                nn_), rot, steps_s * 2, 3, dev)
                     add(name + " column_perm", "a:torch gather + gemv", m, t, vq_alg_bytes(cc, m) + kk * 8, 2.0 * m * nn_ * kk)
+            if bits == 12:
+                # the same layer in the token bands the configuration itself does not list: tile GEMM with the
+                # 4096-row codebook looked up in LDS, against decode + GEMM
+                for m in (64, 256):
+                    xm = [torch.randn(m, kk, generator=gen(80 + m)).to(torch.float16).to(dev) for _ in range(2)]
+                    t = time_graph(lambda i: kernels.vq_gemm_tile(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, nn_, None),
+                                   rot, steps_s, 2, dev)
+                    add(name, "b:tile-gemm", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
+                    t = time_graph(lambda i: torch.nn.functional.linear(
+                        xm[i % 2], kernels.vq_dequant(cc["pool"][i], cc["d_cb"], bits, nn_, kk, torch.float16)),
+                        rot, steps_s, 2, dev)
+                    add(name, "c:decode+gemm", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
             del cc
             torch.cuda.empty_cache()
         # config 4: residual VQ (65536 + 256 entry codebooks, Zipf(1.1) indices, per-row scale / bias), fp16
