@@ -44,7 +44,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
-    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "dequant", "q4_gemv_m1", "q4_tile_m128",
+    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_tile_m128",
                                                     "rms_norm_m4096", "vq_embedding_m4096", "q4_embedding_m4096"],
                     help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
                          "on the config-3 / config-5 shape and print a one-line JSON with its HIP-event time")
@@ -175,7 +175,7 @@ def main():
             fn = lambda i: kernels.q_linear(x, pool[i], sc, 4, 32)
             alg, flops = n * k // 2 + n * k // 32 * 2 + m * k * 2 + m * n * 2, 2.0 * m * n * k
         else:
-            nc, bits = (4096, 12) if args.case == "gemv_nc4096_m1" else (65536, 16)
+            nc, bits = (4096, 12) if args.case in ("gemv_nc4096_m1", "tile_nc4096_m128") else (65536, 16)
             cb = (torch.randn(nc, 8, generator=g) * 0.02).to(torch.float16)
             if bits == 16:
                 base = torch.randint(0, 65536, (n * k // 8,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8)
@@ -183,14 +183,14 @@ def main():
                 base = IndexPacking.pack(torch.randint(0, nc, (n * k // 8,), generator=g), bits)
             pool = [base.to(dev).clone() for _ in range(n_rot)]
             cb16, cbb = cb.to(dev), cb.to(torch.bfloat16).to(dev)
-            m = 256 if args.case == "tile_m256" else 1
+            m = 256 if args.case == "tile_m256" else 128 if args.case == "tile_nc4096_m128" else 1
             x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
             if args.case == "sliced_m1":
                 sl0 = kernels.vq_slice_indices(base, bits, n, k, 8, nc, device=dev)
                 spool = [sl0] + [kernels.SlicedIndices(sl0.blob.clone(), sl0.header) for _ in range(n_rot - 1)]
                 ws = torch.empty(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
                 fn = lambda i: kernels.vq_linear_sliced(x, spool[i], cbb, None, workspace=ws)
-            elif args.case == "tile_m256":
+            elif args.case in ("tile_m256", "tile_nc4096_m128"):
                 fn = lambda i: kernels.vq_gemm_tile(x, pool[i], cbb, bits, n, None)
             elif args.case == "dequant":
                 fn = lambda i: kernels.vq_dequant(pool[i], cb16, bits, n, k, torch.bfloat16)
