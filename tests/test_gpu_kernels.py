@@ -377,11 +377,12 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
     """One-hot activations read the decoded weight back through the contraction kernels: with
     x = rows of the identity, y[m, n] is the single product 1 * W[n, k_m], which f32 accumulation
     and the final rounding leave untouched.  So the MFMA GEMV (16 rows at a time) and the tile
-    GEMM (all K rows at once, with and without a reduction split) must reproduce the one-pass
+    GEMM (all K rows at once; on this shape it splits the reduction in two) must reproduce the one-pass
     decode, itself checked bit for bit against the oracle, exactly."""
-    from neuropress_amd import kernels
+    from neuropress_amd import _lib, kernels
 
-    n, k = 200, 512
+    n, k = 200, 1024
+    assert _lib.load().npamd_gemm_tile_workspace_bytes(230, n, k) > 0  # this shape splits the reduction
     if kind.startswith("vq"):
         bits = int(kind[2:4])
         vl = 4 if kind.endswith("vl4") else 8  # 10-bit stream: the element-wise kernels
@@ -411,7 +412,7 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
     for k0 in (0, 48, k - 16):
         assert torch.equal(gemv(eye[k0:k0 + 16]), wt[k0:k0 + 16]), f"GEMV, rows {k0}.."
     assert torch.equal(gemv(eye[7:9]), wt[7:9])   # two tokens (int4: still the MFMA kernel)
-    assert torch.equal(tile(eye), wt), "tile GEMM, 512 tokens"
+    assert torch.equal(tile(eye), wt), "tile GEMM, 1024 tokens"
     assert torch.equal(tile(eye[100:330]), wt[100:330]), "tile GEMM, 230 tokens"
 
 
