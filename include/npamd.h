@@ -203,6 +203,32 @@ int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
                          const float* bias, void* y, int64_t ldy, int M, int act_dtype,
                          void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * Decode GEMV over a prefix-coded index stream, read as it is stored (M <= NPAMD_GEMV_MAX_M):
+ *   y[m, n] = sum_k x[m, k] * codebook[idx(n, k/VL), k%VL] (+ bias[n]).
+ * Replaces vq_linear_tiered / vq_linear_ntier / vq_linear_zero_escape
+ * (neuropress/kernels/__init__.py:589-659, 711-762, 974-1049; kernels/vq_linear_tiered.cu,
+ * vq_linear_ntier.cu, vq_linear_zero_escape.cu): one entry point for the three formats of
+ * neuropress/transforms/vq_packing.py:298-1384, whose streams the caller passes separately, with
+ * the per-row cumulative class counts ([N + 1] int32 each) of the packers' compute_row_offsets.
+ *   flat = 0: n_classes - 1 cascaded one-bit class streams (stream k: one bit per index not
+ *             claimed by classes < k, 0 = class k).  Two-tier: n_classes = 2, bases {0, 0};
+ *             n-tier: bases {0, 2^bits[0], 2^bits[1], ...}.
+ *   flat = 1: one stream of two class bits per index, n_classes = 4 (zero-escape: widths
+ *             {0, 4, 8, cold_bits}, bases {0, 1, 17, 257}).
+ * Index = payload_base[c] + the payload_bits[c]-bit field number (row_offsets[c][n] + rank of the
+ * index among the row's class-c indices) of payload_streams[c]; a width of 0 means no payload.
+ * The pointer arrays are host arrays of device pointers.  The codebook must be in the activation
+ * dtype.  One wave per output row, wave64 ballot + population count for the ranks.
+ */
+int npamd_vq_gemv_coded(const void* x, int64_t ldx, int flat, int n_classes,
+                        const uint8_t* const* class_streams, const int64_t* class_bytes,
+                        const uint8_t* const* payload_streams, const int64_t* payload_bytes,
+                        const int* payload_bits, const uint32_t* payload_base,
+                        const int32_t* const* row_offsets, const void* codebook, int codebook_dtype,
+                        int nc, int vl, const float* bias, void* y, int64_t ldy, int M, int N, int K,
+                        int act_dtype, void* stream);
+
 /* ------------------------------------------------- residual VQ (RVQ) ---- */
 /*
  * Two codebooks + per-output-row fp16 scale and bias (no counterpart in the

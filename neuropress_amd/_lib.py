@@ -41,6 +41,8 @@ SIGNATURES: dict[str, list] = {
     "npamd_vq_sliced_check": [_vp, _i64],
     "npamd_vq_fused_supported": [_int, _int, _int],
     "npamd_q_fused_supported": [_int, _int, _int],
+    "npamd_vq_gemv_coded": [_vp, _i64, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp,
+                            _i64, _int, _int, _int, _int, _vp],  # fmt: skip
     "npamd_vq_sliced_workspace_bytes": [_vp, _int],
     "npamd_vq_gemv_sliced": [_vp, _i64, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _int, _int, _vp, _i64, _vp],
     "npamd_rvq_dequant": [_vp, _i64, _int, _vp, _i64, _int, _vp, _int, _vp, _int, _vp, _vp, _int,

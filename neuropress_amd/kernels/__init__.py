@@ -391,6 +391,114 @@ def vq_linear_sliced(
     return y
 
 
+def _vq_linear_coded(what, x, flat, class_streams, payload_streams, payload_bits, payload_base, row_offsets,
+                     centroids, vector_len, bias):
+    """Shared body of the three prefix-coded GEMV wrappers (``npamd_vq_gemv_coded``)."""
+    import ctypes
+
+    streams = [*class_streams, *payload_streams, *row_offsets]
+    _check_device(what, x, centroids, bias, *streams)
+    x = _x2d(x, what)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"{what}: x must be float16 or bfloat16, got {x.dtype}")
+    cb = _centroids_f16(centroids, what).to(x.dtype)
+    if cb.shape[1] != vector_len:
+        raise RuntimeError(f"{what}: vector_len does not match the codebook")
+    m, k = x.shape
+    if k % vector_len:
+        raise RuntimeError(f"{what}: K={k} not divisible by vector_len={vector_len}")
+    if m > _lib.GEMV_MAX_M:
+        raise RuntimeError(f"{what}: M={m} exceeds the fused limit {_lib.GEMV_MAX_M}")
+    n_classes = len(payload_streams)
+    if len(row_offsets) != n_classes or len(payload_bits) != n_classes or len(payload_base) != n_classes:
+        raise RuntimeError(f"{what}: one payload stream, width, base and row-offset table per class")
+    for t in (*class_streams, *payload_streams):
+        if t.dtype != torch.uint8 or not t.is_contiguous():
+            raise RuntimeError(f"{what}: streams must be contiguous uint8 tensors")
+    for t in row_offsets:
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError(f"{what}: row offsets must be contiguous int32 tensors")
+    n = int(row_offsets[0].numel()) - 1
+    if n < 0 or any(int(t.numel()) != n + 1 for t in row_offsets):
+        raise RuntimeError(f"{what}: row offsets must all have N + 1 entries")
+    ptr_array = lambda ts: (ctypes.c_void_p * max(len(ts), 1))(*[t.data_ptr() if t.numel() else None for t in ts])
+    cls_ptrs, pay_ptrs, off_ptrs = ptr_array(class_streams), ptr_array(payload_streams), ptr_array(row_offsets)
+    cls_bytes = (ctypes.c_int64 * max(len(class_streams), 1))(*[t.numel() for t in class_streams])
+    pay_bytes = (ctypes.c_int64 * n_classes)(*[t.numel() for t in payload_streams])
+    bits = (ctypes.c_int * n_classes)(*[int(b) for b in payload_bits])
+    base = (ctypes.c_uint32 * n_classes)(*[int(b) for b in payload_base])
+    y = torch.empty((m, n), device=x.device, dtype=x.dtype)
+    b32 = _bias_f32(bias)
+    _lib.call(
+        "npamd_vq_gemv_coded", x.data_ptr(), x.stride(0), int(flat), n_classes,
+        ctypes.addressof(cls_ptrs), ctypes.addressof(cls_bytes), ctypes.addressof(pay_ptrs), ctypes.addressof(pay_bytes),
+        ctypes.addressof(bits), ctypes.addressof(base), ctypes.addressof(off_ptrs),
+        cb.data_ptr(), _DT[cb.dtype], cb.shape[0], int(vector_len), _ptr(b32), y.data_ptr(), n, m, n, k,
+        _DT[x.dtype], _stream(x),
+    )  # fmt: skip
+    return y
+
+
+def vq_linear_tiered(
+    x: torch.Tensor,
+    prefix_stream: torch.Tensor,
+    hot_stream: torch.Tensor,
+    cold_stream: torch.Tensor,
+    hot_row_off: torch.Tensor,
+    cold_row_off: torch.Tensor,
+    centroids: torch.Tensor,
+    cold_bits: int,
+    hot_bits: int,
+    vector_len: int,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Decode GEMV over a two-tier prefix-coded buffer, ``M <= 16`` (reference:
+    neuropress/kernels/__init__.py:589-659).  The caller splits the buffer into its streams and
+    passes ``TieredIndexPacking.compute_row_offsets`` (on the device)."""
+    return _vq_linear_coded("vq_linear_tiered", x, 0, [prefix_stream], [hot_stream, cold_stream],
+                            [hot_bits, cold_bits], [0, 0], [hot_row_off, cold_row_off], centroids, vector_len, bias)
+
+
+def vq_linear_ntier(
+    x: torch.Tensor,
+    prefix_streams: list[torch.Tensor],
+    tier_streams: list[torch.Tensor],
+    row_offsets: list[torch.Tensor],
+    centroids: torch.Tensor,
+    tier_bits: list[int],
+    vector_len: int,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Decode GEMV over an n-tier (cascaded prefix) buffer, ``M <= 16`` (reference:
+    neuropress/kernels/__init__.py:711-762)."""
+    base = [0] + [1 << int(b) for b in tier_bits[:-1]]
+    return _vq_linear_coded("vq_linear_ntier", x, 0, list(prefix_streams), list(tier_streams), list(tier_bits), base,
+                            list(row_offsets), centroids, vector_len, bias)
+
+
+def vq_linear_zero_escape(
+    x: torch.Tensor,
+    prefix_stream: torch.Tensor,
+    hot_stream: torch.Tensor,
+    warm_stream: torch.Tensor,
+    cold_stream: torch.Tensor,
+    row_off_zero: torch.Tensor,
+    row_off_hot: torch.Tensor,
+    row_off_warm: torch.Tensor,
+    row_off_cold: torch.Tensor,
+    centroids: torch.Tensor,
+    cold_bits: int,
+    vector_len: int,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Decode GEMV over a zero-escape buffer (two class bits per index), ``M <= 16`` (reference:
+    neuropress/kernels/__init__.py:974-1049)."""
+    empty = prefix_stream.new_empty(0)
+    return _vq_linear_coded("vq_linear_zero_escape", x, 1, [prefix_stream], [empty, hot_stream, warm_stream, cold_stream],
+                            [0, 4, 8, cold_bits], [0, 1, 17, 257],
+                            [row_off_zero, row_off_hot, row_off_warm, row_off_cold], centroids, vector_len, bias)
+
+
 def vq_linear_wmma(
     x: torch.Tensor,
     packed_indices: torch.Tensor,

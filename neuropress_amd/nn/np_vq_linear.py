@@ -99,6 +99,9 @@ _TILE_MIN_GRID_FRACTION: float = 0.7
 # tokens, 39 vs 36 us at 256.
 _TILE_SPLIT_MAX_TOKENS: int = 128
 _TILE_SPLIT_LONG_K: int = 8192  # from this many input features on, _TILE_MAX_TOKENS applies
+# Layers of at least this many indices time their slice-list GEMV against the fused one when the
+# lists are built (NPVQLinear._sliced_token_limit).
+_SLICED_TUNE_MIN_INDICES: int = 1 << 20
 # Residual layers (two lookups and three fp16 operations per weight) decode faster in one
 # pass than inside the GEMM: 4096 x 4096, 17-384 tokens, tile 39-57 us against 30-41 us for
 # decode + GEMM; 14336 x 4096 88-119 against 74-102 us.  Only where the dense GEMM itself is
@@ -537,7 +540,11 @@ class NPVQLinear(nn.Module):
         """Band dispatch by token count (reference: neuropress/nn/np_vq_linear.py:1014-1058)."""
         if self.backend in _FUSED_BACKENDS and x.dtype in (torch.float16, torch.bfloat16):
             m = x.numel() // self.in_features
-            if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and self._sliced_ready(x):
+            if (
+                m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend))
+                and self._sliced_ready(x)
+                and m <= self._derived.get("sliced_max_tokens", _SLICED_MAX_TOKENS)
+            ):
                 return self._forward_sliced(x)  # applies column_perm inside the kernel
             if self.column_perm is not None and self._perm_fusable(x, m):
                 return self._fused(x, tile=False, perm=self._perm_i32(x.device))
@@ -594,11 +601,70 @@ class NPVQLinear(nn.Module):
         if sl is None or sl.blob.device != self.packed_indices.device:
             from .. import kernels
 
-            self._derived["sliced"] = kernels.vq_slice_indices(
+            sl = kernels.vq_slice_indices(
                 self.packed_indices, self.bits, self.out_features, self.in_features,
                 self.vector_len, self.proxy.num_centroids,
             )  # fmt: skip
+            self._derived["sliced"] = sl
+            self._derived["sliced_max_tokens"] = self._sliced_token_limit(sl)
         return True
+
+    def _sliced_token_limit(self, sl) -> int:
+        """Most tokens for which this layer's slice-list GEMV beats its fused GEMV.
+
+        With indices spread evenly over the codebook the slice lists win up to
+        ``_SLICED_MAX_TOKENS`` by a wide margin.  A skewed index distribution (one codebook
+        slice holding most of the indices) does two things: the hot slice's workgroups
+        carry more of the work, or outnumber the compute units, and the fused GEMV's
+        lookups start hitting in L1.  Which one wins then depends on the layer (14336 x
+        4096, Zipf(0.7) / Zipf(1.1): one token 16.5 vs 30 / 17 vs 15 us, four tokens 27 vs
+        30 / 28 vs 16 us; 4096 x 4096, Zipf(1.1): 8.1 vs 5.7 us), so every layer of the
+        size the path is meant for is timed here, once, when its lists are built."""
+        if self.n_vectors < _SLICED_TUNE_MIN_INDICES:
+            return _SLICED_MAX_TOKENS
+        dev = sl.blob.device
+        from .. import kernels
+
+        dt = torch.float16
+        cb = self.proxy.centroids_as(dt)
+        stream, bits = self._kernel_stream()
+
+        def timed(fn) -> float:
+            # GPU time, not issue time: eight calls captured in a HIP graph and replayed (launched
+            # eagerly, both kernels finish faster than Python can issue them).
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):
+                fn()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for _ in range(8):
+                        fn()
+                graph.replay()
+                t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t0.record()
+                for _ in range(3):
+                    graph.replay()
+                t1.record()
+                t1.synchronize()
+            torch.cuda.current_stream(dev).wait_stream(side)
+            return t0.elapsed_time(t1)
+
+        limit = 0
+        try:
+            for m in (1, 2, 4, _SLICED_MAX_TOKENS):
+                if m > _SLICED_MAX_TOKENS:
+                    break
+                x = torch.ones(m, self.in_features, dtype=dt, device=dev)
+                t_sliced = timed(lambda: kernels.vq_linear_sliced(x, sl, cb))
+                t_fused = timed(lambda: kernels.vq_linear(x, stream, cb, bits, self.vector_len, None, self.out_features))
+                if t_sliced >= t_fused:
+                    break
+                limit = m
+        except RuntimeError:
+            # e.g. another thread of the process is capturing a graph: keep the measured default
+            return _SLICED_MAX_TOKENS
+        return limit
 
     def _sliced_ready(self, x: torch.Tensor) -> bool:
         if not (x.is_cuda and self._sliced_eligible()):

@@ -191,6 +191,14 @@ class TieredIndexPacking:
         return n, n_hot, cold_bits, hot_bits, prefix, hot, cold
 
     @staticmethod
+    def split_streams(packed: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, int, int]:
+        """``(prefix_stream, hot_stream, cold_stream, cold_bits, hot_bits)``: views of the buffer in
+        the order ``kernels.vq_linear_tiered`` takes them (the reference splits the same way at
+        module construction, nn/np_vq_linear.py:644-696)."""
+        _, _, cold_bits, hot_bits, prefix, hot, cold = TieredIndexPacking._split(packed)
+        return prefix, hot, cold, cold_bits, hot_bits
+
+    @staticmethod
     def unpack(packed: torch.Tensor) -> torch.Tensor:
         n, n_hot, cold_bits, hot_bits, prefix, hot, cold = TieredIndexPacking._split(packed)
         tier_of = _unpack_narrow(prefix, 1, n)
@@ -297,6 +305,24 @@ class NTieredIndexPacking:
             raise ValueError(f"NTieredIndexPacking: buffer too short for {d} tiers ({packed.numel()} < {size}).")
         pairs = _header_words(packed, 3 + 2 * d)[3:]
         return n, d, pairs[0::2], pairs[1::2], size
+
+    @staticmethod
+    def split_streams(packed: torch.Tensor) -> tuple[list[torch.Tensor], list[torch.Tensor], list[int]]:
+        """``(prefix_streams, tier_streams, tier_bits)``: views of the buffer in the order
+        ``kernels.vq_linear_ntier`` takes them."""
+        n, d, counts, bits, at = NTieredIndexPacking._parse_header(packed)
+        prefixes, alive_n = [], n
+        for k in range(d - 1):
+            nb = (alive_n + 7) // 8
+            prefixes.append(packed[at : at + nb])
+            at += nb
+            alive_n -= counts[k]
+        tiers = []
+        for k in range(d):
+            nb = _payload_nbytes(counts[k], bits[k])
+            tiers.append(packed[at : at + nb])
+            at += nb
+        return prefixes, tiers, list(bits)
 
     @staticmethod
     def _tiers_and_payloads(packed: torch.Tensor):
@@ -407,6 +433,18 @@ class ZeroEscapePacking:
                 f"ZeroEscapePacking: bad magic 0x{magic:08X}, expected 0x{ZeroEscapePacking.MAGIC:08X}."
             )
         return n, cold_bits, n_zero, n_hot, n_warm, size
+
+    @staticmethod
+    def split_streams(packed: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, int]:
+        """``(class_stream, hot_stream, warm_stream, cold_stream, cold_bits)``: views of the buffer in
+        the order ``kernels.vq_linear_zero_escape`` takes them."""
+        n, cold_bits, n_zero, n_hot, n_warm, at = ZeroEscapePacking._parse_header(packed)
+        out = []
+        for nb in ((2 * n + 7) // 8, _payload_nbytes(n_hot, 4), _payload_nbytes(n_warm, 8),
+                   _payload_nbytes(n - n_zero - n_hot - n_warm, cold_bits)):
+            out.append(packed[at : at + nb])
+            at += nb
+        return out[0], out[1], out[2], out[3], cold_bits
 
     @staticmethod
     def _classes_and_payloads(packed: torch.Tensor):

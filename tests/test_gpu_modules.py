@@ -135,6 +135,31 @@ def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch
         assert calls == expect
 
 
+def test_skewed_layers_time_the_sliced_gemv_against_the_fused_one(gpu):
+    """Full-size layers are timed when their slice lists are built and take the slice-list GEMV only
+    for the token counts where it won.  Evenly spread indices: it wins at least at one token.
+    Zipf(1.1) indices put nine tenths of them in one codebook slice, where the fused GEMV's lookups
+    hit in L1: the limit can only be lower.  Results are right on either path."""
+    n, k, nc = 4096, 4096, 65536
+    g = cases.gen(91)
+    cb = (torch.randn(nc, 8, generator=g) * 0.02).half()
+    x = (torch.randn(4, k, generator=g) * 0.5).half()
+    limits = {}
+    for name, idx in (("uniform", torch.randint(0, nc, (n * k // 8,), generator=g)),
+                      ("zipf", cases.zipf_indices(g, nc, n * k // 8))):
+        packed = idx.to(torch.int32).to(torch.int16).view(torch.uint8)
+        layer = NPVQLinear(VQProxy(cb).to(gpu), packed, 16, n, k, 8, "cuda_wmma").to(gpu)
+        assert layer.prepare_sliced()
+        limits[name] = layer._derived["sliced_max_tokens"]
+        w = cb[idx].reshape(n, k).float()
+        for m in (1, 4):
+            _close(layer(x[:m].to(gpu)), x[:m].float() @ w.T)
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert 1 <= limits["uniform"] <= vqmod._SLICED_MAX_TOKENS  # one token: 8 us against 12 or more
+    assert 0 <= limits["zipf"] <= limits["uniform"]
+    print("slice-list token limits:", limits, "on", cus, "compute units")
+
+
 def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch):
     """2-bit group quantization and vector length 2 have no MFMA kernel: the modules decode once and
     call the dense GEMM at every token count instead of the fused entry points (whose element-wise
