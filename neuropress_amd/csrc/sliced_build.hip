@@ -115,36 +115,67 @@ struct Geometry {
   int64_t workgroups = 0;
 };
 
+constexpr double kSlicedStartupShare = 0.7;  // a workgroup's start-up time in units of a 1 / target share of the layer
+
 Geometry plan_geometry(int N, int G, const std::vector<int64_t>& slice_count, int64_t n_idx, int target) {
   const int S = (int)slice_count.size();
   const int rb_min = (N + kSlicedTasks - 1) / kSlicedTasks;
   const int kp_min = (G + kSlicedMaxGroups - 1) / kSlicedMaxGroups;
+  std::vector<double> share((size_t)S);
+  std::vector<int> kp_max((size_t)S);
+  for (int s = 0; s < S; ++s) {
+    share[s] = (double)slice_count[s] / (double)n_idx;
+    // Group ranges no finer than about 16 entries per row and range: a workgroup pays for
+    // loading its slice.
+    kp_max[s] = std::max(kp_min, (int)((double)G * share[s] / 16.0 + 0.5));
+  }
   Geometry best;
   double best_cost = 0;
+  // Cost of a geometry: rounds of workgroups over the compute units times (the heaviest
+  // workgroup + the charge for starting one: launch, record and slice loads, barrier, about
+  // 3.9 us, against 5.5 us of streaming for a 1 / target share of a 14336 x 4096 layer).
+  auto consider = [&](Geometry& geo) {
+    geo.workgroups = 0;
+    double heaviest = 0;
+    for (int s = 0; s < S; ++s) {
+      geo.workgroups += (int64_t)geo.parts[s] * geo.row_blocks;
+      heaviest = std::max(heaviest, share[s] / ((double)geo.parts[s] * geo.row_blocks));
+    }
+    const double rounds = (double)((geo.workgroups + target - 1) / target);
+    const double cost = rounds * (heaviest + kSlicedStartupShare / (double)target);
+    if (best.workgroups == 0 || cost < best_cost - 1e-12) {
+      best = geo;
+      best_cost = cost;
+    }
+  };
   for (int rb = rb_min; rb <= 2 * rb_min + 1; ++rb) {
     Geometry geo;
     geo.row_blocks = rb;
     geo.rows_per_block = (N + rb - 1) / rb;
     geo.parts.resize((size_t)S);
-    double heaviest = 0;
+    // (1) Group ranges in proportion to the slice's load (may need more than one round).
     for (int s = 0; s < S; ++s) {
-      const double share = (double)slice_count[s] / (double)n_idx;
-      // Group ranges in proportion to the slice's load, but no finer than about
-      // 16 entries per row and range: a workgroup pays for loading its slice.
-      const int kp_max = std::max(kp_min, (int)((double)G * share / 16.0 + 0.5));
-      int kp = (int)((double)target * share / rb + 0.5);
-      kp = std::max(kp_min, std::min(kp, kp_max));
-      geo.parts[s] = kp;
-      geo.workgroups += (int64_t)kp * rb;
-      heaviest = std::max(heaviest, share / ((double)kp * rb));
+      const int kp = (int)((double)target * share[s] / rb + 0.5);
+      geo.parts[s] = std::max(kp_min, std::min(kp, kp_max[s]));
     }
-    // Rounds of workgroups over the compute units times the heaviest workgroup,
-    // plus a charge per round for loading a slice.
-    const double rounds = (double)((geo.workgroups + target - 1) / target);
-    const double cost = rounds * (heaviest + 0.25 / (double)target);
-    if (best.workgroups == 0 || cost < best_cost - 1e-12) {
-      best = geo;
-      best_cost = cost;
+    consider(geo);
+    // (2) The best that fits one round: start from the fewest ranges and keep splitting the
+    // heaviest slice while the compute units are not all taken.
+    if ((int64_t)S * kp_min * rb <= target) {
+      for (int s = 0; s < S; ++s) geo.parts[s] = kp_min;
+      int64_t used = (int64_t)S * kp_min * rb;
+      while (used + rb <= target) {
+        int pick = -1;
+        double worst = 0;
+        for (int s = 0; s < S; ++s) {
+          const double load = share[s] / ((double)geo.parts[s] * rb);
+          if (geo.parts[s] < kp_max[s] && load > worst) { worst = load; pick = s; }
+        }
+        if (pick < 0) break;
+        geo.parts[pick]++;
+        used += rb;
+      }
+      consider(geo);
     }
   }
   return best;

@@ -617,8 +617,8 @@ class NPVQLinear(nn.Module):
         slice holding most of the indices) does two things: the hot slice's workgroups
         carry more of the work, or outnumber the compute units, and the fused GEMV's
         lookups start hitting in L1.  Which one wins then depends on the layer (14336 x
-        4096, Zipf(0.7) / Zipf(1.1): one token 16.5 vs 30 / 17 vs 15 us, four tokens 27 vs
-        30 / 28 vs 16 us; 4096 x 4096, Zipf(1.1): 8.1 vs 5.7 us), so every layer of the
+        4096, Zipf(0.7) / Zipf(1.1): one token 15.5 vs 30 / 17 vs 15 us, four tokens 29 vs
+        30 / 29 vs 16 us; 4096 x 4096, Zipf(1.1): 8.1 vs 5.7 us), so every layer of the
         size the path is meant for is timed here, once, when its lists are built."""
         if self.n_vectors < _SLICED_TUNE_MIN_INDICES:
             return _SLICED_MAX_TOKENS
