@@ -261,6 +261,23 @@ def test_vq_gemm_tile_fast_path(gpu, oracle_lib, act, bits, nc, m, vl):
     _check(y, _vq_ref(oracle_lib, L, act))
 
 
+@pytest.mark.parametrize("k", [64, 128, 192])
+@pytest.mark.parametrize("m", [1, 130, 300])
+def test_tile_gemm_short_reductions(gpu, oracle_lib, k, m):
+    """One to three 64-k steps: fewer steps than x tiles in flight (two or three) and than the
+    producers' pipeline is deep, so every prefetch past the end re-reads the last step."""
+    from neuropress_amd import kernels
+
+    for nc, bits in ((256, 8), (65536, 16)):
+        L = cases.vq_layer(640 + k + m, 150, k, nc, bits=bits, act=torch.bfloat16, m=m, bias=True, std=0.05)
+        y = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, 150, L["bias"].to(gpu))
+        _check(y, _vq_ref(oracle_lib, L, torch.bfloat16))
+    for nbits in (4, 8):
+        Q = cases.q4_layer(650 + k + m, 150, k, nbits=nbits, gs=32, act=torch.float16, m=m, bias=True)
+        y = kernels.q_gemm_tile(Q["x"].to(gpu), Q["blob"].to(gpu), Q["scale"].to(gpu), nbits, 32, None, Q["bias"].to(gpu))
+        _check(y, _q_ref(oracle_lib, Q, torch.float16))
+
+
 def _rvq_ref(oracle_lib, L, act):
     code = orc.torch_dtype_code(act)
     w = oracle_lib.rvq_decode(L["pm"].numpy(), L["bm"], L["pr"].numpy(), L["br"], orc.to_bits(L["cbm"]),
