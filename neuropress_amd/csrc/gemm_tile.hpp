@@ -208,8 +208,17 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   const int c = lane & 31;
   const int h = lane >> 5;
   const int wrow0 = wave * (32 * MW);              // first tile row of this wave
-  const bool wave_active = (m0 + wrow0) < s.M;     // waves past M compute on clamped rows and never store
+  const bool wave_active = (m0 + wrow0) < s.M;     // false: every row of this wave lies past M
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(s.x);
+
+  if (!wave_active) {
+    // All of this wave's rows lie past M (17..96 tokens leave one to three of the four consumers
+    // without rows): it only keeps the others' barriers company, instead of reading the W tile and
+    // running MFMAs on clamped rows -- at few tokens the LDS traffic per step sets the pace.
+    block_sync_lds();
+    for (int t = 0; t < total; ++t) block_sync_lds();
+    return;
+  }
 
   f32x16 acc[MW][2];
 #pragma unroll
@@ -225,7 +234,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   // a scalar base (the wave's first row, this step's chunk) plus a 32-bit lane offset.
   constexpr int kPiecesW = 4 * MW;
   constexpr int kBufs = XS::kBufs;
-  const int base_row = min(m0 + wrow0, s.M - 1);          // waves past M re-read the last row
+  const int base_row = m0 + wrow0;                         // < M: waves without rows have left
   const uint8_t* const xbase = reinterpret_cast<const uint8_t*>(xg + (int64_t)base_row * s.ldx);
   uint32_t voff[kPiecesW];
 #pragma unroll
@@ -334,7 +343,6 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: D[m = 8*(i/4) + 4h + i%4][n = c] --------------------------
-  if (!wave_active) return;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int n = n0 + t * 32 + c;
