@@ -38,8 +38,10 @@ extern "C" {
 #define NPAMD_ERR_UNSUPPORTED (-2) /* valid request this build has no kernel for */
 #define NPAMD_ERR_LAUNCH (-3)      /* HIP reported an error at launch */
 
-/* Largest token count the fused decode-GEMV entry points accept. */
-#define NPAMD_GEMV_MAX_M 16
+/* Largest token count the fused decode-GEMV entry points accept.  Up to 16 tokens are one MFMA
+ * operand; 17..32 reuse every decoded weight operand for two (the slice-list, prefix-coded and
+ * element-wise kernels take further passes over the weight instead). */
+#define NPAMD_GEMV_MAX_M 32
 
 /* Library ABI version (bumped on any signature change). */
 int npamd_version(void);
@@ -78,8 +80,8 @@ int npamd_vq_gemv(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_b
  * i.e. vq_linear applied to x[..., column_perm] (neuropress/nn/np_vq_linear.py:1027-1028)
  * without the separate gather kernel.  column_perm: K int32 column numbers, each < K,
  * 16-byte aligned.  Every workgroup copies the M rows of x into LDS and permutes them there,
- * so this entry point takes M * K <= 16384 elements, VL = 8, 4/8/12/16-bit indices and
- * K % 64 == 0 only;
+ * so this entry point takes M <= 16 tokens, M * K <= 16384 elements, VL = 8 or 4,
+ * 4/8/12/16-bit indices and K % 64 == 0 only;
  * other requests return NPAMD_ERR_UNSUPPORTED (gather x yourself and call npamd_vq_gemv).
  */
 int npamd_vq_gemv_perm(const void* x, int64_t ldx, const int32_t* column_perm,

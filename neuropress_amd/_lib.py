@@ -14,7 +14,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libnpamd.so"
 
 F16, BF16, F32 = 0, 1, 2
-GEMV_MAX_M = 16
+GEMV_MAX_M = 32
 ABI_VERSION = 2
 
 _vp = ctypes.c_void_p

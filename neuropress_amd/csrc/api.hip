@@ -59,7 +59,7 @@ bool gemv_lds_codebook_enabled() { return env_int("NPAMD_GEMV_LDS_CB", 1) != 0; 
 bool tile_lds_codebook_enabled() { return env_int("NPAMD_TILE_LDS_CB", 1) != 0; }
 bool gemv_lds_activations_forced() { return env_int("NPAMD_GEMV_LDS_X", 0) != 0; }
 
-GemvPlan plan_gemv(int N, int chunks, int max_r) {
+GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {
   const int steps = (chunks + 3) / 4;
   const int tiles = (N + 15) / 16;
   const int64_t jobs = (int64_t)tiles * steps;
@@ -79,7 +79,8 @@ GemvPlan plan_gemv(int N, int chunks, int max_r) {
   if (r_env == 1 || r_env == 2 || r_env == 4) p.R = r_env;
   const int spw_env = env_int("NPAMD_GEMV_SPW", 0);
   if (spw_env > 0) spw = spw_env;
-  const int max_waves = p.R >= 4 ? 8 : 16;
+  int max_waves = p.R >= 4 ? 8 : 16;
+  if (max_waves > max_waves_cap) max_waves = max_waves_cap;
   if ((steps + spw - 1) / spw > max_waves) spw = (steps + max_waves - 1) / max_waves;
   p.steps_per_wave = spw;
   p.waves = (steps + spw - 1) / spw;

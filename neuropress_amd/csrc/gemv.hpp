@@ -1,4 +1,4 @@
-// Fused decode GEMV for small token counts (M <= 16), wave64 + MFMA 16x16x32.
+// Fused decode GEMV for small token counts (M <= 32), wave64 + MFMA 16x16x32.
 //
 // The contraction y[m, n] = sum_k x[m, k] * W[n, k] is issued as
 // D[16 x 16] += A[16 x 32] * B[32 x 16] with A = x (rows m, zero beyond M) and
@@ -6,7 +6,8 @@
 //   A: x[m = c][8 consecutive k of k-slot q]      (16 bytes, zero if c >= M)
 //   B: W[n = n0 + c][the same 8 k]                (16 bytes = one VQ codebook row)
 // so a gathered codebook row is already a B-operand: no LDS, no VALU work on
-// the weights, and M = 1 ... 16 all cost the same.  The kernel is bound by the
+// the weights, and M = 1 ... 16 all cost the same (17 ... 32 tokens: two token
+// tiles, each weight operand feeds two MFMAs).  The kernel is bound by the
 // packed-weight stream from HBM plus, for codebooks larger than L1, the
 // 16-byte gathers out of L2.
 //
@@ -40,8 +41,10 @@ constexpr int kGemvLdsActivationsMax = 16 * 1024;
 
 // R = 4 keeps 32 gathered operands (128 registers) live per lane, so it is
 // limited to 8 waves per block; R <= 2 fits the 128-register budget of 16 waves.
-template <int R>
-constexpr int kGemvMaxWaves = (R >= 4) ? 8 : 16;
+// MT = 2 (17..32 tokens: two MFMA row tiles of tokens share every weight operand) holds a
+// second set of eight x operands and accumulators: 8 waves at up to 256 registers.
+template <int R, int MT = 1>
+constexpr int kGemvMaxWaves = (R >= 4 || MT >= 2) ? 8 : 16;
 
 // CB_LDS: the block first copies the whole codebook into LDS and gathers from
 // there (ds_read_b128) instead of from L1/L2.  Pays off when the table is too
@@ -50,8 +53,8 @@ constexpr int kGemvMaxWaves = (R >= 4) ? 8 : 16;
 // column permutation s.perm on the way when there is one, and reads its A
 // operands from there: the gather x[m, perm[k]] costs K element loads per block
 // instead of a kernel of its own in front of this one.
-template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS>
-__global__ void __launch_bounds__(kGemvMaxWaves<R> * 64)
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS, int MT = 1>
+__global__ void __launch_bounds__((kGemvMaxWaves<R, MT> * 64))
 fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][M][16*R] (+ codebook copy)
   Provider prov(pargs);
@@ -62,7 +65,9 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   // While x is being permuted its unpermuted copy lies where the codebook goes afterwards, so
   // the region in front of x is max(codebook, x) bytes.
   const int red_floats = (n_waves * s.M * 16 * R + 3) & ~3;
-  uint8_t* const lds0 = reinterpret_cast<uint8_t*>(red) + red_floats * (int)sizeof(float);
+  // Without a copy of x the reduction buffer, needed only after the loop, lies over the codebook.
+  constexpr bool kRedOverCodebook = CB_LDS && !X_LDS;
+  uint8_t* const lds0 = reinterpret_cast<uint8_t*>(red) + (kRedOverCodebook ? 0 : red_floats * (int)sizeof(float));
   int cb_lds_bytes = 0;
   if constexpr (CB_LDS) cb_lds_bytes = prov.codebook_vec16() * 16;
   const uint16_t* x_lds = nullptr;
@@ -113,19 +118,26 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   const int q = lane >> 4;
   const int row0 = blockIdx.x * (16 * R);
 
-  f32x4 acc[R];
+  f32x4 acc[R][MT];
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int step_begin = wave * s.steps_per_wave;
   const int step_end = min(step_begin + s.steps_per_wave, s.steps);
   // Loads are branch-free: out-of-range lanes read a clamped (valid) address and
   // their operand is zeroed afterwards, so all gathers of a step are in flight
   // together instead of each sitting behind its own branch and wait.
-  const int x_row = min(c, s.M - 1);
-  const uint16_t* xrow = X_LDS ? x_lds + (int64_t)x_row * (s.chunks * 64)
-                               : reinterpret_cast<const uint16_t*>(s.x) + (int64_t)x_row * s.ldx;
-  const bool x_lane = c < s.M;
+  const uint16_t* xrow[MT];
+  bool x_lane[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int x_row = min(16 * t + c, s.M - 1);
+    xrow[t] = X_LDS ? x_lds + (int64_t)x_row * (s.chunks * 64)
+                    : reinterpret_cast<const uint16_t*>(s.x) + (int64_t)x_row * s.ldx;
+    x_lane[t] = 16 * t + c < s.M;
+  }
   const u32x4 zero4{0, 0, 0, 0};
 
   for (int step = step_begin; step < step_end; ++step) {
@@ -137,12 +149,14 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
 #pragma unroll
     for (int r = 0; r < R; ++r) prov.load(raw[r], min(row0 + 16 * r + c, s.N - 1), kc);
 
-    u32x4 xa[8];
+    u32x4 xa[MT][8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      xa[j] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)kc * 64 + j * 8);
-      xa[j] = (x_lane && kvalid) ? xa[j] : zero4;
-    }
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        xa[t][j] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kc * 64 + j * 8);
+        xa[t][j] = (x_lane[t] && kvalid) ? xa[t][j] : zero4;
+      }
 
     // Rows past N are computed on a clamped row and never stored; a k-slot past
     // K must contribute exactly zero, so its operands are zeroed (x is zero
@@ -168,18 +182,23 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] = mfma16<ACT>(xa[j], b[r][j], acc[r]);
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[r][t] = mfma16<ACT>(xa[t][j], b[r][j], acc[r][t]);
   }
 
-  // D layout: lane (c, q) holds D[m = 4q + i][n = c], i = 0..3.
+  if constexpr (kRedOverCodebook) __syncthreads();  // every wave is done with the codebook
+  // D layout: lane (c, q) holds D[m = 16t + 4q + i][n = c], i = 0..3, for token tile t.
   const int cols = 16 * R;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = 4 * q + i;
-      if (m < s.M) red[((int64_t)wave * s.M + m) * cols + r * 16 + c] = acc[r][i];
-    }
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = 16 * t + 4 * q + i;
+        if (m < s.M) red[((int64_t)wave * s.M + m) * cols + r * 16 + c] = acc[r][t][i];
+      }
   }
   __syncthreads();
   for (int o = threadIdx.x; o < s.M * cols; o += blockDim.x) {
@@ -203,36 +222,39 @@ struct GemvPlan {
   int steps_per_wave;
 };
 
-// max_r: most row tiles per block the caller wants (4, or 2 for lookups served by L2).
-GemvPlan plan_gemv(int N, int chunks, int max_r = 4);
+// max_r: most row tiles per block the caller wants (4, or 2 for lookups served by L2);
+// max_waves_cap: most waves per block its kernel variant is built for.
+GemvPlan plan_gemv(int N, int chunks, int max_r = 4, int max_waves_cap = 16);
 
 // Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
 bool gemv_lds_activations_forced();  // NPAMD_GEMV_LDS_X=1: stage x in LDS also without a permutation (tuning aid)
 
-template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false>
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false, int MT = 1>
 int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const GemvPlan& plan,
                         int cb_bytes, hipStream_t st, const char* what) {
   s.steps_per_wave = plan.steps_per_wave;
   const int blocks = (s.N + 16 * R - 1) / (16 * R);
-  const int red_floats = (plan.waves * s.M * 16 * R + 3) & ~3;
+  const int red_bytes = ((plan.waves * s.M * 16 * R + 3) & ~3) * (int)sizeof(float);
   const int x_bytes = X_LDS ? s.M * s.chunks * 64 * 2 : 0;
   const int cb_lds_bytes = CB_LDS ? cb_bytes : 0;
-  const int lds = red_floats * (int)sizeof(float) + x_bytes +
-                  ((X_LDS && s.perm) ? (cb_lds_bytes > x_bytes ? cb_lds_bytes : x_bytes) : cb_lds_bytes);
+  const int lds = (CB_LDS && !X_LDS)
+                      ? (red_bytes > cb_lds_bytes ? red_bytes : cb_lds_bytes)
+                      : red_bytes + x_bytes +
+                            ((X_LDS && s.perm) ? (cb_lds_bytes > x_bytes ? cb_lds_bytes : x_bytes) : cb_lds_bytes);
   if (lds > 64 * 1024) {
     static int reserved = 0;  // per instantiation: largest dynamic-LDS size enabled so far
     if (lds > reserved) {
       const hipError_t e = hipFuncSetAttribute(
-          reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS>),
+          reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT>),
           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
       if (e != hipSuccess)
         return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
       reserved = lds;
     }
   }
-  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
+  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);
 }
 
@@ -251,6 +273,23 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
     cb_in_lds = cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled();
   // Lookups that go to L2 want many waves in flight more than they want shared x operands
   // (14336 x 4096, 65536-row codebook, one token: 34.6 us with two row tiles, 37.2 with four).
+  if (s.M > 16) {
+    // 17..32 tokens: two token tiles per weight operand, eight waves.  Every block reads all of
+    // x, twice as much as at 16 tokens, so four row tiles per block (half the blocks) pay more
+    // than anywhere else: 14336 x 4096, 4096-row codebook, 17 tokens: 20.0 us at R = 2, 12.9 at 4.
+    const GemvPlan plan = plan_gemv(s.N, s.chunks, (Provider::kGathers && !cb_in_lds) ? 2 : 4, 8);
+    if constexpr (Provider::kLdsCodebook) {
+      if (cb_in_lds) {
+        if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
+        if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
+        return launch_fused_gemv_r<ACT, Provider, 1, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
+      }
+    }
+    if constexpr (!Provider::kGathers)
+      if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, false, false, 2>(s, pargs, plan, 0, st, what);
+    if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, false, false, 2>(s, pargs, plan, 0, st, what);
+    return launch_fused_gemv_r<ACT, Provider, 1, false, false, 2>(s, pargs, plan, 0, st, what);
+  }
   const GemvPlan plan = plan_gemv(s.N, s.chunks, (Provider::kGathers && !cb_in_lds) ? 2 : 4);
   if constexpr (Provider::kLdsCodebook) {
     const bool x_fits = (int64_t)s.M * s.chunks * 64 <= kGemvLdsActivationsMax;

@@ -48,10 +48,10 @@ int dispatch(const VqCall& c) {
   GemvShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K / 64, 0, 0};
   if (c.perm) {
     // The gather is done while x is copied to LDS, which only the MFMA kernel for plain VQ does.
-    if (!(fast_ok(c) && !c.packed_r && (int64_t)c.M * c.K <= kGemvLdsActivationsMax && aligned(c.perm, 16)))
+    if (!(fast_ok(c) && !c.packed_r && c.M <= 16 && (int64_t)c.M * c.K <= kGemvLdsActivationsMax && aligned(c.perm, 16)))
       return fail(NPAMD_ERR_UNSUPPORTED,
                   "%s: column_perm needs VL = 8 or 4, 4/8/12/16-bit indices, K %% 64 == 0, 16-byte aligned "
-                  "buffers and M * K <= %d (got M=%d K=%d)", c.what, kGemvLdsActivationsMax, c.M, c.K);
+                  "buffers, M <= 16 and M * K <= %d (got M=%d K=%d)", c.what, kGemvLdsActivationsMax, c.M, c.K);
     s.perm = c.perm;
   }
   if (fast_ok(c)) {
@@ -103,7 +103,7 @@ extern "C" int npamd_vq_fused_supported(int K, int vl, int bits) {
 
 extern "C" int npamd_vq_gemv_perm_supported(int M, int N, int K, int nc, int vl, int bits) {
   const bool bits_ok = bits == 4 || bits == 8 || bits == 12 || bits == 16;
-  if (!((vl == 8 || vl == 4) && bits_ok && K > 0 && K % 64 == 0 && M >= 1 && M <= NPAMD_GEMV_MAX_M && N >= 1 && nc >= 1)) return 0;
+  if (!((vl == 8 || vl == 4) && bits_ok && K > 0 && K % 64 == 0 && M >= 1 && M <= 16 && N >= 1 && nc >= 1)) return 0;
   if ((int64_t)M * K > kGemvLdsActivationsMax) return 0;
   return gemv_perm_keeps_occupancy(M, N, K / 64, vl == 8 ? nc * 16 : (nc % 2 == 0 ? nc * 8 : 0)) ? 1 : 0;
 }

@@ -229,7 +229,7 @@ def vq_linear(
     out_features: int | None = None,
     column_perm: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Fused decode GEMV, ``M <= 16`` (reference: neuropress/kernels/__init__.py:209-245).
+    """Fused decode GEMV, ``M <= 32`` (reference: neuropress/kernels/__init__.py:209-245).
 
     ``column_perm`` (int32 ``[K]``, optional, not in the reference's signature): compute
     ``vq_linear(x[..., column_perm], ...)`` with the gather done inside the kernel; see
@@ -245,7 +245,7 @@ def vq_linear(
 
 def vq_linear_perm_supported(m: int, n: int, k: int, num_centroids: int, vector_len: int, bits: int) -> bool:
     """Whether :func:`vq_linear` should be given ``column_perm`` for this shape: the kernel takes it
-    (``M * K <= 16384``, VL 8, 4/8/12/16-bit indices, ``K % 64 == 0``) and its LDS copy of x
+    (``M <= 16``, ``M * K <= 16384``, VL 8 or 4, 4/8/12/16-bit indices, ``K % 64 == 0``) and its LDS copy of x
     does not reduce the workgroups per compute unit."""
     return bool(_lib.load().npamd_vq_gemv_perm_supported(int(m), int(n), int(k), int(num_centroids),
                                                          int(vector_len), int(bits)))  # fmt: skip
@@ -352,7 +352,7 @@ def vq_linear_sliced(
     partials_only: bool = False,
     column_perm: torch.Tensor | None = None,
 ) -> torch.Tensor | None:
-    """Decode GEMV over the slice-list form, ``M <= 16`` (``npamd_vq_gemv_sliced``).
+    """Decode GEMV over the slice-list form, ``M <= 32`` (``npamd_vq_gemv_sliced``).
 
     *centroids* must already be in ``x.dtype`` (the modules cache that copy).
     *workspace*: optional float32 scratch of ``sliced.workspace_bytes(M) / 4`` elements;
@@ -452,7 +452,7 @@ def vq_linear_tiered(
     vector_len: int,
     bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Decode GEMV over a two-tier prefix-coded buffer, ``M <= 16`` (reference:
+    """Decode GEMV over a two-tier prefix-coded buffer, ``M <= 32`` (reference:
     neuropress/kernels/__init__.py:589-659).  The caller splits the buffer into its streams and
     passes ``TieredIndexPacking.compute_row_offsets`` (on the device)."""
     return _vq_linear_coded("vq_linear_tiered", x, 0, [prefix_stream], [hot_stream, cold_stream],
@@ -469,7 +469,7 @@ def vq_linear_ntier(
     vector_len: int,
     bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Decode GEMV over an n-tier (cascaded prefix) buffer, ``M <= 16`` (reference:
+    """Decode GEMV over an n-tier (cascaded prefix) buffer, ``M <= 32`` (reference:
     neuropress/kernels/__init__.py:711-762)."""
     base = [0] + [1 << int(b) for b in tier_bits[:-1]]
     return _vq_linear_coded("vq_linear_ntier", x, 0, list(prefix_streams), list(tier_streams), list(tier_bits), base,
@@ -491,7 +491,7 @@ def vq_linear_zero_escape(
     vector_len: int,
     bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Decode GEMV over a zero-escape buffer (two class bits per index), ``M <= 16`` (reference:
+    """Decode GEMV over a zero-escape buffer (two class bits per index), ``M <= 32`` (reference:
     neuropress/kernels/__init__.py:974-1049)."""
     empty = prefix_stream.new_empty(0)
     return _vq_linear_coded("vq_linear_zero_escape", x, 1, [prefix_stream], [empty, hot_stream, warm_stream, cold_stream],
@@ -510,7 +510,7 @@ def vq_linear_wmma(
 ) -> torch.Tensor:
     """GEMV/GEMM auto-dispatch on M (reference: neuropress/kernels/__init__.py:335-354).
 
-    ``M <= 16`` runs the fused GEMV, larger M the tile-decode MFMA GEMM.
+    ``M <= 32`` runs the fused GEMV, larger M the tile-decode MFMA GEMM.
     """
     if centroids.dim() == 2 and centroids.shape[1] != vector_len:
         raise RuntimeError("vq_linear_wmma: vector_len does not match the codebook")
@@ -589,7 +589,7 @@ def rvq_linear(
     bias: torch.Tensor | None = None,
     tile: bool | None = None,
 ) -> torch.Tensor:
-    """Fused residual-VQ linear; ``tile=None`` picks GEMV for ``M <= 16`` else the tile GEMM."""
+    """Fused residual-VQ linear; ``tile=None`` picks GEMV for ``M <= 32`` else the tile GEMM."""
     what = "rvq_linear"
     _check_device(what, x, packed_main, packed_res, centroids_main, centroids_res)
     x = _x2d(x, what)
@@ -696,7 +696,7 @@ def q_linear(
 ) -> torch.Tensor:
     """Fused group-quantized dequant + linear (reference: neuropress/kernels/__init__.py:109-151).
 
-    ``M <= 16`` runs the fused GEMV, larger M the fused MFMA GEMM; the reference
+    ``M <= 32`` runs the fused GEMV, larger M the fused MFMA GEMM; the reference
     runs its GEMV at every M (neuropress/kernels/q4_linear.cu:137-139).
     """
     m = x.numel() // x.shape[-1] if x.shape[-1] else 0

@@ -50,6 +50,13 @@ _Q_TILE_MIN_GRID_FRACTION: float = 0.7
 _Q_TILE_SPLIT_MAX_TOKENS: int = 256
 _Q_TILE_SPLIT_LONG_K: int = 8192
 _Q_FUSED_MAX_TOKENS: int = 16
+# 17..32 tokens: the GEMV reuses every dequantized operand for two 16-token tiles, and each
+# workgroup reads all of x from L2, so it beats the fused GEMM while x is small.  Measured
+# (GEMV vs fused GEMM, 17 / 24 / 32 tokens): int4 14336 x 4096 17.0 / 17.8 / 19.9 vs 26-28 us,
+# 4096 x 14336 25.5 / 29.5 / 33.8 vs 28 us; with zero points 21-24 vs 41-43 us and 29-37 vs 41 us;
+# int8 14336 x 4096 22-25 vs 25-27 us, 4096 x 14336 28-37 vs 26-27 us.
+_Q_FUSED_WIDE_MAX_TOKENS: int = 32
+_Q_FUSED_WIDE_MAX_ACTIVATIONS = {4: 1 << 18, 8: 1 << 17}  # tokens x in_features, by bit width
 
 _ALLOW_FALLBACK: bool = os.environ.get("NEUROPRESS_ALLOW_KERNEL_FALLBACK", "").strip() in (
     "1", "true", "yes",
@@ -291,6 +298,16 @@ class NPLinear(nn.Module):
             _Q_TILE_MIN_GRID_FRACTION, _Q_TILE_SPLIT_MAX_TOKENS, _Q_TILE_SPLIT_LONG_K,
         )  # fmt: skip
 
+    def _gemv_max_tokens(self, m: int) -> int:
+        """End of the GEMV band for a call of *m* tokens: 16, or 32 while x stays small."""
+        if _Q_FUSED_MAX_TOKENS < m <= _Q_FUSED_WIDE_MAX_TOKENS:
+            cap = _Q_FUSED_WIDE_MAX_ACTIVATIONS.get(self.nbits, 0)
+            if self.zero_point is not None and self.nbits == 4:
+                cap = 1 << 30  # the fused GEMM pays for the zero points per tile: GEMV at any K
+            if m * self.in_features <= cap:
+                return _Q_FUSED_WIDE_MAX_TOKENS
+        return _Q_FUSED_MAX_TOKENS
+
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:
         """HIP path by token count; takes the place of np_linear.py:731-761."""
         if not x.is_cuda:
@@ -303,13 +320,14 @@ class NPLinear(nn.Module):
             # element-wise kernel, slower at every token count than decoding once and calling the
             # dense GEMM (14336 x 4096, 8 bits: 99 us against 57 us at one token, 452 against 57 at 16).
             fused_ok = x.dtype in (torch.float16, torch.bfloat16) and self._mfma_layer()
-            if fused_ok and m > _Q_FUSED_MAX_TOKENS:
+            gemv_max = self._gemv_max_tokens(m)
+            if fused_ok and m > gemv_max:
                 limit = _Q_TILE_MAX_TOKENS
                 if self.in_features >= _Q_TILE_SPLIT_LONG_K:
                     limit = max(limit, _Q_TILE_LONG_K_MAX_TOKENS)
                 fused_ok = m <= limit and self._tile_grid_fills_gpu(x, m)
             if fused_ok:
-                if m <= _Q_FUSED_MAX_TOKENS:
+                if m <= gemv_max:
                     return kernels.q_linear(
                         x, self.u8_blob, self.scale, self.nbits, self.group_size,
                         self.zero_point, self._bias_f32(),

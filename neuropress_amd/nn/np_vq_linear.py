@@ -15,15 +15,16 @@ token count ``m = x.numel() // in_features``:
 ====================  ==============================  ==========================
 band                  condition                        kernel
 ====================  ==============================  ==========================
-(a) fused GEMV        ``m <= _FUSED_MAX_TOKENS``       ``kernels.vq_linear``
+(a) fused GEMV        ``m <= _FUSED_MAX_TOKENS``, or   ``kernels.vq_linear``
+                      ``m <= 32`` while x is small
 (b) tile-decode GEMM  ``m <= _TILE_MAX_TOKENS``        ``kernels.vq_gemm_tile``
 (c) decode + GEMM     otherwise                        ``kernels.vq_dequant`` + ``F.linear``
 ====================  ==============================  ==========================
 
 The dispatch rule itself is the reference's (np_vq_linear.py:1014-1058); the
 thresholds are re-derived for one MI355X and stay overridable through the same
-environment variables.  Entropy-coded index formats (tiered / n-tier /
-zero-escape) are not supported and are rejected at construction.
+environment variables.  Prefix-coded index formats (tiered / n-tier /
+zero-escape) are expanded to the fixed-width stream once, at construction.
 """
 
 from __future__ import annotations
@@ -61,6 +62,15 @@ def _env_int(names: tuple[str, ...], default: int) -> int:
 # contraction as 16-row MFMA tiles, so 1..16 tokens cost the same: the fused
 # band ends at 16 here (2 in the reference, whose GEMV re-reads the weight per token).
 _FUSED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_FUSED_MAX_TOKENS",), 16)
+# 17..32 tokens: the GEMV reuses every decoded operand for two 16-token tiles.  Each of its
+# workgroups reads all of x from L2, so it wins while x is small (tokens x in_features at most
+# _FUSED_WIDE_MAX_ACTIVATIONS).  Measured, GEMV vs tile GEMM at 17 / 24 / 32 tokens, bf16:
+# 14336 x 4096, 4096-row codebook 12.9 / 14.6 / 16.2 vs 27 us, 65536-row 42 / 44 / 47 vs 46-50 us;
+# 4096 x 4096 8.7 / 9.8 / 11.1 vs 16 us; 4096 x 14336 22.4 / 26.4 / 31.2 vs 28 us.  Residual
+# layers 35-41 vs 70 us (14336 x 4096) and 41-50 vs 74 us (4096 x 14336): GEMV at any length.
+_FUSED_WIDE_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_FUSED_WIDE_MAX_TOKENS",), 32)
+_FUSED_WIDE_MAX_ACTIVATIONS: int = 1 << 18
+_GEMV_KERNEL_MAX_TOKENS: int = 32  # what the GEMV entry points accept (NPAMD_GEMV_MAX_M)
 
 # Decode steps (1-7 tokens) of layers whose codebook is too large to sit in a
 # compute unit's LDS next to the GEMV's buffers (more than 4096 rows): the fused
@@ -559,7 +569,7 @@ class NPVQLinear(nn.Module):
                 # the dense GEMM at every token count (14336 x 4096: 99 us against 57 us at one token).
                 return self._forward_dequant_gemm(x)
             m = x.numel() // self.in_features
-            if m > _fused_max_tokens(self.backend):
+            if m > self._gemv_max_tokens(m):
                 if (
                     self.backend != VQBackend.CUDA_LUT
                     and m <= _TILE_MAX_TOKENS
@@ -683,6 +693,14 @@ class NPVQLinear(nn.Module):
             perm = self.column_perm.to(device=device, dtype=torch.int32).contiguous()
             self._derived["perm_i32"] = perm
         return perm
+
+    def _gemv_max_tokens(self, m: int) -> int:
+        """End of band (a) for a call of *m* tokens: the fused limit, or 32 while x stays small."""
+        limit = _fused_max_tokens(self.backend)
+        if limit == 16 and 16 < m <= min(_FUSED_WIDE_MAX_TOKENS, 32):
+            if self.is_residual or m * self.in_features <= _FUSED_WIDE_MAX_ACTIVATIONS:
+                return 32
+        return limit
 
     def _perm_fusable(self, x: torch.Tensor, m: int) -> bool:
         """Whether the fused GEMV gathers ``x[..., column_perm]`` itself for this call."""
@@ -872,14 +890,14 @@ class NPVQLinear(nn.Module):
 
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:
         """Band (a) (reference: np_vq_linear.py:1173-1187).  Above the kernel's
-        16-token limit (reachable only with a raised threshold) the tile GEMM runs."""
+        32-token limit (reachable only with a raised threshold) the tile GEMM runs."""
         m = x.numel() // self.in_features
-        return self._fused(x, tile=m > 16)
+        return self._fused(x, tile=m > _GEMV_KERNEL_MAX_TOKENS)
 
     def _forward_cuda_wmma(self, x: torch.Tensor) -> torch.Tensor:
         """GEMV / GEMM by token count (reference: np_vq_linear.py:1250-1267)."""
         m = x.numel() // self.in_features
-        return self._fused(x, tile=m > 16)
+        return self._fused(x, tile=m > _GEMV_KERNEL_MAX_TOKENS)
 
     def _forward_cuda_lut(self, x: torch.Tensor) -> torch.Tensor:
         """Reached only when ``_LUT_MAX_TOKENS`` was raised above 0.
@@ -890,7 +908,7 @@ class NPVQLinear(nn.Module):
         it is not rebuilt.  The same result is produced by the fused kernels.
         """
         m = x.numel() // self.in_features
-        return self._fused(x, tile=m > 16)
+        return self._fused(x, tile=m > _GEMV_KERNEL_MAX_TOKENS)
 
     # ------------------------------------------------------------------
 

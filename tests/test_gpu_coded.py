@@ -128,7 +128,7 @@ def test_coded_gemv_argument_errors(gpu):
     with pytest.raises(RuntimeError, match="float16 or bfloat16"):
         kernels.vq_linear_tiered(L["x"].float().to(gpu), *args)
     with pytest.raises(RuntimeError, match="exceeds the fused limit"):
-        kernels.vq_linear_tiered(torch.zeros(17, 64, dtype=torch.float16, device=gpu), *args)
+        kernels.vq_linear_tiered(torch.zeros(33, 64, dtype=torch.float16, device=gpu), *args)
     bad = list(args)
     bad[3] = d(hot_off)[:-1]
     with pytest.raises(RuntimeError, match="N \\+ 1 entries"):

@@ -151,7 +151,7 @@ def _check(y: torch.Tensor, ref: np.ndarray):
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,nc", [(4, 16), (8, 256), (12, 4096), (16, 65536)])
-@pytest.mark.parametrize("m", [1, 2, 5, 16])
+@pytest.mark.parametrize("m", [1, 2, 5, 16, 17, 32])
 @pytest.mark.parametrize("vl", [8, 4])
 def test_vq_gemv_fast_path(gpu, oracle_lib, act, bits, nc, m, vl):
     from neuropress_amd import kernels
@@ -287,7 +287,7 @@ def _rvq_ref(oracle_lib, L, act):
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,tile", [(1, False), (4, False), (4, True), (150, True)])
+@pytest.mark.parametrize("m,tile", [(1, False), (4, False), (25, False), (4, True), (150, True)])
 def test_rvq_linear(gpu, oracle_lib, act, m, tile):
     from neuropress_amd import kernels
 
@@ -359,7 +359,7 @@ def test_q4_linear_fast_path(gpu, oracle_lib, act, gs, m, nbits, asym):
 
 
 @pytest.mark.parametrize("rows", [1, 2, 4])
-@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("m", [1, 5, 16, 29])
 def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
     """The fused GEMV shares x between 1, 2 or 4 row tiles of a block; which one a layer gets
     depends on its row count and the device's size, so every variant is forced here (tuning
@@ -374,7 +374,7 @@ def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
         dev = {key: L[key].to(gpu) for key in ("x", "packed", "cb", "bias")}
         y = kernels.vq_linear(dev["x"], dev["packed"], dev["cb"], bits, 8, dev["bias"], out_features=n)
         _check(y, _vq_ref(oracle_lib, L, torch.bfloat16))
-        if nc == 256:
+        if nc == 256 and m <= 16:  # the permuted GEMV takes up to 16 tokens
             perm = torch.randperm(k, generator=cases.gen(3 + m))
             yp = kernels.vq_linear(dev["x"], dev["packed"], dev["cb"], bits, 8, dev["bias"], out_features=n,
                                    column_perm=perm.to(torch.int32).to(gpu))
@@ -428,6 +428,8 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
     wt = w.t().contiguous()  # [K, N]: row k is what token "one-hot k" must produce
     for k0 in (0, 48, k - 16):
         assert torch.equal(gemv(eye[k0:k0 + 16]), wt[k0:k0 + 16]), f"GEMV, rows {k0}.."
+    assert torch.equal(gemv(eye[40:72]), wt[40:72]), "GEMV, 32 tokens (two token tiles)"
+    assert torch.equal(gemv(eye[5:26]), wt[5:26]), "GEMV, 21 tokens"
     assert torch.equal(gemv(eye[7:9]), wt[7:9])   # two tokens (int4: still the MFMA kernel)
     assert torch.equal(tile(eye), wt), "tile GEMM, 1024 tokens"
     assert torch.equal(tile(eye[100:330]), wt[100:330]), "tile GEMM, 230 tokens"
@@ -474,7 +476,7 @@ def test_empty_and_error_paths(gpu):
     with pytest.raises(RuntimeError, match="bits"):
         kernels.vq_dequant(packed, cb, 3, 16, 64, torch.float16)
     with pytest.raises(RuntimeError, match="exceeds the fused limit"):
-        kernels.vq_linear(torch.zeros(17, 64, device=gpu, dtype=torch.float16), packed, cb, 8, 8, None, 16)
+        kernels.vq_linear(torch.zeros(33, 64, device=gpu, dtype=torch.float16), packed, cb, 8, 8, None, 16)
     with pytest.raises(RuntimeError, match="GPU"):
         kernels.vq_dequant(L["packed"], L["cb"], 8, 16, 64, torch.float16)
     with pytest.raises(RuntimeError, match="float16 or bfloat16"):

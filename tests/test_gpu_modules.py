@@ -187,8 +187,9 @@ def test_layers_outside_the_mfma_kernels_go_to_decode_and_gemm(gpu, monkeypatch)
 
 
 def test_narrow_layers_take_the_split_tile_band(gpu, monkeypatch):
-    """A 2048 x 4096 layer has 32 column tiles: the module still routes 17..128 tokens (int4:
-    17..256) to the tile GEMM (which splits the reduction), and more tokens to decode + GEMM."""
+    """A 2048 x 4096 layer has 32 column tiles: up to 32 tokens run the GEMV, and the module still
+    routes 33..128 tokens (int4: 33..256) to the tile GEMM (which splits the reduction), and more
+    tokens to decode + GEMM."""
     import neuropress_amd.nn.np_linear as qmod
 
     L = cases.vq_layer(77, 2048, 4096, 4096, bits=12, bias=True, std=0.02)
@@ -205,11 +206,11 @@ def test_narrow_layers_take_the_split_tile_band(gpu, monkeypatch):
                             lambda *a, _real=real, _name=name, **kw: (calls.append((_name, a[0].shape[0])), _real(*a, **kw))[1])
     w = L["cb"][L["idx"]].reshape(2048, 4096).half().float()
     wq = ((Q["codes"].float() - 8).reshape(2048, 128, 32) * Q["scale"].float().reshape(2048, 128, 1)).reshape(2048, 4096)
-    for m in (17, 128, 129, 257):
+    for m in (17, 32, 33, 128, 129, 257):
         x = (torch.randn(m, 4096, generator=cases.gen(m)) * 0.5).half()
         _close(layer(x.to(gpu)), torch.nn.functional.linear(x.float(), w, L["bias"].float()))
         _close(qlayer(x.to(gpu)), torch.nn.functional.linear(x.float(), wq.half().float(), Q["bias"].float()))
-    assert calls == [("vq_gemm_tile", 17), ("q_gemm_tile", 17), ("vq_gemm_tile", 128), ("q_gemm_tile", 128),
+    assert calls == [("vq_gemm_tile", 33), ("q_gemm_tile", 33), ("vq_gemm_tile", 128), ("q_gemm_tile", 128),
                      ("q_gemm_tile", 129)]
     from neuropress_amd import _lib
 

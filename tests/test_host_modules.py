@@ -109,8 +109,9 @@ def test_residual_layer_torch_path_matches_definition():
 # ------------------------------------------------------------ band dispatch ---
 
 
-def _fused_layer_with_spies(monkeypatch, backend, lut_max_tokens=16, tile_max_tokens=0):
+def _fused_layer_with_spies(monkeypatch, backend, lut_max_tokens=16, tile_max_tokens=0, wide_max_tokens=16):
     monkeypatch.setattr(vqmod, "_FUSED_MAX_TOKENS", 16)
+    monkeypatch.setattr(vqmod, "_FUSED_WIDE_MAX_TOKENS", wide_max_tokens)  # 16: no 17..32-token GEMV band
     monkeypatch.setattr(vqmod, "_LUT_MAX_TOKENS", lut_max_tokens)
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", tile_max_tokens)
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
@@ -132,6 +133,22 @@ def test_mid_sized_batches_use_tile_band(monkeypatch, backend):
     for m in (16, 17, 64, 65):
         layer(torch.randn(m, 32, dtype=torch.float16))
     assert calls == ["fused", "tile", "tile", "dense"]
+
+
+def test_small_activations_keep_the_gemv_up_to_32_tokens(monkeypatch):
+    """17..32 tokens stay in band (a) while tokens x in_features is within the cap."""
+    layer, calls = _fused_layer_with_spies(monkeypatch, Backend.CUDA_WMMA, tile_max_tokens=64, wide_max_tokens=32)
+    for m in (16, 17, 32, 33):
+        layer(torch.randn(m, 32, dtype=torch.float16))
+    assert calls == ["fused", "fused", "fused", "tile"]
+    del calls[:]
+    monkeypatch.setattr(vqmod, "_FUSED_WIDE_MAX_ACTIVATIONS", 20 * 32)
+    for m in (17, 20, 21, 32):
+        layer(torch.randn(m, 32, dtype=torch.float16))
+    assert calls == ["fused", "fused", "tile", "tile"]
+    # a raised fused threshold is taken as given
+    monkeypatch.setattr(vqmod, "_FUSED_MAX_TOKENS", 24)
+    assert layer._gemv_max_tokens(30) == 24
 
 
 def test_lut_layers_skip_tile_band(monkeypatch):
@@ -351,7 +368,7 @@ def test_c_abi_validates_arguments_without_a_gpu():
     with pytest.raises(RuntimeError, match="not divisible"):
         _lib.call("npamd_vq_gemv", None, 64, None, 0, 8, None, 0, 16, 8, None, None, 4, 1, 4, 60, 0, None)
     with pytest.raises(RuntimeError, match="exceeds the fused limit"):
-        _lib.call("npamd_vq_gemv", None, 64, None, 1 << 20, 8, None, 0, 16, 8, None, None, 4, 17, 4, 64, 0, None)
+        _lib.call("npamd_vq_gemv", None, 64, None, 1 << 20, 8, None, 0, 16, 8, None, None, 4, 33, 4, 64, 0, None)
     _lib.call("npamd_vq_dequant", None, 0, 8, None, 16, 8, 0, None, 0, None)  # empty: success, no launch
     # entry points added around the path: same rule
     with pytest.raises(RuntimeError, match="row stride smaller than the row"):

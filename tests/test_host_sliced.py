@@ -178,7 +178,7 @@ def test_gemv_sliced_validates_before_touching_the_gpu():
     with pytest.raises(RuntimeError, match="f16 or bf16"):
         call(act=_lib.F32, cbdt=_lib.F32)
     with pytest.raises(RuntimeError, match="exceeds the fused limit"):
-        call(m=17)
+        call(m=33)
     with pytest.raises(RuntimeError, match="row stride"):
         call(ldx=k - 8)
     with pytest.raises(RuntimeError, match="null pointer"):
