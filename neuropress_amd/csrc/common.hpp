@@ -126,33 +126,61 @@ __device__ __forceinline__ uint32_t read_index(const uint8_t* __restrict__ packe
 // eight 16-bit values packed in four dwords, for the widths whose 8-index
 // group is a whole number of dwords.  The caller guarantees the group lies
 // inside the stream and the stream base is 16-byte aligned.
+// The two halves of that: the memory reads alone (BITS / 4 dwords, the rest of the vector
+// zero), and the arithmetic that spreads them into eight 16-bit fields.  A software pipeline
+// that requests packed bytes many iterations before it needs the indices keeps the raw
+// dwords and extracts at the point of use -- arithmetic on a loaded value placed next to the
+// load makes the compiler wait for the load there.
 template <int BITS>
-__device__ __forceinline__ u32x4 load_idx8(const uint8_t* __restrict__ packed, int64_t i0) {
+__device__ __forceinline__ u32x4 load_raw8(const uint8_t* __restrict__ packed, int64_t i0) {
   static_assert(BITS == 4 || BITS == 8 || BITS == 12 || BITS == 16, "fast widths only");
-  u32x4 r;
+  u32x4 r{0u, 0u, 0u, 0u};
   if constexpr (BITS == 16) {
     r = *reinterpret_cast<const u32x4*>(packed + i0 * 2);
   } else if constexpr (BITS == 8) {
     const u32x2 w = *reinterpret_cast<const u32x2*>(packed + i0);
-    r.x = (w.x & 0xFFu) | ((w.x & 0xFF00u) << 8);
-    r.y = ((w.x >> 16) & 0xFFu) | ((w.x >> 8) & 0xFF0000u);
-    r.z = (w.y & 0xFFu) | ((w.y & 0xFF00u) << 8);
-    r.w = ((w.y >> 16) & 0xFFu) | ((w.y >> 8) & 0xFF0000u);
+    r.x = w.x;
+    r.y = w.y;
   } else if constexpr (BITS == 4) {
-    const uint32_t w = *reinterpret_cast<const uint32_t*>(packed + (i0 >> 1));
+    r.x = *reinterpret_cast<const uint32_t*>(packed + (i0 >> 1));
+  } else {  // 12 bits: 8 indices in 3 dwords
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(packed + (i0 >> 3) * 12);
+    r.x = p[0];
+    r.y = p[1];
+    r.z = p[2];
+  }
+  return r;
+}
+
+template <int BITS>
+__device__ __forceinline__ u32x4 extract_idx8(const u32x4& raw) {
+  u32x4 r;
+  if constexpr (BITS == 16) {
+    r = raw;
+  } else if constexpr (BITS == 8) {
+    r.x = (raw.x & 0xFFu) | ((raw.x & 0xFF00u) << 8);
+    r.y = ((raw.x >> 16) & 0xFFu) | ((raw.x >> 8) & 0xFF0000u);
+    r.z = (raw.y & 0xFFu) | ((raw.y & 0xFF00u) << 8);
+    r.w = ((raw.y >> 16) & 0xFFu) | ((raw.y >> 8) & 0xFF0000u);
+  } else if constexpr (BITS == 4) {
+    const uint32_t w = raw.x;
     r.x = (w & 0xFu) | ((w & 0xF0u) << 12);
     r.y = ((w >> 8) & 0xFu) | ((w & 0xF000u) << 4);
     r.z = ((w >> 16) & 0xFu) | ((w >> 4) & 0xF0000u);
     r.w = ((w >> 24) & 0xFu) | ((w >> 12) & 0xF0000u);
-  } else {  // 12 bits: 8 indices in 3 dwords
-    const uint32_t* p = reinterpret_cast<const uint32_t*>(packed + (i0 >> 3) * 12);
-    const uint32_t a = p[0], b = p[1], c = p[2];
+  } else {
+    const uint32_t a = raw.x, b = raw.y, c = raw.z;
     r.x = (a & 0xFFFu) | ((a << 4) & 0x0FFF0000u);
     r.y = ((a >> 24) | ((b & 0xFu) << 8)) | ((b << 12) & 0x0FFF0000u);
     r.z = ((b >> 16) & 0xFFFu) | (((b >> 28) | ((c & 0xFFu) << 4)) << 16);
     r.w = ((c >> 8) & 0xFFFu) | ((c >> 4) & 0x0FFF0000u);
   }
   return r;
+}
+
+template <int BITS>
+__device__ __forceinline__ u32x4 load_idx8(const uint8_t* __restrict__ packed, int64_t i0) {
+  return extract_idx8<BITS>(load_raw8<BITS>(packed, i0));
 }
 
 __device__ __forceinline__ uint32_t idx8_get(const u32x4& v, int j) {

@@ -24,7 +24,9 @@
 //           into LDS (swizzled 128-byte rows); see XStage.
 //   W tile  [64][64 k], rows padded to 144 bytes, a ring of three.  Every
 //           producer decodes a quarter of every step's tile (16 columns x 8 operands; lane = column x
-//           operand pair), keeps kDepth steps in flight in registers and
+//           operand pair), keeps kDepth steps in flight in registers -- packed
+//           bytes and looked-up rows exactly as they arrived, all arithmetic on
+//           them deferred to the iteration that needs its result -- and
 //           writes a finished pair to LDS two iterations before its step.
 // One block barrier per macro-step, executed by all eight waves.  Because the
 // W tile of step t+1 is complete at the barrier that ends iteration t-1, a
@@ -74,6 +76,14 @@ constexpr int kDepth = 8;  // steps in flight per producer wave (2 operands each
 // registers are consumed.
 __device__ __forceinline__ void block_sync_lds() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+// The same, except that the wave's KEEP youngest LDS operations may still be in flight: LDS
+// operations of a wave complete in order, so everything issued before them (the producer's
+// stores into the W tile) is done, while the codebook lookups it issued after the stores, whose
+// results it needs many steps later, do not hold up the barrier.
+template <int KEEP>
+__device__ __forceinline__ void block_sync_lds_keep() {
+  asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(KEEP) : "memory");
 }
 
 // How the x tile reaches LDS: `global_load_lds_dwordx4` writes the loaded bytes straight into
@@ -153,29 +163,42 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     //      iterations ago,
     //   3. loads the packed bytes of step t+1+2*kDepth.
     // Loads are consumed in the order they were issued, so waiting for the
-    // oldest never drains the younger ones.
+    // oldest never drains the younger ones.  That only holds while nothing
+    // touches a loaded value before its turn: the providers keep packed bytes
+    // and looked-up rows as they arrived (load_pair, gather_pair) and do all
+    // arithmetic on them in the iteration that needs the result (gather_pair on
+    // the packed bytes, finish_pair on the rows) -- an index extraction or an
+    // fp16 -> bf16 conversion placed next to its load makes the compiler wait
+    // for that load, the youngest, and with it for every load in flight.
     const int q = wave - 4;
     const int col = 16 * q + (lane & 15);
     const int jp = lane >> 4;
     // Branch-free decode: columns past N and steps past the last one read
     // clamped (valid) addresses; their results land where nobody looks.
     const int ncol = min(n0 + col, s.N - 1);
+    prov.prepare_row(ncol);
     typename Provider::PairRaw raws[kDepth];
-    u32x4 ops[kDepth][2];
+    typename Provider::PairOps ops[kDepth];
+    // LDS lookups that may stay in flight across the step's barrier (codebook in LDS only).
+    constexpr int kKeep = CB_LDS ? Provider::kLdsOpsPerGather : 0;
     auto load_raw = [&](typename Provider::PairRaw& raw, int step) {
       prov.load_pair(raw, ncol, chunk_of(min(step, steps - 1)), jp);
     };
-    auto store_w = [&](const u32x4 (&b)[2], int slot) {
+    auto store_w = [&](const typename Provider::PairOps& o, int slot) {
+      u32x4 b0, b1;
+      prov.finish_pair(o, b0, b1);
       uint8_t* dst = ws + slot * kWBufBytes + col * kRowBytes + jp * 32;
-      *reinterpret_cast<u32x4*>(dst) = b[0];
-      *reinterpret_cast<u32x4*>(dst + 16) = b[1];
+      *reinterpret_cast<u32x4*>(dst) = b0;
+      *reinterpret_cast<u32x4*>(dst + 16) = b1;
     };
     // Iteration t: the operands of step t+2 (gathered kDepth iterations ago) go to ring slot
     // (t+2) % 3, their registers are refilled with the gathers of step t+2+kDepth, and the
-    // packed bytes of step t+2+2*kDepth are requested.
-    auto advance = [&](u32x4 (&b)[2], typename Provider::PairRaw& raw, int t, int slot) {
-      store_w(b, slot);
-      prov.operand_pair(raw, b[0], b[1]);
+    // packed bytes of step t+2+2*kDepth are requested.  The stores come first and the lookups
+    // after them, in that order in the instruction stream: block_sync_lds_keep counts on it.
+    auto advance = [&](typename Provider::PairOps& o, typename Provider::PairRaw& raw, int t, int slot) {
+      store_w(o, slot);
+      asm volatile("" ::: "memory");
+      prov.gather_pair(raw, jp, o);
       load_raw(raw, t + 2 + 2 * kDepth);
     };
 
@@ -184,7 +207,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p);
 #pragma unroll
-    for (int p = 0; p < kDepth; ++p) prov.operand_pair(raws[p], ops[p][0], ops[p][1]);
+    for (int p = 0; p < kDepth; ++p) prov.gather_pair(raws[p], jp, ops[p]);
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p + kDepth);
     advance(ops[0], raws[0], -2, 0);
@@ -198,7 +221,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
       for (int d = 0; d < kDepth; ++d) {
         advance(ops[(d + 2) % kDepth], raws[(d + 2) % kDepth], t0 + d, slot);
         slot = slot == kWRing - 1 ? 0 : slot + 1;
-        block_sync_lds();
+        block_sync_lds_keep<kKeep>();
       }
     }
     return;
@@ -251,16 +274,24 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
                  :: "s"(dst), "v"(voff[i]), "s"(src) : "memory");
   };
   auto tile_src = [&](int step) { return xbase + (int64_t)chunk_of(min(step, steps - 1)) * (kStepK * 2); };
+  // Operand sets in registers: the reads of k group j + kAhead are issued in front of the
+  // MFMAs of group j.  One group ahead: reading three ahead (four sets, a fourth x tile) at up
+  // to 128 tokens, where a group is only two MFMAs, changed nothing measurable.
+  constexpr int kSets = 2;
+  constexpr int kAhead = kSets - 1;
+  constexpr int kPieceOfGroup[4] = {0, (kPiecesW + 2) / 3, (2 * kPiecesW + 2) / 3, kPiecesW};
+  constexpr bool kIssueAtEnd = kBufs == 2;
   // The consumers issue no other vector memory instruction in the loop, so the in-order
-  // counter counts tiles: with tiles up to step + kBufs - 1 requested, tile step + 1 has
-  // landed once at most (kBufs - 2) tiles' worth of loads are outstanding.
-  constexpr int kOutstandingOk = (kBufs - 2) * kPiecesW;
+  // counter counts tiles.  The first read of tile step + 1 comes in front of group 4 - kAhead
+  // of step `step`; by then tiles up to step + kBufs - 2 are requested in full and of tile
+  // step + kBufs - 1 the pieces issued behind the groups before that one, so tile step + 1
+  // has landed once no more than those loads are outstanding.
+  constexpr int kOutstandingOk = kIssueAtEnd ? 0 : (kBufs - 3) * kPiecesW + kPieceOfGroup[4 - kAhead];
 
-  // With three tiles in LDS, tile step + 2 is requested behind the MFMAs of k groups 0..2 of
-  // step `step` (its buffer held tile step - 1).  With two, there is no such slack: tile
+  // With three or four tiles in LDS, tile step + kBufs - 1 is requested behind the MFMAs of k
+  // groups 0..2 of step `step` (its buffer held tile step - 1).  With two, there is no such slack: tile
   // step + 2 goes into the buffer of tile `step` itself, as soon as that tile's last operands
   // have been read (behind the MFMAs of group 3), which leaves it almost two steps to arrive.
-  constexpr bool kIssueAtEnd = kBufs == 2;
   constexpr int kPrologueTiles = kIssueAtEnd ? kBufs : kBufs - 1;
 #pragma unroll
   for (int p = 0; p < kPrologueTiles; ++p) {
@@ -271,7 +302,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"((kPrologueTiles - 1) * kPiecesW) : "memory");
   block_sync_lds();
 
-  u32x4 a[2][MW], b[2][2];
+  u32x4 a[kSets][MW], b[kSets][2];
   const uint32_t row_off = (uint32_t)((wrow0 + c) * XS::kXRowBytes);
   uint32_t slot_off[4];
 #pragma unroll
@@ -285,8 +316,6 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     for (int mt = 0; mt < MW; ++mt)
       a[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * XS::kXRowBytes);
   };
-  constexpr int kPieceOfGroup[4] = {0, (kPiecesW + 2) / 3, (2 * kPiecesW + 2) / 3, kPiecesW};
-
   // buf = step % kBufs (compile-time through the unrolled loops below).
   auto one_step = [&](int buf, int step, int wslot) {
     const int wnext = wslot == kWRing - 1 ? 0 : wslot + 1;
@@ -295,17 +324,18 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     const uint8_t* src = tile_src(kIssueAtEnd ? step + kBufs : step + kBufs - 1);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if (j < 3) {
-        read_ops((j + 1) & 1, buf, wslot, j + 1);
+      constexpr int kFirstOfNext = 4 - kAhead;  // the group in front of which the next step's tiles are first read
+      if (j < kFirstOfNext) {
+        read_ops((j + kAhead) % kSets, buf, wslot, j + kAhead);
       } else {
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kOutstandingOk) : "memory");
-        read_ops(0, nbuf, wnext, 0);
+        if (j == kFirstOfNext) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kOutstandingOk) : "memory");
+        read_ops((j + kAhead) % kSets, nbuf, wnext, j + kAhead - 4);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mt = 0; mt < MW; ++mt) {
-        acc[mt][0] = mfma32<ACT>(a[j & 1][mt], b[j & 1][0], acc[mt][0]);
-        acc[mt][1] = mfma32<ACT>(a[j & 1][mt], b[j & 1][1], acc[mt][1]);
+        acc[mt][0] = mfma32<ACT>(a[j % kSets][mt], b[j % kSets][0], acc[mt][0]);
+        acc[mt][1] = mfma32<ACT>(a[j % kSets][mt], b[j % kSets][1], acc[mt][1]);
       }
       if (!kIssueAtEnd && j < 3) {
 #pragma unroll
@@ -319,7 +349,8 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     }
   };
 
-  read_ops(0, 0, 0, 0);
+#pragma unroll
+  for (int g = 0; g < kAhead; ++g) read_ops(g, 0, 0, g);
   int wslot = 0;
   const int whole = steps / kBufs * kBufs;
   for (int t0 = 0; t0 < whole; t0 += kBufs) {

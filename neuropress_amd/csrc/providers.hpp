@@ -16,7 +16,9 @@
 // wave owns operands 2*jp and 2*jp+1 of its column:
 //
 //   load_pair(raw, n, kc, jp)     -- packed bytes for that operand pair
-//   operand_pair(raw, b0, b1)     -- the two operands
+//   gather_pair(raw, jp, ops)     -- issues the lookups (or dequantizes) for the two operands
+//   finish_pair(ops, b0, b1)      -- the two operands, once the producer is about to write them
+//   prepare_row(n)                -- once per producer lane: what its row needs besides packed bytes
 //
 // A B-operand of a VQ weight with VL = 8 is exactly one codebook row, so the
 // 16-byte gather lands in MFMA layout with no shuffling (VL = 4: two rows, two 8-byte gathers).  For int4 the eight
@@ -90,34 +92,41 @@ struct VqProvider {
     return c;
   }
 
+  // The tile GEMM's producers request packed bytes sixteen steps ahead: PairRaw holds what the
+  // load returned, untouched, and gather_pair extracts the indices when it looks them up.
+  __device__ __forceinline__ void prepare_row(int) {}  // nothing per row outside the packed bytes
   struct PairRaw {
-    uint32_t pair;   // VL = 8: indices of operands 2*jp (low half) and 2*jp+1 (high half)
-    uint32_t pair1;  // VL = 4: `pair` holds the two rows of operand 2*jp, `pair1` those of 2*jp+1
+    u32x4 w;  // the 8-index group that holds this lane's operands, as loaded
   };
   __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
     const int64_t i0 = ((int64_t)n * a.chunks + kc) * kIdxPerChunk;
+    // VL = 8: the four lane-groups of a column read the same 8-index group: one request.
+    // VL = 4: operands 2jp, 2jp+1 = indices 4jp .. 4jp+3, half of index group jp >> 1.
+    r.w = load_raw8<BITS>(a.packed, VL == 8 ? i0 : i0 + 8 * (jp >> 1));
+  }
+  // gather_pair only issues the lookups; what they return stays untouched in PairOps until the
+  // producer writes the pair, many steps later, and finish_pair converts it then.  Arithmetic
+  // on the looked-up rows next to the lookup would make the wave wait for it on the spot.
+  struct PairOps {
+    u32x4 b0, b1;
+  };
+  static constexpr int kLdsOpsPerGather = VL == 8 ? 2 : 4;  // LDS reads of one gather_pair from an LDS codebook
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o) const {
+    const u32x4 v = extract_idx8<BITS>(r.w);
     if constexpr (VL == 8) {
-      // the four lane-groups of a column read the same 8-index group: one request
-      r.pair = select_dword(load_idx8<BITS>(a.packed, i0), jp);
+      const uint32_t pair = select_dword(v, jp);  // indices of operands 2*jp (low half) and 2*jp+1
+      o.b0 = cb[min(pair & 0xFFFFu, a.nc_minus_1)];
+      o.b1 = cb[min(pair >> 16, a.nc_minus_1)];
     } else {
-      // operands 2jp, 2jp+1 = indices 4jp .. 4jp+3: dwords 2(jp&1), 2(jp&1)+1 of index group jp>>1
-      const u32x4 v = load_idx8<BITS>(a.packed, i0 + 8 * (jp >> 1));
-      r.pair = (jp & 1) ? v.z : v.x;
-      r.pair1 = (jp & 1) ? v.w : v.y;
+      const uint32_t pair = (jp & 1) ? v.z : v.x;   // the two rows of operand 2*jp
+      const uint32_t pair1 = (jp & 1) ? v.w : v.y;  // those of operand 2*jp+1
+      o.b0 = row_pair(pair & 0xFFFFu, pair >> 16);
+      o.b1 = row_pair(pair1 & 0xFFFFu, pair1 >> 16);
     }
   }
-  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
-    if constexpr (VL == 8) {
-      b0 = cb[min(r.pair & 0xFFFFu, a.nc_minus_1)];
-      b1 = cb[min(r.pair >> 16, a.nc_minus_1)];
-    } else {
-      b0 = row_pair(r.pair & 0xFFFFu, r.pair >> 16);
-      b1 = row_pair(r.pair1 & 0xFFFFu, r.pair1 >> 16);
-    }
-    if constexpr (CONV) {
-      b0 = cb_to_act<ACT>(b0);
-      b1 = cb_to_act<ACT>(b1);
-    }
+  __device__ __forceinline__ void finish_pair(const PairOps& o, u32x4& b0, u32x4& b1) const {
+    b0 = CONV ? cb_to_act<ACT>(o.b0) : o.b0;
+    b1 = CONV ? cb_to_act<ACT>(o.b1) : o.b1;
   }
 };
 
@@ -160,27 +169,43 @@ struct RvqProvider {
     return combine(idx8_get(r.im, J), idx8_get(r.ir, J), r.s2, r.b2);
   }
 
+  // As loaded (see VqProvider::PairRaw); the row's scale and bias do not change from step to
+  // step, so the producer reads them once (prepare_row) instead of with every pair.
   struct PairRaw {
-    uint32_t pm, pr, s2, b2;
+    u32x4 wm, wr;
   };
+  uint32_t s2 = 0x3C003C00u, b2 = 0u;  // scale (1.0) and bias of the producer lane's row, replicated pairs
+  __device__ __forceinline__ void prepare_row(int n) {
+    if (a.row_scale) s2 = (uint32_t)a.row_scale[n] * 0x10001u;
+    if (a.row_bias) b2 = (uint32_t)a.row_bias[n] * 0x10001u;
+  }
   __device__ __forceinline__ void load_pair(PairRaw& r, int n, int kc, int jp) const {
     const int64_t i0 = ((int64_t)n * a.chunks + kc) * 8;
-    r.pm = select_dword(load_idx8<BITS_M>(a.packed_m, i0), jp);
-    r.pr = select_dword(load_idx8<BITS_R>(a.packed_r, i0), jp);
-    r.s2 = 0x3C003C00u;
-    r.b2 = 0u;
-    if (a.row_scale) r.s2 = (uint32_t)a.row_scale[n] * 0x10001u;
-    if (a.row_bias) r.b2 = (uint32_t)a.row_bias[n] * 0x10001u;
+    r.wm = load_raw8<BITS_M>(a.packed_m, i0);
+    r.wr = load_raw8<BITS_R>(a.packed_r, i0);
   }
-  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
-    b0 = combine(r.pm & 0xFFFFu, r.pr & 0xFFFFu, r.s2, r.b2);
-    b1 = combine(r.pm >> 16, r.pr >> 16, r.s2, r.b2);
+  struct PairOps {
+    u32x4 cm0, cr0, cm1, cr1;  // main and residual rows of the two operands, as gathered
+  };
+  static constexpr int kLdsOpsPerGather = 0;  // both codebooks are gathered from memory
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o) const {
+    const uint32_t pm = select_dword(extract_idx8<BITS_M>(r.wm), jp);
+    const uint32_t pr = select_dword(extract_idx8<BITS_R>(r.wr), jp);
+    o.cm0 = a.cb_m[min(pm & 0xFFFFu, a.ncm_minus_1)];
+    o.cr0 = a.cb_r[min(pr & 0xFFFFu, a.ncr_minus_1)];
+    o.cm1 = a.cb_m[min(pm >> 16, a.ncm_minus_1)];
+    o.cr1 = a.cb_r[min(pr >> 16, a.ncr_minus_1)];
+  }
+  __device__ __forceinline__ void finish_pair(const PairOps& o, u32x4& b0, u32x4& b1) const {
+    b0 = combine_rows(o.cm0, o.cr0, s2, b2);
+    b1 = combine_rows(o.cm1, o.cr1, s2, b2);
   }
 
   __device__ __forceinline__ u32x4 combine(uint32_t im, uint32_t ir, uint32_t s2, uint32_t b2) const {
+    return combine_rows(a.cb_m[min(im, a.ncm_minus_1)], a.cb_r[min(ir, a.ncr_minus_1)], s2, b2);
+  }
+  __device__ __forceinline__ u32x4 combine_rows(const u32x4& cm, const u32x4& cr, uint32_t s2, uint32_t b2) const {
 #pragma clang fp contract(off)
-    const u32x4 cm = a.cb_m[min(im, a.ncm_minus_1)];
-    const u32x4 cr = a.cb_r[min(ir, a.ncr_minus_1)];
     const f16x2 s = __builtin_bit_cast(f16x2, s2);
     const f16x2 b = __builtin_bit_cast(f16x2, b2);
     const bool has_s = a.row_scale != nullptr, has_b = a.row_bias != nullptr;
@@ -251,6 +276,7 @@ struct Q4Provider {
     return dequant8(w, (J < 4) ? r.s_lo : r.s_hi, (J < 4) ? r.z_lo : r.z_hi);
   }
 
+  __device__ __forceinline__ void prepare_row(int) {}  // nothing per row outside the packed bytes
   struct PairRaw {
     u32x2 w;      // 16 nibbles = operands 2*jp, 2*jp+1
     uint32_t s2;  // their scale (one 32-k group), replicated
@@ -262,9 +288,17 @@ struct Q4Provider {
     r.s2 = (uint32_t)a.scale[g] * 0x10001u;
     if constexpr (ASYM) r.z = a.zp[g];
   }
-  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
-    b0 = dequant8(r.w.x, r.s2, r.z);
-    b1 = dequant8(r.w.y, r.s2, r.z);
+  struct PairOps {
+    u32x4 b0, b1;  // finished operands: the dequantization waits for nothing but the packed bytes
+  };
+  static constexpr int kLdsOpsPerGather = 0;
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int, PairOps& o) const {
+    o.b0 = dequant8(r.w.x, r.s2, r.z);
+    o.b1 = dequant8(r.w.y, r.s2, r.z);
+  }
+  __device__ __forceinline__ void finish_pair(const PairOps& o, u32x4& b0, u32x4& b1) const {
+    b0 = o.b0;
+    b1 = o.b1;
   }
 
   // Eight nibbles of one dword -> one operand, natural k order.
@@ -357,6 +391,7 @@ struct Q8Provider {
     return dequant8((J & 1) ? ww.z : ww.x, (J & 1) ? ww.w : ww.y, (J < 4) ? r.s_lo : r.s_hi, (J < 4) ? r.z_lo : r.z_hi);
   }
 
+  __device__ __forceinline__ void prepare_row(int) {}  // nothing per row outside the packed bytes
   struct PairRaw {
     u32x4 w;      // 16 bytes = operands 2*jp, 2*jp+1
     uint32_t s2;  // their scale (one 32-k group), replicated
@@ -368,9 +403,17 @@ struct Q8Provider {
     r.s2 = (uint32_t)a.scale[g] * 0x10001u;
     if constexpr (ASYM) r.z = a.zp[g];
   }
-  __device__ __forceinline__ void operand_pair(const PairRaw& r, u32x4& b0, u32x4& b1) const {
-    b0 = dequant8(r.w.x, r.w.y, r.s2, r.z);
-    b1 = dequant8(r.w.z, r.w.w, r.s2, r.z);
+  struct PairOps {
+    u32x4 b0, b1;  // finished operands
+  };
+  static constexpr int kLdsOpsPerGather = 0;
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int, PairOps& o) const {
+    o.b0 = dequant8(r.w.x, r.w.y, r.s2, r.z);
+    o.b1 = dequant8(r.w.z, r.w.w, r.s2, r.z);
+  }
+  __device__ __forceinline__ void finish_pair(const PairOps& o, u32x4& b0, u32x4& b1) const {
+    b0 = o.b0;
+    b1 = o.b1;
   }
 
   // Eight bytes (two dwords) -> one operand.

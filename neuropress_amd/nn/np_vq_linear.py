@@ -112,12 +112,11 @@ _TILE_SPLIT_LONG_K: int = 8192  # from this many input features on, _TILE_MAX_TO
 # Layers of at least this many indices time their slice-list GEMV against the fused one when the
 # lists are built (NPVQLinear._sliced_token_limit).
 _SLICED_TUNE_MIN_INDICES: int = 1 << 20
-# Residual layers (two lookups and three fp16 operations per weight) decode faster in one
-# pass than inside the GEMM: 4096 x 4096, 17-384 tokens, tile 39-57 us against 30-41 us for
-# decode + GEMM; 14336 x 4096 88-119 against 74-102 us.  Only where the dense GEMM itself is
-# slow (long reductions: 4096 x 14336, 64-384 tokens, 86-119 against 90-124 us) does the
-# tile band pay.
-_RVQ_TILE_MIN_K: int = 8192
+# Residual layers take the tile band under the same grid rule as plain ones.  Measured, tile
+# GEMM vs decode + GEMM, bf16, 33 / 128 / 256 tokens: 14336 x 4096 58 / 63 / 77 against 74 / 75 /
+# 91 us; 4096 x 4096 28 / 33 / 43 against 33 / 42 / 41 us; 4096 x 14336 60 / 68 / 89 against
+# 76 / 106 / 100 us; 1024 x 4096 (too few column blocks, decode + GEMM by the grid rule) 21 / 23 /
+# 28 against 24 / 21 / 22 us.
 
 # Opt-in: when a HIP kernel call fails, warn once and run torch ops instead (the
 # reference's behaviour).  Off by default so a missing or broken kernel library
@@ -749,8 +748,6 @@ class NPVQLinear(nn.Module):
         features) covers at least ``_TILE_MIN_GRID_FRACTION`` of the compute units."""
         if not x.is_cuda:
             return True
-        if self.is_residual and self.in_features < _RVQ_TILE_MIN_K:
-            return False
         if not self._mfma_layer():
             return False  # the tile entry point would run its element-wise fallback
         cus = self._derived.get("cus")

@@ -97,7 +97,6 @@ def test_nplinear_bands(gpu, act, monkeypatch):
 def test_residual_module_bands(gpu, monkeypatch):
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)  # small layers: force the tile band
-    monkeypatch.setattr(vqmod, "_RVQ_TILE_MIN_K", 0)
     L = cases.rvq_layer(12, 48, 256, nc_main=65536, nc_res=256)
     mk = lambda backend: NPVQLinear(VQProxy(L["cbm"]), L["pm"], L["bm"], 48, 256, 8, backend,
                                     residual_proxy=VQProxy(L["cbr"]), packed_residual=L["pr"],
@@ -111,9 +110,9 @@ def test_residual_module_bands(gpu, monkeypatch):
         _close(layer(x.to(gpu)), x.float() @ w.T)
 
 
-def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch):
-    """A residual layer with K < 8192 goes from the fused GEMV straight to decode + GEMM; with a
-    long reduction it takes the tile GEMM like a plain layer."""
+def test_residual_layers_take_the_gemv_to_32_tokens_and_then_the_tile_band(gpu, monkeypatch):
+    """A residual layer keeps the fused GEMV up to 32 tokens at any reduction length and takes the
+    tile GEMM above, like a plain layer."""
     from neuropress_amd import kernels
 
     calls = []
@@ -121,7 +120,7 @@ def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch
     monkeypatch.setattr(kernels, "rvq_linear",
                         lambda *a, _real=real, **kw: (calls.append((a[0].shape[0], kw.get("tile"))), _real(*a, **kw))[1])
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
-    for k, expect in ((256, [(4, False)]), (8192, [(4, False), (40, True)])):
+    for k, expect in ((256, [(4, False), (32, False), (40, True)]), (16384, [(4, False), (32, False), (40, True)])):
         L = cases.rvq_layer(21, 32, k, nc_main=4096, nc_res=16)
         layer = NPVQLinear(VQProxy(L["cbm"]), L["pm"], L["bm"], 32, k, 8, "cuda_wmma",
                            residual_proxy=VQProxy(L["cbr"]), packed_residual=L["pr"], residual_bits=L["br"],
@@ -129,7 +128,7 @@ def test_residual_layers_skip_the_tile_band_on_short_reductions(gpu, monkeypatch
         layer.proxy.to(gpu), layer.residual_proxy.to(gpu)
         w = layer._dense_weight_torch(torch.float16).float().cpu()
         calls.clear()
-        for m in (4, 40):
+        for m in (4, 32, 40):
             x = (torch.randn(m, k, generator=cases.gen(m)) * 0.3).half()
             _close(layer(x.to(gpu)), x.float() @ w.T)
         assert calls == expect
