@@ -117,13 +117,6 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   uint8_t* const xs = lds;                             // [XS::kBufs][BM][XS::kXRowBytes]
   uint8_t* const ws = lds + XS::kBufs * kXBufBytes;    // [kWRing][64][kRowBytes]
   Provider prov(pargs);
-  if constexpr (CB_LDS) {
-    u32x4* cb_lds = reinterpret_cast<u32x4*>(lds + XS::kLdsBytes);
-    const u32x4* src = prov.global_codebook();
-    for (int i = threadIdx.x; i < prov.codebook_vec16(); i += 512) cb_lds[i] = src[i];
-    prov.use_codebook(cb_lds);
-    __syncthreads();
-  }
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -149,6 +142,26 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   // The padding iterations decode clamped addresses into buffers nobody reads.
   const int total = (steps + kDepth - 1) / kDepth * kDepth;
 
+  // Producer lane: column 16q + l % 16 of the tile, operand pair jp = l / 16 (see below).  Its
+  // first packed bytes are requested here, in front of the codebook copy, so that the two
+  // memory round trips at the start of a block overlap instead of following each other.
+  const int pcol = 16 * (wave & 3) + (lane & 15);
+  const int jp = lane >> 4;
+  const int ncol = min(n0 + pcol, s.N - 1);  // columns past N read a clamped (valid) row
+  typename Provider::PairRaw raws[kDepth];
+  if (wave >= 4) {
+    prov.prepare_row(ncol);
+#pragma unroll
+    for (int p = 0; p < kDepth; ++p) prov.load_pair(raws[p], ncol, chunk_of(min(p, steps - 1)), jp);
+  }
+  if constexpr (CB_LDS) {
+    u32x4* cb_lds = reinterpret_cast<u32x4*>(lds + XS::kLdsBytes);
+    const u32x4* src = prov.global_codebook();
+    for (int i = threadIdx.x; i < prov.codebook_vec16(); i += 512) cb_lds[i] = src[i];
+    prov.use_codebook(cb_lds);
+    __syncthreads();
+  }
+
   if (wave >= 4) {
     // ====================== producer wave q ================================
     // Every producer works every iteration on a quarter of the W tile: lane
@@ -170,14 +183,9 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     // the packed bytes, finish_pair on the rows) -- an index extraction or an
     // fp16 -> bf16 conversion placed next to its load makes the compiler wait
     // for that load, the youngest, and with it for every load in flight.
-    const int q = wave - 4;
-    const int col = 16 * q + (lane & 15);
-    const int jp = lane >> 4;
     // Branch-free decode: columns past N and steps past the last one read
     // clamped (valid) addresses; their results land where nobody looks.
-    const int ncol = min(n0 + col, s.N - 1);
-    prov.prepare_row(ncol);
-    typename Provider::PairRaw raws[kDepth];
+    const int col = pcol;
     typename Provider::PairOps ops[kDepth];
     // LDS lookups that may stay in flight across the step's barrier (codebook in LDS only).
     constexpr int kKeep = CB_LDS ? Provider::kLdsOpsPerGather : 0;
@@ -205,9 +213,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     // Prologue: steps 0..kDepth-1 in flight, packed bytes of kDepth..2*kDepth-1 loaded; then
     // "iterations -2 and -1": store steps 0 and 1 and refill their registers.
 #pragma unroll
-    for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p);
-#pragma unroll
-    for (int p = 0; p < kDepth; ++p) prov.gather_pair(raws[p], jp, ops[p]);
+    for (int p = 0; p < kDepth; ++p) prov.gather_pair(raws[p], jp, ops[p]);  // packed bytes requested above
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p + kDepth);
     advance(ops[0], raws[0], -2, 0);
@@ -222,6 +228,12 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
         advance(ops[(d + 2) % kDepth], raws[(d + 2) % kDepth], t0 + d, slot);
         slot = slot == kWRing - 1 ? 0 : slot + 1;
         block_sync_lds_keep<kKeep>();
+        // Operands that come from memory: nothing moves from one step into another.  Left
+        // alone, the scheduler gathers the arithmetic of all kDepth steps of the unrolled body
+        // at its top, and with it their waits, the last of which is for the gathers issued one
+        // step earlier.  (With the codebook in LDS the free schedule already waits for the
+        // oldest load only, and is the faster one at 128 tokens.)
+        if constexpr (!CB_LDS) __builtin_amdgcn_sched_barrier(0);
       }
     }
     return;

@@ -113,10 +113,10 @@ _TILE_SPLIT_LONG_K: int = 8192  # from this many input features on, _TILE_MAX_TO
 # lists are built (NPVQLinear._sliced_token_limit).
 _SLICED_TUNE_MIN_INDICES: int = 1 << 20
 # Residual layers take the tile band under the same grid rule as plain ones.  Measured, tile
-# GEMM vs decode + GEMM, bf16, 33 / 128 / 256 tokens: 14336 x 4096 58 / 63 / 77 against 74 / 75 /
-# 91 us; 4096 x 4096 28 / 33 / 43 against 33 / 42 / 41 us; 4096 x 14336 60 / 68 / 89 against
-# 76 / 106 / 100 us; 1024 x 4096 (too few column blocks, decode + GEMM by the grid rule) 21 / 23 /
-# 28 against 24 / 21 / 22 us.
+# GEMM vs decode + GEMM, bf16, 33 / 128 / 256 tokens: 14336 x 4096 53 / 56 / 72 against 75 / 76 /
+# 92 us; 4096 x 4096 26 / 31 / 40 against 33 / 42 / 41 us; 4096 x 14336 54 / 63 / 84 against
+# 78 / 107 / 100 us; 1024 x 4096 (too few column blocks, decode + GEMM by the grid rule) 20 / 22 /
+# 27 against 24 / 21 / 22 us.
 
 # Opt-in: when a HIP kernel call fails, warn once and run torch ops instead (the
 # reference's behaviour).  Off by default so a missing or broken kernel library
