@@ -318,7 +318,7 @@ def main():
             add("cfg3 14336x4096 bf16", "a:sliced-gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
         del spool[1:]
         torch.cuda.empty_cache()
-        for m in (1, 2, 16):
+        for m in (1, 2, 16, 32):  # 32: two 16-token tiles per decoded operand
             xm = [torch.randn(m, k, generator=gen(50 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
             t = time_graph(lambda i: kernels.vq_linear(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n),
                            n_rot, steps_s * 2, 3, dev)
@@ -356,7 +356,7 @@ def main():
         del c3d
         torch.cuda.empty_cache()
         # config 2 gate/up (12-bit stream, 4096-entry codebook) and config 1
-        for name, (nn_, kk, nc, bits), ms in (("cfg2 8192x2048 f16 12-bit", (8192, 2048, 4096, 12), (1, 2)),
+        for name, (nn_, kk, nc, bits), ms in (("cfg2 8192x2048 f16 12-bit", (8192, 2048, 4096, 12), (1, 2, 32)),
                                               ("cfg1 2048x640 f16 8-bit", (2048, 640, 256, 8), (1, 16))):
             rot = max(2, min(256, POOL_BYTES // (nn_ * kk // 8 * bits // 8)))
             cc = vq_case(dev, 1002, nn_, kk, nc, bits, torch.float16, rot)
@@ -407,11 +407,14 @@ def main():
             pms = [pm.to(dev).clone() for _ in range(rot)]
             prs = [pr.to(dev).clone() for _ in range(rot)]
             alg4 = lambda m: cnt * 3 + (65536 + 256) * 16 + nn_ * 4 + m * kk * 2 + m * nn_ * 2
-            for m in (1, 384):
+            for m in (1, 32, 128, 384):
                 xm = [torch.randn(m, kk, generator=gen(40 + m)).to(torch.float16).to(dev) for _ in range(2)]
-                if m == 1:
+                if m <= 32:
                     f = lambda i: kernels.rvq_linear(xm[i % 2], pms[i], 16, prs[i], 8, cbm, cbr, rsc, rbi, nn_)
                     band = "a:fused-gemv"
+                elif m == 128:
+                    f = lambda i: kernels.rvq_linear(xm[i % 2], pms[i], 16, prs[i], 8, cbm, cbr, rsc, rbi, nn_, tile=True)
+                    band = "b:tile-gemm"
                 else:
                     f = lambda i: torch.nn.functional.linear(
                         xm[i % 2], kernels.rvq_dequant(pms[i], 16, prs[i], 8, cbm, cbr, rsc, rbi, nn_, kk, torch.float16))
@@ -430,11 +433,11 @@ def main():
         rot = max(2, POOL_BYTES // blob.numel())
         blobs = [blob.to(dev)]
         blobs += [blobs[0].clone() for _ in range(rot - 1)]
-        for m in (1, 16, 256):
+        for m in (1, 16, 32, 256):
             xm = [torch.randn(m, kk, generator=gen(90 + m)).to(torch.float16).to(dev) for _ in range(2)]
             t = time_graph(lambda i: kernels.q_linear(xm[i % 2], blobs[i], sc, 4, 32), rot, steps_s, 2, dev)
             algq = nn_ * kk // 2 + nn_ * kk // 32 * 2 + m * kk * 2 + m * nn_ * 2
-            add("cfg5 int4 14336x4096 f16", "a:gemv" if m <= 16 else "b:tile-gemm", m, t, algq, 2.0 * m * nn_ * kk)
+            add("cfg5 int4 14336x4096 f16", "a:gemv" if m <= 32 else "b:tile-gemm", m, t, algq, 2.0 * m * nn_ * kk)
         del blobs
         torch.cuda.empty_cache()
         # neighbours of the linear on a decode step: RMSNorm and the embedding lookups (Llama-3-8B sizes)
