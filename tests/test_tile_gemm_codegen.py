@@ -1,0 +1,66 @@
+"""What the tile GEMM's relaxed step barrier relies on, checked in the generated code.
+
+A producer wave of ``tile_gemm_kernel`` with the codebook in LDS ends a step with
+``s_waitcnt lgkmcnt(N); s_barrier`` where N is the number of codebook lookups it issued after its two
+stores into the W tile (``block_sync_lds_keep`` in ``csrc/gemm_tile.hpp``).  LDS operations of a wave
+complete in order, so the stores are done when at most N operations are outstanding -- provided the
+compiler kept the stores in front of the lookups, issued no other LDS operation behind them, and has
+no scalar or flat load in flight whose return would be counted out of order.  The source pins that
+order with a compiler barrier; this test compiles the VQ tile GEMM for gfx950 (device code only, no
+GPU needed, about a minute) and reads the order off the assembly of every instantiation.
+"""
+
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from neuropress_amd import build
+
+
+def _assembly(tmp_path):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    out = tmp_path / "vq_gemm.s"
+    cmd = [hipcc, *build.CXXFLAGS, *build.DEVICE_FLAGS, "-S", "--cuda-device-only",
+           str(build.CSRC / "vq_gemm.hip"), "-o", str(out)]  # fmt: skip
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    return out.read_text().split("\n")
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not build.Path("/opt/rocm/bin/hipcc").exists(),
+                    reason="needs hipcc")  # fmt: skip
+def test_relaxed_step_barriers_follow_stores_then_lookups(tmp_path):
+    lines = _assembly(tmp_path)
+    starts = [i for i, ln in enumerate(lines) if re.match(r"^_ZN5npamd16tile_gemm_kernel\S*: ;", ln)]
+    assert len(starts) >= 100  # every (activation, width, vector length, tokens band, LDS) instantiation
+    kernels_with_relaxed, relaxed = 0, 0
+    for i in starts:
+        name = lines[i].split(":")[0]
+        end = next(j for j in range(i, len(lines)) if lines[j].startswith(".Lfunc_end"))
+        body = lines[i:end]
+        found = 0
+        for k, ln in enumerate(body[:-1]):
+            m = re.search(r"s_waitcnt lgkmcnt\((\d+)\)", ln)
+            if not (m and int(m.group(1)) > 0 and "s_barrier" in body[k + 1]):
+                continue
+            keep = int(m.group(1))
+            ops = []
+            j = k - 1
+            while j >= 0 and "s_barrier" not in body[j]:
+                op = re.match(r"\s+(ds_\w+|s_load\w+|s_buffer_load\w+|flat_\w+)", body[j])
+                if op:
+                    ops.append(op.group(1))
+                j -= 1
+            ops.reverse()
+            assert not [o for o in ops if not o.startswith("ds_")], (name, ops)  # nothing counted out of order
+            assert len(ops) > keep and all(o.startswith("ds_read") for o in ops[-keep:]), (name, ops)
+            assert all(o.startswith("ds_write") for o in ops[:-keep]), (name, ops)  # the stores, and only them, in front
+            found += 1
+        if found:
+            # the LDS-codebook variant (last template argument true), eight unrolled steps
+            assert name.endswith("ELb1EEEvNS_9GemmShapeENT0_4ArgsE") and found == 8, (name, found)
+            kernels_with_relaxed += 1
+            relaxed += found
+    assert kernels_with_relaxed >= 40 and relaxed == 8 * kernels_with_relaxed
