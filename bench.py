@@ -44,7 +44,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
-    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_tile_m128",
+    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "tile_m384", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_tile_m128",
                                                     "rms_norm_m4096", "vq_embedding_m4096", "q4_embedding_m4096"],
                     help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
                          "on the config-3 / config-5 shape and print a one-line JSON with its HIP-event time")
@@ -183,14 +183,14 @@ def main():
                 base = IndexPacking.pack(torch.randint(0, nc, (n * k // 8,), generator=g), bits)
             pool = [base.to(dev).clone() for _ in range(n_rot)]
             cb16, cbb = cb.to(dev), cb.to(torch.bfloat16).to(dev)
-            m = 256 if args.case == "tile_m256" else 128 if args.case == "tile_nc4096_m128" else 1
+            m = 256 if args.case == "tile_m256" else 384 if args.case == "tile_m384" else 128 if args.case == "tile_nc4096_m128" else 1
             x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
             if args.case == "sliced_m1":
                 sl0 = kernels.vq_slice_indices(base, bits, n, k, 8, nc, device=dev)
                 spool = [sl0] + [kernels.SlicedIndices(sl0.blob.clone(), sl0.header) for _ in range(n_rot - 1)]
                 ws = torch.empty(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
                 fn = lambda i: kernels.vq_linear_sliced(x, spool[i], cbb, None, workspace=ws)
-            elif args.case in ("tile_m256", "tile_nc4096_m128"):
+            elif args.case in ("tile_m256", "tile_m384", "tile_nc4096_m128"):
                 fn = lambda i: kernels.vq_gemm_tile(x, pool[i], cbb, bits, n, None)
             elif args.case == "dequant":
                 fn = lambda i: kernels.vq_dequant(pool[i], cb16, bits, n, k, torch.bfloat16)
@@ -300,6 +300,27 @@ def main():
         },
         "checks": {"decode_bit_exact": decode_exact, "output_within_1e-2": ok, "max_abs_err": max_abs},
     }
+
+    # The second half of the metric: the tile-decode GEMM at M = 384 on the same layer, priced against the
+    # dense bf16 MFMA peak.  Timed here so that the line carries it with --no-sweep too.
+    m2 = 384
+    xm2 = [torch.randn(m2, k, generator=gen(60 + m2)).to(torch.bfloat16).to(dev) for _ in range(2)]
+    us_tile = time_graph(lambda i: kernels.vq_gemm_tile(xm2[i % 2], c3["pool"][i], c3["d_cb_act"], 16, n, None),
+                         n_rot, max(10, args.steps // 10), 2, dev)
+    flops2 = 2.0 * m2 * n * k
+    y2 = kernels.vq_gemm_tile(xm2[0], c3["pool"][0], c3["d_cb_act"], 16, n, None)
+    ok2, max_abs2 = check_against_cpu(y2, (xm2[0].float() @ w_gpu.float().T).cpu())
+    result["roofline_m384"] = {
+        "bound": "mfma", "achieved": round(flops2 / us_tile / 1e6, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(flops2 / us_tile / 1e6 / MFMA_PEAK_TFLOPS, 4),
+        # FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch, profiles/vq_tile_gemm_cfg3_14336x4096_m384.md
+        "traffic": 60422 * 1024 * 2 + 11670 * 1024,
+        "kernel": "tile_gemm_kernel<bf16, VqProvider<bf16,16>, MW=3>", "flops_per_launch": flops2,
+        "avg_launch_us": round(us_tile, 3), "M": m2, "output_within_1e-2": ok2, "max_abs_err": max_abs2,
+        "note": "same layer and codebook as `roofline`, 384 tokens, one launch decodes every weight once and "
+                "contracts it with MFMA 32x32x16; HIP-graph replay over the rotating index pool",
+    }
+    del xm2, y2
 
     # ---------------- sweep over the other bands / configs ----------------------
     sweep = []
