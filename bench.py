@@ -205,7 +205,7 @@ def main():
             if args.case == "sliced_m1":
                 sl0 = kernels.vq_slice_indices(base, bits, n, k, 8, nc, device=dev)
                 spool = [sl0] + [kernels.SlicedIndices(sl0.blob.clone(), sl0.header) for _ in range(n_rot - 1)]
-                ws = torch.empty(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
+                ws = torch.zeros(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
                 fn = lambda i: kernels.vq_linear_sliced(x, spool[i], cbb, None, workspace=ws)
             elif args.case in ("tile_m256", "tile_m384", "tile_nc4096_m128"):
                 fn = lambda i: kernels.vq_gemm_tile(x, pool[i], cbb, bits, n, None)
@@ -262,16 +262,13 @@ def main():
     sl0 = kernels.vq_slice_indices(c3["packed"], 16, n, k, 8, 65536, device=dev)
     s_rot = max(2, POOL_BYTES // sl0.total_bytes)
     spool = [sl0] + [kernels.SlicedIndices(sl0.blob.clone(), sl0.header) for _ in range(s_rot - 1)]
-    ws = torch.empty(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
+    ws = torch.zeros(sl0.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
 
     def step(i):
         ys[i % n_rot] = kernels.vq_linear_sliced(xs[i % n_rot], spool[i], c3["d_cb_act"], None, workspace=ws)
 
     us = time_graph(step, s_rot, args.steps, args.warmup, dev)
-    # The dominant kernel alone (sliced_gemv_kernel, partial sums only), for the roofline line.
-    us_main = time_graph(lambda i: kernels.vq_linear_sliced(xs[i % n_rot], spool[i], c3["d_cb_act"], None,
-                                                            workspace=ws, partials_only=True),
-                         s_rot, args.steps, args.warmup, dev)
+    us_main = us  # one kernel per call: the finish is part of sliced_gemv_kernel
     alg = vq_alg_bytes(c3, 1)
     gbs = alg / us / 1e3
     gbs_main = alg / us_main / 1e3
@@ -350,7 +347,7 @@ def main():
         steps_s = max(10, args.steps // 10)
         for m in (2, 4, 7):
             xm2 = [torch.randn(m, k, generator=gen(50 + m)).to(torch.bfloat16).to(dev) for _ in range(2)]
-            ws2 = torch.empty(sl0.workspace_bytes(m) // 4, device=dev, dtype=torch.float32)
+            ws2 = torch.zeros(sl0.workspace_bytes(m) // 4, device=dev, dtype=torch.float32)
             t = time_graph(lambda i: kernels.vq_linear_sliced(xm2[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2),
                            s_rot, steps_s * 2, 3, dev)
             add("cfg3 14336x4096 bf16", "a:sliced-gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
@@ -376,7 +373,7 @@ def main():
         c3d = vq_case(dev, 1003, 4096, 14336, 65536, 16, torch.bfloat16, n_rot)
         sld = kernels.vq_slice_indices(c3d["packed"], 16, 4096, 14336, 8, 65536, device=dev)
         sdpool = [sld] + [kernels.SlicedIndices(sld.blob.clone(), sld.header) for _ in range(s_rot - 1)]
-        wsd = torch.empty(sld.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
+        wsd = torch.zeros(sld.workspace_bytes(1) // 4, device=dev, dtype=torch.float32)
         xd = torch.randn(1, 14336, generator=gen(71)).to(torch.bfloat16).to(dev)
         t = time_graph(lambda i: kernels.vq_linear_sliced(xd, sdpool[i], c3d["d_cb_act"], None, workspace=wsd),
                        s_rot, steps_s * 2, 3, dev)

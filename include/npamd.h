@@ -154,12 +154,12 @@ typedef struct npamd_sliced_header {
   int32_t n_workgroups;   /* grid size of the GEMV */
   int32_t n_partials;     /* partial-sum vectors per output row */
   int32_t groups_max;     /* largest group range of a workgroup */
-  int32_t reserved32;
-  int64_t n_quads;        /* 768-byte entry quads */
+  uint32_t flags;         /* bit 0: workgroup w works on codebook slice w % n_slices */
+  int64_t n_quads;        /* 768-byte entry quads = n_workgroups * (sum of wave_quads) */
   int64_t n_entries;      /* real (non-padding) entries = N * K / VL */
   int64_t off_workgroups, off_rowmap, off_entries;
   int64_t total_bytes;
-  int64_t reserved[4];
+  uint16_t wave_quads[16]; /* entry quads of wave w's strip, the same in every workgroup */
 } npamd_sliced_header;
 
 /*
@@ -181,7 +181,7 @@ int npamd_vq_sliced_build(const uint8_t* packed_host, int64_t n_bytes, int bits,
  */
 int npamd_vq_sliced_check(const void* blob_host, int64_t blob_bytes);
 
-/* Bytes of f32 workspace npamd_vq_gemv_sliced needs for M tokens. */
+/* Bytes of workspace npamd_vq_gemv_sliced needs for M tokens (zero-filled by the caller once). */
 int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, int M);
 
 /*
@@ -191,9 +191,16 @@ int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, 
  * `header_host` is a host copy of the blob's header, `blob` the whole blob in
  * device memory.  The codebook must be in the activation dtype.  `workspace`
  * is device memory of npamd_vq_sliced_workspace_bytes() bytes, 16-byte aligned,
- * contents irrelevant before the call; afterwards it holds, per token, the
- * n_partials partial-sum vectors [n_partials][N] (f32) whose sum over the first
- * axis is the un-biased result.  With y == NULL only those are produced.
+ * ZERO-FILLED before its first use; every call hands it back zero-filled, so calls
+ * that follow each other on one stream may share it (calls that overlap must not).
+ * A row's result is spread over the workgroups that hold the codebook slices its
+ * indices point into.  With fewer than 256 of them per row (any codebook of up to
+ * 2^16 rows) every lane adds its partial sum, as a fixed-point number in units of
+ * 2^-24, to a 64-bit word of the workspace with one atomic; the lane that completes
+ * a row's count adds the bias, rounds once and stores y -- one kernel, and the sum
+ * does not depend on the order of arrival (partial sums of magnitude 2^15 or more go
+ * through a float accumulator).  Otherwise the partial sums are written out and a
+ * second kernel adds them in a fixed order.
  * `column_perm`: NULL, or K int32 column numbers (16-byte aligned, each < ldx):
  * the kernel then reads x[m, column_perm[k]] wherever it would read x[m, k],
  * i.e. the x[..., column_perm] the reference applies before every VQ matmul

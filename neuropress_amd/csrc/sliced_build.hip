@@ -53,45 +53,67 @@ inline uint32_t host_read_index(const uint8_t* packed, int64_t n_bytes, int64_t 
   return (uint32_t)((w >> off) & ((1u << bits) - 1u));
 }
 
-// Entry j of a lane's 12-byte quad record: row = bytes 2j, 2j+1 (little endian), group = byte 8 + j.
+// Entry j of a lane's 12-byte quad record: bytes 2j, 2j+1 (little endian) hold the row in bits 0-12
+// and bit 8 of the group in bit 15, byte 8 + j the group's low eight bits.
 // In memory an entry is handled as row | group << 16.
 inline void put_entry(uint8_t* quad_lane, int j, uint32_t e) {
-  quad_lane[2 * j + 0] = (uint8_t)(e & 0xFF);
-  quad_lane[2 * j + 1] = (uint8_t)((e >> 8) & 0xFF);
-  quad_lane[8 + j] = (uint8_t)((e >> 16) & 0xFF);
+  const uint32_t row = e & 0x1FFFu, g = e >> 16;
+  const uint32_t field = row | ((g >> 8) << 15);
+  quad_lane[2 * j + 0] = (uint8_t)(field & 0xFF);
+  quad_lane[2 * j + 1] = (uint8_t)(field >> 8);
+  quad_lane[8 + j] = (uint8_t)(g & 0xFF);
 }
 
 inline uint32_t get_entry(const uint8_t* quad_lane, int j) {
-  return (uint32_t)quad_lane[2 * j] | ((uint32_t)quad_lane[2 * j + 1] << 8) | ((uint32_t)quad_lane[8 + j] << 16);
+  const uint32_t field = (uint32_t)quad_lane[2 * j] | ((uint32_t)quad_lane[2 * j + 1] << 8);
+  const uint32_t g = (uint32_t)quad_lane[8 + j] | ((field >> 15) << 8);
+  return (field & 0x1FFFu) | (g << 16);
 }
 
 // Order the entries of the 64 tasks of a strip so that, step by step, the LDS reads of a
-// wave collide as little as possible.  A 64-lane 16-byte LDS read is served in two halves of 32
-// lanes; a half takes as many cycles as its fullest 16-byte bank group holds distinct addresses
-// ((address / 16) % 16, two being free) -- measured: 2.2 ns conflict-free, 3.6 ns with four
-// addresses per group, 13.4 ns with sixteen.  Random rows give about five per group.  A lane may
-// sum its entries in any order, so for every step each lane takes, among its remaining
-// entries, the one whose activation vector (group % 16; shared vectors count once) and codebook
-// row (row % 16) fall into the emptiest groups of its half.
+// wave collide as little as possible.  A 64-lane 16-byte LDS read (ds_read_b128) is served
+// in four passes of 16 lanes -- lanes {0-3, 12-15, 20-27}, {4-11, 16-19, 28-31} and the same
+// two sets 32 lanes further on (found by timing reads in which exactly two lanes share a bank
+// group) -- and a pass takes one cycle per distinct address of its fullest 16-byte bank
+// group ((address / 16) % 16): 4.3 cycles per read when every pass has its 16 lanes in 16
+// different groups, one more for every further address in a group.  Random rows put about three
+// addresses into the fullest group of a pass.  A lane may sum its entries in any order, so
+// for every step each lane takes, among its remaining entries, the one whose activation
+// vector (group % 16; a vector already read in the pass costs nothing) and codebook row
+// (row % 16) fall into the emptiest bank groups of its pass.
+inline int lds_pass_of_lane(int lane) {
+  const int l = lane & 31;
+  const bool first = l < 4 || (l >= 12 && l < 16) || (l >= 20 && l < 28);
+  return (lane >> 5) * 2 + (first ? 0 : 1);
+}
+
 void spread_bank_groups(std::vector<uint32_t>* const* tasks, int lanes, int64_t steps) {
-  constexpr int kXWeight = 2;  // the activation read is repeated per token
+  constexpr int kXWeight = 1;
+  int pass_lanes[4][16], pass_count[4] = {0, 0, 0, 0};
+  for (int lane = 0; lane < lanes; ++lane) {
+    const int p = lds_pass_of_lane(lane);
+    pass_lanes[p][pass_count[p]++] = lane;
+  }
   for (int64_t t = 0; t < steps; ++t) {
-    for (int half = 0; half < 2; ++half) {
+    for (int p = 0; p < 4; ++p) {
       int g_count[16] = {0}, r_count[16] = {0};
       uint8_t g_seen[kSlicedMaxGroups] = {0};
-      for (int lane = half * 32; lane < std::min(lanes, half * 32 + 32); ++lane) {
-        std::vector<uint32_t>& e = *tasks[lane];
+      // Lanes with the fewest entries left choose first: they have the least freedom.
+      int order[16];
+      for (int i = 0; i < pass_count[p]; ++i) order[i] = pass_lanes[p][i];
+      std::stable_sort(order, order + pass_count[p], [&](int a, int b) { return tasks[a]->size() < tasks[b]->size(); });
+      for (int i = 0; i < pass_count[p]; ++i) {
+        std::vector<uint32_t>& e = *tasks[order[i]];
         if ((int64_t)e.size() <= t) continue;
         size_t best = (size_t)t;
         int best_cost = 1 << 30;
-        for (size_t i = (size_t)t; i < e.size(); ++i) {
-          const uint32_t row = e[i] & 0xFFFFu, g = e[i] >> 16;
-          const int gc = g_seen[g] ? 0 : std::max(0, g_count[g & 15] - 1);
-          const int rc = std::max(0, r_count[row & 15] - 1);
-          const int cost = kXWeight * gc + rc;
+        for (size_t j = (size_t)t; j < e.size(); ++j) {
+          const uint32_t row = e[j] & 0xFFFFu, g = e[j] >> 16;
+          const int gc = g_seen[g] ? 0 : g_count[g & 15];
+          const int cost = kXWeight * gc + r_count[row & 15];
           if (cost < best_cost) {
             best_cost = cost;
-            best = i;
+            best = j;
             if (cost == 0) break;
           }
         }
@@ -220,7 +242,9 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
       for (int s = 0; s < S; ++s) slice_count[(size_t)s] += c[(size_t)s];
   }
 
-  const Geometry geo = plan_geometry(N, G, slice_count, n_idx, target_workgroups);
+  Geometry geo = plan_geometry(N, G, slice_count, n_idx, target_workgroups);
+  // Group ranges have a fixed length per slice, ceil(G / parts); no range may come out empty.
+  for (int& parts : geo.parts) parts = (G + (G + parts - 1) / parts - 1) / ((G + parts - 1) / parts);
   std::vector<int> partial_base((size_t)S);
   int n_partials = 0;
   for (int s = 0; s < S; ++s) {
@@ -248,33 +272,39 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   }
   const int n_wg = (int)jobs.size();
 
-  // Every workgroup is built on its own (quad numbers local to the workgroup), then the entry
-  // sections are concatenated in workgroup order.
+  // Pass 1, one workgroup at a time: the tasks in strip and lane order.  Pass 2 writes them at
+  // the places the layer-wide strip lengths fix.
+  struct Built {
+    std::vector<uint32_t> entries;  // the tasks' entries, one task after the other in lane order
+    uint32_t begin[kSlicedTasks + 1];
+    int steps[kSlicedWaves];        // longest task of each strip
+    int64_t real_entries;
+  };
   std::vector<SlicedWorkgroup> wgs((size_t)n_wg);
   std::vector<uint32_t> rowmap((size_t)n_wg * kSlicedTasks, kSlicedNoRow);
-  std::vector<std::vector<uint8_t>> wg_quads((size_t)n_wg);
-  std::vector<int64_t> wg_entries((size_t)n_wg, 0);
+  std::vector<Built> built((size_t)n_wg);
 
   const char* spread_env = getenv("NPAMD_SLICED_SPREAD");
   const bool spread = !(spread_env && *spread_env == '0');
   parallel_for(n_wg, [&](int w) {
     std::vector<std::vector<uint32_t>> task((size_t)geo.rows_per_block);
     std::vector<int> order;
-    std::vector<uint8_t>& quads = wg_quads[(size_t)w];
-    int64_t real_entries = 0;
+    Built& b = built[(size_t)w];
     const Job& job = jobs[w];
     SlicedWorkgroup& wg = wgs[w];
-    memset(&wg, 0, sizeof(wg));
-    const int g_begin = (int)((int64_t)G * job.part / geo.parts[job.slice]);
-    const int g_end = (int)((int64_t)G * (job.part + 1) / geo.parts[job.slice]);
+    const int range_groups = (G + geo.parts[job.slice] - 1) / geo.parts[job.slice];
+    const int g_begin = job.part * range_groups;
+    const int g_end = std::min(G, g_begin + range_groups);
     const int row0 = job.block * geo.rows_per_block;
     const int rows = std::max(0, std::min(geo.rows_per_block, N - row0));
     wg.slice = (uint32_t)job.slice;
     wg.partial = (uint32_t)(partial_base[job.slice] + job.part);
     wg.g_begin = (uint32_t)g_begin;
     wg.g_count = (uint32_t)(g_end - g_begin);
+    wg.row_begin = (uint32_t)std::min(row0, N);
+    wg.row_count = (uint32_t)rows;
+    wg.reserved[0] = wg.reserved[1] = 0;
 
-    for (int r = 0; r < rows; ++r) task[(size_t)r].clear();
     for (int g = g_begin; g < g_end; ++g) {
       const uint32_t* col = &idx_t[(size_t)g * N + row0];
       for (int r = 0; r < rows; ++r) {
@@ -287,57 +317,49 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
     order.resize((size_t)rows);
     std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(),
-                     [&](int a, int b) { return task[(size_t)a].size() > task[(size_t)b].size(); });
-    const uint32_t pad = (uint32_t)kSlicedPadRow;  // the zero row, group 0
-    for (int s = 0; s * 64 < rows; ++s) {
+                     [&](int a, int c) { return task[(size_t)a].size() > task[(size_t)c].size(); });
+    b.real_entries = 0;
+    for (int s = 0; s < kSlicedWaves; ++s) {
       const int first = s * 64;
-      const int lanes = std::min(64, rows - first);
-      const int64_t steps = (int64_t)task[(size_t)order[(size_t)first]].size();
-      const int64_t nq = (steps + 3) / 4;
-      if (spread) {
+      const int lanes = std::max(0, std::min(64, rows - first));
+      b.steps[s] = lanes ? (int)task[(size_t)order[(size_t)first]].size() : 0;
+      if (spread && lanes) {
         std::vector<uint32_t>* strip_tasks[64];
         for (int lane = 0; lane < lanes; ++lane) strip_tasks[lane] = &task[(size_t)order[(size_t)(first + lane)]];
-        spread_bank_groups(strip_tasks, lanes, steps);
+        spread_bank_groups(strip_tasks, lanes, b.steps[s]);
       }
-      wg.wave[s].quad_begin = nq ? (uint32_t)(quads.size() / kSlicedQuadBytes) : 0u;
-      wg.wave[s].steps = (uint32_t)steps;
-      const size_t base = quads.size();
-      quads.resize(base + (size_t)nq * kSlicedQuadBytes);
       for (int lane = 0; lane < 64; ++lane) {
-        const std::vector<uint32_t>* t = nullptr;
-        if (lane < lanes) {
-          const int r = order[(size_t)(first + lane)];
-          t = &task[(size_t)r];
-          rowmap[(size_t)w * kSlicedTasks + (size_t)s * 64 + lane] = (uint32_t)(row0 + r);
-          real_entries += (int64_t)t->size();
-        }
-        for (int64_t i = 0; i < nq * 4; ++i) {
-          const uint32_t e = (t && i < (int64_t)t->size()) ? (*t)[(size_t)i] : pad;
-          put_entry(&quads[base + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12], (int)(i % 4), e);
-        }
+        b.begin[first + lane] = (uint32_t)b.entries.size();
+        if (lane >= lanes) continue;
+        const int r = order[(size_t)(first + lane)];
+        rowmap[(size_t)w * kSlicedTasks + (size_t)first + lane] = (uint32_t)(row0 + r);
+        b.entries.insert(b.entries.end(), task[(size_t)r].begin(), task[(size_t)r].end());
       }
     }
-    wg_entries[(size_t)w] = real_entries;
+    b.begin[kSlicedTasks] = (uint32_t)b.entries.size();
+    b.real_entries = (int64_t)b.entries.size();
   });
 
-  std::vector<uint8_t> quads;
+  // Strip w of every workgroup gets the length of the layer's longest strip w.
+  uint16_t wave_quads[kSlicedWaves];
+  int64_t wave_begin[kSlicedWaves + 1];
   int64_t real_entries = 0;
   int groups_max = 1;
-  {
-    size_t total = 0;
-    for (auto& q : wg_quads) total += q.size();
-    quads.reserve(std::max<size_t>(total, kSlicedQuadBytes));
-    for (int w = 0; w < n_wg; ++w) {
-      const uint32_t base = (uint32_t)(quads.size() / kSlicedQuadBytes);
-      for (int s = 0; s < kSlicedWaves; ++s)
-        if (wgs[(size_t)w].wave[s].steps) wgs[(size_t)w].wave[s].quad_begin += base;
-      quads.insert(quads.end(), wg_quads[(size_t)w].begin(), wg_quads[(size_t)w].end());
-      std::vector<uint8_t>().swap(wg_quads[(size_t)w]);
-      real_entries += wg_entries[(size_t)w];
-      groups_max = std::max(groups_max, (int)wgs[(size_t)w].g_count);
-    }
+  wave_begin[0] = 0;
+  for (int s = 0; s < kSlicedWaves; ++s) {
+    int longest = 0;
+    for (int w = 0; w < n_wg; ++w) longest = std::max(longest, built[(size_t)w].steps[s]);
+    NPAMD_REQUIRE((longest + 3) / 4 <= 65535, "%s: a row has %d indices in one slice and group range", what, longest);
+    wave_quads[s] = (uint16_t)((longest + 3) / 4);
+    wave_begin[s + 1] = wave_begin[s] + wave_quads[s];
   }
-  if (quads.empty()) quads.resize(kSlicedQuadBytes, 0);  // waves without a strip still load quad 0
+  const int64_t wg_quads = std::max<int64_t>(wave_begin[kSlicedWaves], 1);  // never an empty entry section
+  for (int w = 0; w < n_wg; ++w) {
+    real_entries += built[(size_t)w].real_entries;
+    groups_max = std::max(groups_max, (int)wgs[(size_t)w].g_count);
+  }
+  bool round_robin = true;
+  for (int s = 0; s < S; ++s) round_robin = round_robin && geo.parts[(size_t)s] == geo.parts[0];
 
   npamd_sliced_header h;
   memset(&h, 0, sizeof(h));
@@ -349,22 +371,42 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   h.n_workgroups = n_wg;
   h.n_partials = n_partials;
   h.groups_max = groups_max;
-  h.n_quads = (int64_t)(quads.size() / kSlicedQuadBytes);
+  h.flags = round_robin ? kSlicedRoundRobin : 0u;
+  h.n_quads = (int64_t)n_wg * wg_quads;
   h.n_entries = real_entries;
+  memcpy(h.wave_quads, wave_quads, sizeof(wave_quads));
   h.off_workgroups = sizeof(h);
   h.off_rowmap = align_up(h.off_workgroups + (int64_t)n_wg * (int64_t)sizeof(SlicedWorkgroup), 256);
   h.off_entries = align_up(h.off_rowmap + (int64_t)rowmap.size() * 4, 256);
-  h.total_bytes = align_up(h.off_entries + (int64_t)quads.size(), 256);
+  h.total_bytes = align_up(h.off_entries + h.n_quads * kSlicedQuadBytes, 256);
   *blob_bytes = h.total_bytes;
   if (blob == nullptr) return NPAMD_OK;
   NPAMD_REQUIRE(capacity >= h.total_bytes, "%s: buffer of %lld bytes, %lld needed", what,
                 (long long)capacity, (long long)h.total_bytes);
   uint8_t* out = (uint8_t*)blob;
-  memset(out, 0, (size_t)h.total_bytes);
+  memset(out, 0, (size_t)h.off_entries);
   memcpy(out, &h, sizeof(h));
   memcpy(out + h.off_workgroups, wgs.data(), wgs.size() * sizeof(SlicedWorkgroup));
   memcpy(out + h.off_rowmap, rowmap.data(), rowmap.size() * 4);
-  memcpy(out + h.off_entries, quads.data(), quads.size());
+  memset(out + h.off_entries + h.n_quads * kSlicedQuadBytes, 0,
+         (size_t)(h.total_bytes - h.off_entries - h.n_quads * kSlicedQuadBytes));
+  // Pass 2: every lane's entries, padded to the strip's length with the zero row (group 0).
+  const uint32_t pad = (uint32_t)kSlicedPadRow;
+  parallel_for(n_wg, [&](int w) {
+    const Built& b = built[(size_t)w];
+    uint8_t* wg_out = out + h.off_entries + (int64_t)w * wg_quads * kSlicedQuadBytes;
+    if (wave_begin[kSlicedWaves] == 0) memset(wg_out, 0, kSlicedQuadBytes);  // the one quad of an entry-less layer
+    for (int s = 0; s < kSlicedWaves; ++s) {
+      uint8_t* strip = wg_out + wave_begin[s] * kSlicedQuadBytes;
+      const int64_t slots = 4 * (int64_t)wave_quads[s];
+      for (int lane = 0; lane < 64; ++lane) {
+        const uint32_t* e = b.entries.data() + b.begin[s * 64 + lane];
+        const int64_t len = (int64_t)b.begin[s * 64 + lane + 1] - (int64_t)b.begin[s * 64 + lane];
+        for (int64_t i = 0; i < slots; ++i)
+          put_entry(strip + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4), i < len ? e[i] : pad);
+      }
+    }
+  });
   return NPAMD_OK;
 }
 
@@ -382,12 +424,18 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
                 "%s: bad slice geometry", what);
   NPAMD_REQUIRE(h.groups_max >= 1 && h.groups_max <= kSlicedMaxGroups, "%s: group range %d too long", what, h.groups_max);
   NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1 && h.n_quads >= 1, "%s: bad counts", what);
+  int64_t wave_begin[kSlicedWaves + 1];
+  wave_begin[0] = 0;
+  for (int s = 0; s < kSlicedWaves; ++s) wave_begin[s + 1] = wave_begin[s] + h.wave_quads[s];
+  const int64_t wg_quads = std::max<int64_t>(wave_begin[kSlicedWaves], 1);
+  NPAMD_REQUIRE(h.n_quads == (int64_t)h.n_workgroups * wg_quads, "%s: entry section does not match the strip lengths", what);
+  NPAMD_REQUIRE((h.flags & ~kSlicedRoundRobin) == 0, "%s: unknown flags", what);
   const int64_t end_wg = h.off_workgroups + (int64_t)h.n_workgroups * (int64_t)sizeof(SlicedWorkgroup);
   const int64_t end_rm = h.off_rowmap + (int64_t)h.n_workgroups * kSlicedTasks * 4;
   const int64_t end_en = h.off_entries + h.n_quads * kSlicedQuadBytes;
   NPAMD_REQUIRE(h.off_workgroups >= (int64_t)sizeof(h) && end_wg <= h.off_rowmap && end_rm <= h.off_entries &&
                     end_en <= h.total_bytes && h.off_entries % 16 == 0 && h.off_rowmap % 4 == 0 &&
-                    h.off_workgroups % 4 == 0,
+                    h.off_workgroups % 16 == 0,
                 "%s: section offsets out of order or outside the blob", what);
   const uint8_t* base = (const uint8_t*)blob;
   const SlicedWorkgroup* wgs = (const SlicedWorkgroup*)(base + h.off_workgroups);
@@ -400,29 +448,49 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
     const SlicedWorkgroup& wg = wgs[w];
     NPAMD_REQUIRE(wg.slice < (uint32_t)h.n_slices && wg.partial < (uint32_t)h.n_partials,
                   "%s: workgroup %d: slice/partial out of range", what, w);
+    if (h.flags & kSlicedRoundRobin) {
+      // What the kernel computes instead of reading the record.
+      const int parts = h.n_partials / h.n_slices;
+      const int row_blocks = parts ? h.n_workgroups / (parts * h.n_slices) : 0;
+      NPAMD_REQUIRE(parts >= 1 && row_blocks >= 1 && parts * h.n_slices == h.n_partials &&
+                        row_blocks * h.n_partials == h.n_workgroups,
+                    "%s: counts do not form the regular geometry the header states", what);
+      const int range_groups = (G + parts - 1) / parts;
+      const int rows_per_block = (h.n + row_blocks - 1) / row_blocks;
+      const uint32_t part = (uint32_t)((w / h.n_slices) / row_blocks);
+      const int block = (w / h.n_slices) % row_blocks;
+      const int row_begin = std::min(block * rows_per_block, h.n);
+      NPAMD_REQUIRE(wg.slice == (uint32_t)(w % h.n_slices) && wg.partial == wg.slice * (uint32_t)parts + part &&
+                        wg.g_begin == part * (uint32_t)range_groups &&
+                        wg.g_count == (uint32_t)std::min(range_groups, G - (int)wg.g_begin) &&
+                        wg.row_begin == (uint32_t)row_begin &&
+                        wg.row_count == (uint32_t)std::max(0, std::min(rows_per_block, h.n - row_begin)),
+                    "%s: workgroup %d does not follow the regular geometry the header states", what, w);
+    }
     NPAMD_REQUIRE(wg.g_count >= 1 && wg.g_count <= (uint32_t)h.groups_max && (int64_t)wg.g_begin + wg.g_count <= G,
                   "%s: workgroup %d: group range out of bounds", what, w);
+    NPAMD_REQUIRE(wg.row_count <= (uint32_t)kSlicedTasks && (int64_t)wg.row_begin + wg.row_count <= h.n,
+                  "%s: workgroup %d: row block out of bounds", what, w);
     const uint32_t slice_len = (uint32_t)std::min(h.slice_rows, h.nc - (int)wg.slice * h.slice_rows);
     for (int s = 0; s < kSlicedWaves; ++s) {
-      const SlicedWave& wave = wg.wave[s];
-      const int64_t nq = ((int64_t)wave.steps + 3) / 4;
-      NPAMD_REQUIRE((int64_t)wave.quad_begin + std::max<int64_t>(nq, 1) <= h.n_quads,
-                    "%s: workgroup %d wave %d: entries out of bounds", what, w, s);
+      const int64_t nq = h.wave_quads[s];
+      const int64_t quad_begin = (int64_t)w * wg_quads + wave_begin[s];
       for (int lane = 0; lane < 64; ++lane) {
         const uint32_t row = rowmap[(size_t)w * kSlicedTasks + (size_t)s * 64 + lane];
-        NPAMD_REQUIRE(row == kSlicedNoRow || row < (uint32_t)h.n, "%s: workgroup %d: row out of range", what, w);
+        NPAMD_REQUIRE(row == kSlicedNoRow || (row >= wg.row_begin && row - wg.row_begin < wg.row_count),
+                      "%s: workgroup %d: row outside the workgroup's row block", what, w);
         if (row != kSlicedNoRow) {
           uint8_t& c = covered[(size_t)wg.partial * h.n + row];
           NPAMD_REQUIRE(c == 0, "%s: partial %u row %u written twice", what, wg.partial, row);
           c = 1;
         }
         for (int64_t i = 0; i < nq * 4; ++i) {
-          const uint32_t e = get_entry(quads + ((size_t)wave.quad_begin + (size_t)(i / 4)) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4));
+          const uint32_t e = get_entry(quads + ((size_t)quad_begin + (size_t)(i / 4)) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4));
           const uint32_t local = e & 0xFFFFu, g_local = e >> 16;
           NPAMD_REQUIRE(g_local < wg.g_count && (local < slice_len || local == (uint32_t)kSlicedPadRow),
                         "%s: workgroup %d: entry field out of range", what, w);
           if (local != (uint32_t)kSlicedPadRow) {
-            NPAMD_REQUIRE(row != kSlicedNoRow && i < (int64_t)wave.steps, "%s: workgroup %d: live entry in a lane without a row", what, w);
+            NPAMD_REQUIRE(row != kSlicedNoRow, "%s: workgroup %d: live entry in a lane without a row", what, w);
             uint8_t& f = filed[(size_t)row * G + wg.g_begin + g_local];
             NPAMD_REQUIRE(f == 0, "%s: index (%u, %u) filed twice", what, row, wg.g_begin + g_local);
             f = 1;
@@ -439,5 +507,7 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
 
 extern "C" int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* h, int M) {
   if (h == nullptr || M < 1) return 0;
+  // Fewer than 256 partial sums per row: a 64-bit word and a float per (token, row).
+  if (h->n_partials < 256) return (int64_t)h->n * 12 * (int64_t)M;
   return (int64_t)h->n_partials * (int64_t)h->n * 4 * (int64_t)M;
 }

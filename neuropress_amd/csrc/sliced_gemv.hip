@@ -1,7 +1,7 @@
 // Decode GEMV over the slice-list form of the indices (see sliced_format.hpp).
 //
-// One workgroup of 16 waves holds the activations of its group range (up to 4 KiB
-// per token, up to seven tokens per launch), one 8192-row codebook slice (128 KiB)
+// One workgroup of 16 waves holds the activations of its group range (up to 8 KiB
+// per token, up to seven tokens per launch), one 4096-row codebook slice (64 KiB)
 // and a zero row in LDS.  Every lane owns one output row and
 // walks the entries filed under (slice, group range, row): two 16-byte LDS reads
 // (codebook row, activation vector) and four packed dot products per entry, the
@@ -9,6 +9,10 @@
 // vector of its (slice, group range); a second kernel adds the partial vectors
 // of a row in a fixed order, adds the bias and rounds once.  No atomics: the
 // result does not depend on timing.
+#include <stdlib.h>
+
+#include <mutex>
+
 #include "common.hpp"
 #include "sliced_format.hpp"
 
@@ -23,9 +27,30 @@ struct SlicedArgs {
   const SlicedWorkgroup* wgs;
   const uint32_t* rowmap;
   const uint8_t* entries;
-  float* partials;  // [n_partials][n]
+  float* partials;  // two-kernel finish: [n_partials][n] per token
+  // Fused finish (n_partials < 256): one 64-bit word per (token, row), zero between calls.
+  // Bits 16-63: sum of the partial sums in units of 2^-24 (two's complement); bits 8-15: how
+  // many of them went to `spill` instead; bits 0-7: how many lanes have added so far.
+  unsigned long long* sums;
+  float* spill;       // [token][row], zero between calls: partial sums the fixed-point word cannot hold
+  const float* bias;  // f32 [n] or null
+  void* y;
+  int64_t ldy;
+  int n_partials, fused_finish;
   int n, nc, slice_rows;
+  int wg_quads;       // entry quads per workgroup
+  // Regular geometry (regular != 0): every slice has `parts` group ranges of `range_groups`
+  // groups and workgroup w = (part * row_blocks + row block) * n_slices + slice, so a workgroup
+  // knows its slice and group range without reading its record.
+  int regular, n_slices, row_blocks, parts, range_groups, groups, rows_per_block;
+  uint32_t magic_slices, magic_blocks;  // ceil(2^32 / n_slices), ceil(2^32 / row_blocks)
+  uint32_t wave_info[kSlicedWaves];     // quads of the wave's strip | first quad inside the workgroup << 16
 };
+
+// n / d for n * d < 2^32 with magic = ceil(2^32 / d) (d = 1: magic does not fit, n is returned).
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t d, uint32_t magic) {
+  return d == 1u ? n : __umulhi(n, magic);
+}
 
 // Operands are taken by value: __builtin_bit_cast applied directly to a vector
 // element expression (v.y) reads element 0 with this compiler.
@@ -49,21 +74,26 @@ struct Quad {
   uint32_t d0, d1, d2;
 };
 
-// Entry quads requested ahead per lane.  Measured on a 14336 x 4096 layer: 3 in flight 10.6 us,
-// 8 in flight 12.1 us (the entries then arrive wave by wave instead of interleaved, and the
-// last waves start working late).
-constexpr int kQuadsInFlight = 3;
+// Entry quads a lane keeps requested ahead of the one it works on.
+constexpr int kDepth = 3;
+// Straight-line code exists for strips of up to this many quads, at up to kStraightTokens tokens.
+constexpr int kMaxStraightQuads = 16;
+constexpr int kStraightTokens = 2;
 // LDS map: activations of the group range, then the slice, then the zero row that
 // padding entries select.  Both bases fit the 16-bit offset field of an LDS read.
 constexpr int kMaxTokens = 7;  // tokens per pass over the entries (an eighth token's activations would not fit in LDS)
-constexpr int kLdsX = 0;       // [token][group] vectors: a token's 256 vectors are contiguous, so the
+constexpr int kLdsX = 0;       // [token][group] vectors: a token's 512 vectors are contiguous, so the
                                // lanes of a read spread over all sixteen 16-byte bank groups
 constexpr int kLdsSlice = kSlicedMaxGroups * 16 * kMaxTokens;
-constexpr int kLdsBytes = kLdsSlice + (kSlicedMaxSliceRows + 1) * 16;
+constexpr int kLdsStage = kLdsSlice + (kSlicedMaxSliceRows + 1) * 16;  // [token][row of the block] sums, fused finish
+constexpr int kLdsBytes = kLdsStage + kMaxTokens * kSlicedTasks * 4;
 static_assert(kLdsBytes <= kSlicedLdsBytes && kLdsSlice < 65536, "LDS map");
+// The first eight waves copy the slice into LDS.
+constexpr int kLoaderThreads = kSlicedTasks / 2;
+constexpr int kSliceLoads = kSlicedMaxSliceRows / kLoaderThreads;
 
-__device__ __forceinline__ void load_quad(Quad& q, const uint8_t* strip_lane, int qi) {
-  __builtin_memcpy(&q, __builtin_assume_aligned(strip_lane + (size_t)qi * kSlicedQuadBytes, 4), 12);
+__device__ __forceinline__ void load_quad(Quad& q, const uint8_t* p) {
+  __builtin_memcpy(&q, __builtin_assume_aligned(p, 4), 12);
 }
 
 template <uint32_t MASK>
@@ -73,22 +103,36 @@ __device__ __forceinline__ uint32_t low_field(uint32_t v) {
   return r;
 }
 
-// The four entries of one quad.  A lane's record is four 16-bit rows followed by
-// four 8-bit groups, so each LDS address is one field extracted and shifted: two
-// instructions.  (Written as a plain mask, the low fields become shift + mask + add.)
+// The LDS byte addresses of the four entries of one quad: codebook row and activation vector.
+// A lane's record is four 16-bit row fields followed by four group bytes.
+struct QuadAddr {
+  uint32_t row[4], grp[4];
+};
+
+__device__ __forceinline__ QuadAddr quad_addresses(const Quad& q) {
+  QuadAddr ad;
+  // Row fields: bits 0-12 the row, bit 15 the ninth bit of the group (256 groups = 4096 bytes).
+  const uint32_t f[4] = {q.d0, q.d0 >> 16, q.d1, q.d1 >> 16};
+  const uint32_t glow[4] = {low_field<0xFFu>(q.d2), (q.d2 >> 8) & 0xFFu, (q.d2 >> 16) & 0xFFu, q.d2 >> 24};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    ad.row[j] = (f[j] & 0x1FFFu) << 4;
+    ad.grp[j] = (glow[j] << 4) | ((f[j] & 0x8000u) >> 3);
+  }
+  return ad;
+}
+
 // Per entry: one codebook row and M activation vectors from LDS, 4 M dot products.
 template <int ACT, int M>
-__device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, float (&acc)[M][2]) {
-  const uint32_t row[4] = {low_field<0xFFFFu>(q.d0), q.d0 >> 16, low_field<0xFFFFu>(q.d1), q.d1 >> 16};
-  const uint32_t grp[4] = {low_field<0xFFu>(q.d2), (q.d2 >> 8) & 0xFFu, (q.d2 >> 16) & 0xFFu, q.d2 >> 24};
+__device__ __forceinline__ void run_quad(const QuadAddr& ad, const uint8_t* lds, float (&acc)[M][2]) {
   constexpr int kBatch = M > 2 ? 2 : 4;  // entries whose LDS reads are issued together
 #pragma unroll
   for (int j0 = 0; j0 < 4; j0 += kBatch) {
     u32x4 c[kBatch], xv[kBatch][M];
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {
-      c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + (row[j0 + j] << 4));
-      const uint8_t* xg = lds + kLdsX + (grp[j0 + j] << 4);
+      c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + ad.row[j0 + j]);
+      const uint8_t* xg = lds + kLdsX + ad.grp[j0 + j];
 #pragma unroll
       for (int m = 0; m < M; ++m) xv[j][m] = *reinterpret_cast<const u32x4*>(xg + m * (kSlicedMaxGroups * 16));
     }
@@ -99,38 +143,104 @@ __device__ __forceinline__ void run_quad(const Quad& q, const uint8_t* lds, floa
   }
 }
 
+// Fused finish: the lane adds its partial sum, as a 40.24 fixed-point number, to the row's word
+// with one returning atomic; integer addition does not depend on the order of arrival, so the
+// result is the same from run to run.  The lane whose addition completes the count converts the
+// sum back, adds the bias, rounds once, stores y and clears the word for the next call.  A
+// partial sum of magnitude 2^15 or more (or a NaN) goes to a float accumulator instead, which
+// the finishing lane adds in (those sums are added in order of arrival).
+constexpr float kFixedOne = 16777216.f;     // 2^24
+constexpr float kFixedLimit = 32768.f;      // 2^15: 255 such sums stay inside 47 bits
+template <int ACT>
+__device__ __forceinline__ void finish_row(const SlicedArgs& a, int m, uint32_t row, float v) {
+  const size_t cell = (size_t)m * a.n + row;
+  const bool fits = fabsf(v) < kFixedLimit;  // false for NaN and infinities
+  unsigned long long add = 1ull;
+  if (fits) {
+    add += (unsigned long long)(long long)__float2ll_rn(v * kFixedOne) << 16;
+  } else {
+    __hip_atomic_fetch_add(a.spill + cell, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // returns: done before the count
+    add += 0x100ull;
+  }
+  const unsigned long long old = __hip_atomic_fetch_add(a.sums + cell, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if ((int)(old & 0xFFull) != a.n_partials - 1) return;
+  const unsigned long long total = old + add;
+  float sum = (float)((double)((long long)total >> 16) * (1.0 / 16777216.0));  // exact product, one rounding
+  if ((total >> 8) & 0xFFull) sum += __hip_atomic_exchange(a.spill + cell, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (a.bias) sum += a.bias[row];
+  store_from_f32<ACT>((uint16_t*)a.y + (size_t)m * a.ldy, row, sum);
+  __hip_atomic_store(a.sums + cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The NQ quads of a strip, of which the first min(kDepth, NQ) have been requested into q.
+// Straight-line code: the compiler knows how many loads are in flight at each use of a quad.
+template <int ACT, int M, int NQ>
+__device__ __forceinline__ void walk_strip(Quad (&q)[kDepth], const uint8_t* strip_lane, const uint8_t* lds,
+                                           float (&acc)[M][2]) {
+  constexpr int D = kDepth;
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    // The addresses are taken out of the quad before its registers are asked for again.
+    const QuadAddr ad = quad_addresses(q[i % D]);
+    if (i + D < NQ) load_quad(q[i % D], strip_lane + (size_t)(i + D) * kSlicedQuadBytes);
+    run_quad<ACT, M>(ad, lds, acc);
+  }
+}
+
 template <int ACT, int M, bool PERM>
 __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr int D = kDepth;
   u32x4* xl = reinterpret_cast<u32x4*>(lds + kLdsX);
   u32x4* cb = reinterpret_cast<u32x4*>(lds + kLdsSlice);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const SlicedWorkgroup& wg = a.wgs[blockIdx.x];
-  const int steps = (int)wg.wave[wave].steps;
-  const int nq = (steps + 3) >> 2;  // a strip is padded to whole quads, so padded steps are run too
-  const uint8_t* strip_lane = a.entries + (size_t)wg.wave[wave].quad_begin * kSlicedQuadBytes + (size_t)lane * 12;
+  const uint32_t info = a.wave_info[wave];
+  const int nq = (int)(info & 0xFFFFu);
+  // A wave without a strip (nq = 0) reads the workgroup's first quad and ignores it.
+  const uint8_t* const strip_lane = a.entries +
+                                    ((size_t)blockIdx.x * (size_t)a.wg_quads + (size_t)(nq ? info >> 16 : 0u)) * kSlicedQuadBytes +
+                                    (size_t)lane * 12;
+  uint32_t slice, partial, g_begin, g_count, row_begin, row_count;
+  if (a.regular) {
+    const uint32_t w = blockIdx.x;
+    const uint32_t j = fast_div(w, (uint32_t)a.n_slices, a.magic_slices);
+    const uint32_t part = fast_div(j, (uint32_t)a.row_blocks, a.magic_blocks);
+    slice = w - j * (uint32_t)a.n_slices;
+    partial = slice * (uint32_t)a.parts + part;
+    g_begin = part * (uint32_t)a.range_groups;
+    g_count = min((uint32_t)a.range_groups, (uint32_t)a.groups - g_begin);
+    row_begin = min((j - part * (uint32_t)a.row_blocks) * (uint32_t)a.rows_per_block, (uint32_t)a.n);
+    row_count = min((uint32_t)a.rows_per_block, (uint32_t)a.n - row_begin);
+  } else {
+    const SlicedWorkgroup wg = a.wgs[blockIdx.x];
+    slice = wg.slice; partial = wg.partial; g_begin = wg.g_begin; g_count = wg.g_count;
+    row_begin = wg.row_begin; row_count = wg.row_count;
+  }
 
   // Requests in the order they are needed: the slice and the activations (mostly
   // L2 hits) first, then the entries, which stream from HBM while the slice is
-  // being stored and the first quads are worked on.
-  Quad q[kQuadsInFlight];
+  // being stored and the first quads are worked on.  The first eight waves copy the slice;
+  // the others have nothing in front of their first entry requests.
+  Quad q[D];
   {
-    const int slice_len = min(a.slice_rows, a.nc - (int)wg.slice * a.slice_rows);
-    const u32x4* src = a.codebook + (int64_t)wg.slice * a.slice_rows;
-    const int g_count = (int)wg.g_count;
-    u32x4 t[8];
+    const int slice_len = min(a.slice_rows, a.nc - (int)slice * a.slice_rows);
+    const u32x4* src = a.codebook + (int64_t)slice * a.slice_rows;
+    const bool loader = tid < kLoaderThreads;  // wave-uniform
+    u32x4 t[kSliceLoads];
+    if (loader) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) t[i] = src[min(tid + i * kSlicedTasks, slice_len - 1)];
-    // Thread t stages group t % 256 of tokens t / 256 and t / 256 + 4 (256 groups x 7 tokens at most).
-    constexpr int kXLoads = M > 4 ? 2 : 1;
+      for (int i = 0; i < kSliceLoads; ++i) t[i] = src[min(tid + i * kLoaderThreads, slice_len - 1)];
+    }
+    // Thread t stages group t % 512 of tokens t / 512, t / 512 + 2, ... (512 groups x 7 tokens at most).
+    constexpr int kXLoads = (M + 1) / 2;
     const int xg = tid & (kSlicedMaxGroups - 1), xm = tid / kSlicedMaxGroups;
-    const int xvec = (int)wg.g_begin + min(xg, g_count - 1);
+    const int xvec = (int)g_begin + min(xg, (int)g_count - 1);
     const uint16_t* xrow[kXLoads];
     u32x4 xt[kXLoads], perm_lo, perm_hi;
 #pragma unroll
-    for (int i = 0; i < kXLoads; ++i) xrow[i] = a.x + (int64_t)min(xm + 4 * i, M - 1) * a.ldx;
+    for (int i = 0; i < kXLoads; ++i) xrow[i] = a.x + (int64_t)min(xm + 2 * i, M - 1) * a.ldx;
     if constexpr (PERM) {  // the eight source columns of this vector; the elements follow below
       perm_lo = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec];
       perm_hi = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec + 1];
@@ -139,10 +249,9 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
       for (int i = 0; i < kXLoads; ++i) xt[i] = reinterpret_cast<const u32x4*>(xrow[i])[xvec];
     }
     __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
-    // The first quads (past the strip's end: its last quad again, or quad 0
-    // of the blob for a wave without a strip; no branch around a load).
+    // The first quads (past the strip's end: its last quad again; no branch around a load).
 #pragma unroll
-    for (int i = 0; i < kQuadsInFlight; ++i) load_quad(q[i], strip_lane, max(min(i, nq - 1), 0));
+    for (int i = 0; i < D; ++i) load_quad(q[i], strip_lane + (size_t)max(min(i, nq - 1), 0) * kSlicedQuadBytes);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (PERM) {
       const uint32_t pc[8] = {perm_lo.x, perm_lo.y, perm_lo.z, perm_lo.w, perm_hi.x, perm_hi.y, perm_hi.z, perm_hi.w};
@@ -154,56 +263,89 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
         xt[i] = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
       }
     }
+    if (loader) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      if (tid + i * kSlicedTasks < slice_len) cb[tid + i * kSlicedTasks] = t[i];
+      for (int i = 0; i < kSliceLoads; ++i)
+        if (tid + i * kLoaderThreads < slice_len) cb[tid + i * kLoaderThreads] = t[i];
+    }
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i)
-      if (xg < g_count && xm + 4 * i < M) xl[(xm + 4 * i) * kSlicedMaxGroups + xg] = xt[i];
+      if (xg < (int)g_count && xm + 2 * i < M) xl[(xm + 2 * i) * kSlicedMaxGroups + xg] = xt[i];
     if (tid == kSlicedTasks - 1) cb[kSlicedPadRow] = u32x4{0u, 0u, 0u, 0u};  // what padding entries select
   }
   const uint32_t row = a.rowmap[(size_t)blockIdx.x * kSlicedTasks + tid];
   __syncthreads();
 
-  // kQuadsInFlight quads stay in flight: each one is replaced by the quad that many
-  // further on as soon as it has been read.
   float acc[M][2];
 #pragma unroll
   for (int m = 0; m < M; ++m) acc[m][0] = acc[m][1] = 0.f;
-  int q0 = 0;
-  for (; q0 + 2 * kQuadsInFlight <= nq; q0 += kQuadsInFlight) {
+  if (M <= kStraightTokens && nq <= kMaxStraightQuads) {
+    // Strips of up to kMaxStraightQuads quads (all of them, unless a row's indices crowd into one
+    // slice) are walked by straight-line code picked by the strip's length: no loop carries a
+    // register that is being loaded (a loop drains the quads in flight at every back-edge to
+    // rename them).
+    switch (nq) {
+#define NPAMD_STRIP_CASE(NQ) \
+  case NQ: walk_strip<ACT, M, NQ>(q, strip_lane, lds, acc); break;
+      NPAMD_STRIP_CASE(1) NPAMD_STRIP_CASE(2) NPAMD_STRIP_CASE(3) NPAMD_STRIP_CASE(4)
+      NPAMD_STRIP_CASE(5) NPAMD_STRIP_CASE(6) NPAMD_STRIP_CASE(7) NPAMD_STRIP_CASE(8)
+      NPAMD_STRIP_CASE(9) NPAMD_STRIP_CASE(10) NPAMD_STRIP_CASE(11) NPAMD_STRIP_CASE(12)
+      NPAMD_STRIP_CASE(13) NPAMD_STRIP_CASE(14) NPAMD_STRIP_CASE(15) NPAMD_STRIP_CASE(16)
+#undef NPAMD_STRIP_CASE
+      default: break;
+    }
+  } else {
+    // Longer strips and more tokens: three plain loops.
+    int q0 = 0;
+    for (; q0 + 2 * D <= nq; q0 += D) {
 #pragma unroll
-    for (int i = 0; i < kQuadsInFlight; ++i) {
-      const Quad cur = q[i];
-      load_quad(q[i], strip_lane, q0 + i + kQuadsInFlight);
-      run_quad<ACT, M>(cur, lds, acc);
+      for (int i = 0; i < D; ++i) {
+        const QuadAddr ad = quad_addresses(q[i]);
+        load_quad(q[i], strip_lane + (size_t)(q0 + i + D) * kSlicedQuadBytes);
+        run_quad<ACT, M>(ad, lds, acc);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      if (q0 + i >= nq) break;
+      const QuadAddr ad = quad_addresses(q[i]);
+      if (q0 + i + D < nq) load_quad(q[i], strip_lane + (size_t)(q0 + i + D) * kSlicedQuadBytes);
+      run_quad<ACT, M>(ad, lds, acc);
+    }
+    q0 += D;
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      if (q0 + i >= nq) break;
+      run_quad<ACT, M>(quad_addresses(q[i]), lds, acc);
     }
   }
+  if (a.fused_finish) {
+    // The lanes of a wave work for rows scattered over the workgroup's block (strips are sorted
+    // by length); the sums change hands through LDS so that thread t finishes row row_begin + t
+    // and a wave's atomics, bias reads and stores fall on consecutive addresses.
+    float* stage = reinterpret_cast<float*>(lds + kLdsStage);
+    if (row != kSlicedNoRow) {
 #pragma unroll
-  for (int i = 0; i < kQuadsInFlight; ++i) {
-    if (q0 + i >= nq) break;
-    const Quad cur = q[i];
-    if (q0 + i + kQuadsInFlight < nq) load_quad(q[i], strip_lane, q0 + i + kQuadsInFlight);
-    run_quad<ACT, M>(cur, lds, acc);
-  }
-  q0 += kQuadsInFlight;
+      for (int m = 0; m < M; ++m) stage[m * kSlicedTasks + (row - row_begin)] = acc[m][0] + acc[m][1];
+    }
+    __syncthreads();
+    if ((uint32_t)tid < row_count) {
 #pragma unroll
-  for (int i = 0; i < kQuadsInFlight; ++i) {
-    if (q0 + i >= nq) break;
-    run_quad<ACT, M>(q[i], lds, acc);
-  }
-  if (row != kSlicedNoRow) {
+      for (int m = 0; m < M; ++m) finish_row<ACT>(a, m, row_begin + (uint32_t)tid, stage[m * kSlicedTasks + tid]);
+    }
+  } else if (row != kSlicedNoRow) {
 #pragma unroll
     for (int m = 0; m < M; ++m)
-      a.partials[(size_t)m * a.token_stride + (size_t)wg.partial * a.n + row] = acc[m][0] + acc[m][1];
+      a.partials[(size_t)m * a.token_stride + (size_t)partial * a.n + row] = acc[m][0] + acc[m][1];
   }
 }
 
+// Two-kernel finish (256 partial vectors or more per row):
 // y[token][row] = round(sum over the partial vectors + bias).  16 rows per block
 // (blockIdx.y = token); the partial vectors are dealt over 16 threads per row,
 // whose sums are then added in a fixed order.
 template <int ACT>
-__global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restrict__ partials, int n_partials,
+__global__ void __launch_bounds__(256) sliced_reduce_kernel(float* __restrict__ partials, int n_partials,
                                                              int n, const float* __restrict__ bias,
                                                              void* __restrict__ y, int64_t ldy) {
   __shared__ float red[16][17];
@@ -213,7 +355,10 @@ __global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restr
   y = (uint16_t*)y + (size_t)blockIdx.y * ldy;
   float sum = 0.f;
   if (row < n)
-    for (int p = j; p < n_partials; p += 16) sum += partials[(size_t)p * n + row];
+    for (int p = j; p < n_partials; p += 16) {
+      sum += partials[(size_t)p * n + row];
+      partials[(size_t)p * n + row] = 0.f;  // the workspace is handed back zero-filled
+    }
   red[j][r] = sum;
   __syncthreads();
   if (j == 0 && row < n) {
@@ -227,16 +372,16 @@ __global__ void __launch_bounds__(256) sliced_reduce_kernel(const float* __restr
 
 template <int ACT, int M, bool PERM>
 int launch_sliced_tokens_p(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
-  static int reserved = 0;
-  if (reserved == 0) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M, PERM>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    if (e != hipSuccess)
-      return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(e));
-    reserved = kLdsBytes;
-  }
+  static std::once_flag once;
+  static hipError_t reserve_error = hipSuccess;
+  std::call_once(once, [] {
+    reserve_error = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M, PERM>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  });
+  if (reserve_error != hipSuccess)
+    return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(reserve_error));
   sliced_gemv_kernel<ACT, M, PERM><<<n_workgroups, kSlicedTasks, kLdsBytes, st>>>(a);
-  return NPAMD_OK;
+  return check_launch(what);
 }
 
 template <int ACT, int M>
@@ -244,6 +389,12 @@ int launch_sliced_tokens(const SlicedArgs& a, int n_workgroups, hipStream_t st, 
   return a.column_perm ? launch_sliced_tokens_p<ACT, M, true>(a, n_workgroups, st, what)
                        : launch_sliced_tokens_p<ACT, M, false>(a, n_workgroups, st, what);
 }
+
+// The fused finish counts the partial sums of a row in eight bits.
+inline bool sliced_fused_finish(const npamd_sliced_header& h) { return h.n_partials < 256; }
+
+// ceil(2^32 / d) for fast_div; d = 1 never uses it.
+inline uint32_t div_magic(uint32_t d) { return d <= 1u ? 0u : (uint32_t)(((1ull << 32) + d - 1) / d); }
 
 template <int ACT>
 int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void* x, int64_t ldx,
@@ -258,9 +409,35 @@ int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void*
   a.n = h.n; a.nc = h.nc; a.slice_rows = h.slice_rows;
   a.ldx = ldx;
   a.token_stride = (int64_t)h.n_partials * (int64_t)h.n;
+  a.n_partials = h.n_partials;
+  a.fused_finish = sliced_fused_finish(h);
+  a.bias = bias;
+  a.ldy = ldy;
+  uint32_t begin = 0;
+  for (int w = 0; w < kSlicedWaves; ++w) {
+    a.wave_info[w] = (uint32_t)h.wave_quads[w] | (begin << 16);
+    begin += h.wave_quads[w];
+  }
+  a.wg_quads = (int)(begin ? begin : 1u);
+  // The regular geometry, when the header states it and the counts bear it out.
+  a.groups = h.k / 8;
+  a.n_slices = h.n_slices;
+  a.parts = h.n_partials / h.n_slices;
+  a.row_blocks = a.parts ? h.n_workgroups / (a.parts * h.n_slices) : 0;
+  a.range_groups = a.parts ? (a.groups + a.parts - 1) / a.parts : 0;
+  a.rows_per_block = a.row_blocks ? (h.n + a.row_blocks - 1) / a.row_blocks : 0;
+  a.regular = (h.flags & kSlicedRoundRobin) && a.parts >= 1 && a.row_blocks >= 1 &&
+              a.parts * h.n_slices == h.n_partials && a.row_blocks * h.n_partials == h.n_workgroups &&
+              (int64_t)(a.parts - 1) * a.range_groups < a.groups && a.rows_per_block <= kSlicedTasks &&
+              h.n_workgroups < 65536 && h.n_slices < 65536;
+  a.magic_slices = div_magic((uint32_t)a.n_slices);
+  a.magic_blocks = div_magic((uint32_t)a.row_blocks);
   for (int m0 = 0; m0 < M; m0 += kMaxTokens) {
     a.x = (const uint16_t*)x + (size_t)m0 * ldx;
     a.partials = workspace + (size_t)m0 * a.token_stride;
+    a.sums = reinterpret_cast<unsigned long long*>(workspace) + (size_t)m0 * h.n;
+    a.spill = workspace + 2 * (size_t)M * h.n + (size_t)m0 * h.n;
+    a.y = (uint16_t*)y + (size_t)m0 * ldy;
     int rc;
     switch (M - m0 >= kMaxTokens ? kMaxTokens : M - m0) {
       case 1: rc = launch_sliced_tokens<ACT, 1>(a, h.n_workgroups, st, what); break;
@@ -273,7 +450,7 @@ int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void*
     }
     if (rc != NPAMD_OK) return rc;
   }
-  if (y)
+  if (!a.fused_finish)
     sliced_reduce_kernel<ACT><<<dim3((h.n + 15) / 16, M), 256, 0, st>>>(workspace, h.n_partials, h.n, bias, y, ldy);
   return check_launch(what);
 }
@@ -301,7 +478,7 @@ extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* c
   NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1, "%s: bad counts in header", what);
   NPAMD_REQUIRE(ldx >= h.k && ldy >= h.n, "%s: row stride smaller than the row", what);
   if (M == 0) return NPAMD_OK;
-  NPAMD_REQUIRE(x && blob && codebook && workspace, "%s: null pointer", what);
+  NPAMD_REQUIRE(x && blob && codebook && workspace && y, "%s: null pointer", what);
   NPAMD_REQUIRE(ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(codebook) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(blob) % 16) == 0 &&

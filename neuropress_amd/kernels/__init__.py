@@ -269,7 +269,7 @@ class SlicedIndices:
     """
 
     _FIELDS = ("magic", "version", "n", "k", "vl", "nc", "slice_rows", "n_slices", "n_workgroups",
-               "n_partials", "groups_max", "reserved32", "n_quads", "n_entries", "off_workgroups",
+               "n_partials", "groups_max", "flags", "n_quads", "n_entries", "off_workgroups",
                "off_rowmap", "off_entries", "total_bytes")  # fmt: skip
 
     def __init__(self, blob: torch.Tensor, header: bytes):
@@ -281,9 +281,10 @@ class SlicedIndices:
         self.blob = blob
         self.header = header
         self._header_buf = ctypes.create_string_buffer(header, len(header))
-        values = struct.unpack("<2I10i6q", header[:96])
+        values = struct.unpack("<2I9iI6q", header[:96])
         for name, value in zip(self._FIELDS, values):
             setattr(self, name, value)
+        self.wave_quads = struct.unpack("<16H", header[96:128])
 
     @property
     def header_ptr(self) -> int:
@@ -343,21 +344,38 @@ def vq_slice_indices(
     return SlicedIndices(blob.to(dev), header)
 
 
+_SLICED_WORKSPACES: dict = {}
+
+
+def sliced_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """The zero-filled scratch of :func:`vq_linear_sliced` for the current stream of *device*.
+
+    Every call hands its workspace back zero-filled, so one buffer per (device, stream) serves
+    all layers whose calls follow each other on that stream.  Grown (and zero-filled again) on
+    demand; allocate it before a graph capture starts, e.g. through ``NPVQLinear.prepare_sliced``.
+    """
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _SLICED_WORKSPACES.get(key)
+    if ws is None or ws.numel() * 4 < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20) // 4 + 4, device=device, dtype=torch.float32)
+        _SLICED_WORKSPACES[key] = ws
+    return ws
+
+
 def vq_linear_sliced(
     x: torch.Tensor,
     sliced: SlicedIndices,
     centroids: torch.Tensor,
     bias: torch.Tensor | None = None,
     workspace: torch.Tensor | None = None,
-    partials_only: bool = False,
     column_perm: torch.Tensor | None = None,
-) -> torch.Tensor | None:
+) -> torch.Tensor:
     """Decode GEMV over the slice-list form, ``M <= 32`` (``npamd_vq_gemv_sliced``).
 
     *centroids* must already be in ``x.dtype`` (the modules cache that copy).
-    *workspace*: optional float32 scratch of ``sliced.workspace_bytes(M) / 4`` elements;
-    after the call it holds the ``[M, n_partials, N]`` partial sums.  With
-    *partials_only* nothing else is computed and None is returned.
+    *workspace*: optional float32 scratch of at least ``sliced.workspace_bytes(M) / 4``
+    elements, zero-filled before its first use (every call leaves it zero-filled); by
+    default the per-stream buffer of :func:`sliced_workspace`.
     *column_perm*: int32 ``[K]``; the kernel then computes with ``x[:, column_perm]``
     (the reference's input permutation, np_vq_linear.py:1027-1028) without materialising it.
     """
@@ -378,10 +396,10 @@ def vq_linear_sliced(
         raise RuntimeError(f"{what}: slice lists were built for K={sliced.k}, codebook [{sliced.nc}, {sliced.vl}]")
     need = sliced.workspace_bytes(max(m, 1))
     if workspace is None:
-        workspace = torch.empty(need // 4, device=x.device, dtype=torch.float32)
+        workspace = sliced_workspace(x.device, need)
     elif workspace.dtype != torch.float32 or not workspace.is_contiguous():
         raise RuntimeError(f"{what}: workspace must be a contiguous float32 tensor")
-    y = None if partials_only else torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
+    y = torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
     b32 = _bias_f32(bias)
     _lib.call(
         "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), _ptr(column_perm), sliced.header_ptr, sliced.blob.data_ptr(),

@@ -67,42 +67,52 @@ def within_tol(y: np.ndarray, ref: np.ndarray, atol=1e-2, rtol=1e-2):
 def decode_sliced_blob(blob: np.ndarray) -> tuple[np.ndarray, dict]:
     """Read a slice-list blob back into the ``[N, K/8]`` index matrix it was built from.
 
-    An independent reader of the layout (header, workgroup records with their
-    16 wave records, per-lane row map, and per lane and quad a 12-byte record of
-    four uint16 codebook rows followed by four uint8 groups).  ``hits`` counts how often each (row, group) pair was filed and
-    ``writes`` how often each (partial, row) cell is written; both must be 1
-    everywhere.
+    An independent reader of the layout: header (with the 16 strip lengths every
+    workgroup shares), 32-byte workgroup records, per-lane row map, and per
+    workgroup, wave, quad and lane a 12-byte record of four uint16 fields (13-bit
+    codebook row, top bit = bit 8 of the group) followed by the four groups' low bytes.  ``hits`` counts how often each (row, group)
+    pair was filed and ``writes`` how often each (partial, row) cell is written;
+    both must be 1 everywhere.
     """
     import struct
 
     names = ("magic", "version", "n", "k", "vl", "nc", "slice_rows", "n_slices", "n_workgroups",
-             "n_partials", "groups_max", "reserved32", "n_quads", "n_entries", "off_workgroups",
+             "n_partials", "groups_max", "flags", "n_quads", "n_entries", "off_workgroups",
              "off_rowmap", "off_entries", "total_bytes")  # fmt: skip
-    h = dict(zip(names, struct.unpack("<2I10i6q", blob[:96].tobytes())))
-    assert h["magic"] == 0x4C53504E and h["vl"] == 8
+    h = dict(zip(names, struct.unpack("<2I9iI6q", blob[:96].tobytes())))
+    wave_quads = struct.unpack("<16H", blob[96:128].tobytes())
+    h["wave_quads"] = wave_quads
+    assert h["magic"] == 0x4C53504E and h["version"] == 3 and h["vl"] == 8
     n, groups, n_wg = h["n"], h["k"] // 8, h["n_workgroups"]
-    wgs = np.frombuffer(blob, dtype="<u4", count=n_wg * 40, offset=h["off_workgroups"]).reshape(n_wg, 40).astype(np.int64)
+    wg_quads = max(sum(wave_quads), 1)
+    assert h["n_quads"] == n_wg * wg_quads
+    wgs = np.frombuffer(blob, dtype="<u4", count=n_wg * 8, offset=h["off_workgroups"]).reshape(n_wg, 8).astype(np.int64)
     rowmap = np.frombuffer(blob, dtype="<u4", count=n_wg * 1024, offset=h["off_rowmap"]).reshape(n_wg, 16, 64).astype(np.int64)
-    quads = np.frombuffer(blob, dtype=np.uint8, count=h["n_quads"] * 768, offset=h["off_entries"]).reshape(-1, 64, 12)
+    quads = np.frombuffer(blob, dtype=np.uint8, count=h["n_quads"] * 768, offset=h["off_entries"]).reshape(n_wg, wg_quads, 64, 12)
     idx = np.full((n, groups), -1, dtype=np.int64)
     hits = np.zeros((n, groups), dtype=np.int32)
     writes = np.zeros((h["n_partials"], n), dtype=np.int32)
     for w in range(n_wg):
-        sl, partial, g_begin, g_count = wgs[w, :4]
+        sl, partial, g_begin, g_count, row_begin, row_count = wgs[w, :6]
+        assert row_count <= 1024 and row_begin + row_count <= n
+        if h["flags"] & 1:  # workgroup w works on slice w % n_slices
+            assert sl == w % h["n_slices"]
+        quad_begin = 0
         for s in range(16):
-            quad_begin, steps = wgs[w, 8 + 2 * s], wgs[w, 9 + 2 * s]
+            nq = wave_quads[s]
             rows = rowmap[w, s]
             has_row = rows != 0xFFFFFFFF
+            assert ((rows[has_row] >= row_begin) & (rows[has_row] < row_begin + row_count)).all()
             np.add.at(writes, (np.full(int(has_row.sum()), partial), rows[has_row]), 1)
-            nq = (steps + 3) // 4
             if nq == 0:
                 continue
-            q = quads[quad_begin : quad_begin + nq].astype(np.int64)  # [nq, lane, 12]
-            local = (q[..., 0:8:2] | (q[..., 1:8:2] << 8)).transpose(1, 0, 2).reshape(64, nq * 4)  # [lane, step]
-            g_local = q[..., 8:12].transpose(1, 0, 2).reshape(64, nq * 4)
-            live = local != 8192  # 8192 = the zero row padding entries select
+            q = quads[w, quad_begin : quad_begin + nq].astype(np.int64)  # [nq, lane, 12]
+            quad_begin += nq
+            field = (q[..., 0:8:2] | (q[..., 1:8:2] << 8)).transpose(1, 0, 2).reshape(64, nq * 4)  # [lane, step]
+            local = field & 0x1FFF  # bits 0-12: the row; bit 15: bit 8 of the group
+            g_local = q[..., 8:12].transpose(1, 0, 2).reshape(64, nq * 4) | ((field >> 15) << 8)
+            live = local != 4096  # 4096 = the zero row padding entries select
             assert (g_local < g_count).all() and (local[live] < h["slice_rows"]).all()
-            assert not live[:, steps:].any(), "live entry beyond the strip's step count"
             assert not live[~has_row].any(), "live entry in a lane without a row"
             rr = np.broadcast_to(rows[:, None], local.shape)[live]
             gg = (g_begin + g_local)[live]

@@ -68,7 +68,7 @@ def test_sliced_gemv_in_a_graph(gpu, m):
     L = cases.vq_layer(12, 300, 256, 20000, act=torch.float16, m=m, std=0.05)
     sl = kernels.vq_slice_indices(L["packed"], L["bits"], 300, 256, 8, 20000, device=gpu)
     cb = L["cb"].to(gpu)
-    ws = torch.empty(sl.workspace_bytes(m) // 4, device=gpu, dtype=torch.float32)
+    ws = torch.zeros(sl.workspace_bytes(m) // 4, device=gpu, dtype=torch.float32)
     mk = lambda i: [torch.randn(m, 256, generator=cases.gen(300 + i)).to(torch.float16).to(gpu)]
     _capture_and_replay(gpu, lambda inp: kernels.vq_linear_sliced(inp[0], sl, cb, None, workspace=ws), mk)
 

@@ -70,38 +70,75 @@ def test_sliced_gemv_zipf_indices(gpu, oracle_lib):
 def test_sliced_gemv_full_size_and_fused_gemv_agree(gpu, oracle_lib):
     """The headline benchmark shape (14336 x 4096, 65536 x 8 codebook, bf16), one token: against the
     oracle, against the fused GEMV (same f32-accumulated sum in another order), run to run,
-    and through the partial sums left in the workspace."""
+    and the workspace comes back zero-filled."""
     from neuropress_amd import kernels
 
     act = torch.bfloat16
     L = cases.vq_layer(1003, 14336, 4096, 65536, bits=16, act=act, m=1, bias=True, std=0.02)
-    ws = torch.empty(64 * 14336, device=gpu, dtype=torch.float32)
+    ws = torch.zeros(64 * 14336, device=gpu, dtype=torch.float32)
     y, sl = _run(gpu, L, act, workspace=ws)
     assert sl.n_workgroups <= 2 * torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert sl.n_partials < 256  # one kernel: every lane adds its partial sum with one atomic
     _check(y, _vq_ref(oracle_lib, L, act))
     cb = L["cb"].to(act).to(gpu)
     y_fused = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), cb, 16, 8, L["bias"].to(gpu), 14336)
     assert (y.float() - y_fused.float()).abs().max().item() <= 2 ** -6  # one bf16 ulp at |y| < 4
     for _ in range(3):
+        assert not ws.any()  # handed back zero-filled
         again = kernels.vq_linear_sliced(L["x"].to(gpu), sl, cb, L["bias"].to(gpu), workspace=ws)
         assert torch.equal(again, y)
-    partials = ws[: sl.n_partials * 14336].reshape(sl.n_partials, 14336)
-    total = partials.sum(0, dtype=torch.float64) + L["bias"].to(gpu).double()
-    assert (total - y.double()).abs().max().item() <= 2 ** -6
 
 
-def test_sliced_gemv_partials_only(gpu):
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 3])
+def test_sliced_gemv_partial_sums_outside_the_fixed_point_range(gpu, oracle_lib, act, m):
+    """Partial sums of magnitude 2^15 or more, infinities and NaNs bypass the fixed-point word
+    (float accumulator): large finite results, an overflowing row, a NaN row, and the rows
+    around them come out as the oracle's; the workspace is zero-filled afterwards."""
     from neuropress_amd import kernels
 
-    L = cases.vq_layer(5, 200, 128, 20000, act=torch.float16, m=1, std=0.05)
-    sl = kernels.vq_slice_indices(L["packed"], L["bits"], 200, 128, 8, 20000, device=gpu)
-    cb, x = L["cb"].to(gpu), L["x"].to(gpu)
-    ws = torch.full((sl.workspace_bytes(1) // 4,), float("nan"), device=gpu)
-    assert kernels.vq_linear_sliced(x, sl, cb, workspace=ws, partials_only=True) is None
-    y = kernels.vq_linear_sliced(x, sl, cb)
-    total = ws.reshape(sl.n_partials, 200).sum(0)
-    assert torch.isfinite(total).all()
-    assert (total - y.float()).abs().max().item() < 1e-2
+    n, k, nc = 96, 256, 9000
+    L = cases.vq_layer(31 + m, n, k, nc, act=act, m=m, bias=True, std=0.05)
+    cb = L["cb"].clone()
+    x = L["x"].clone()
+    cb *= 20.0  # entries ~ N(0, 1)
+    x[:, :8] = 1.0e4  # group 0 of every row contributes 1e4 * (sum of eight entries) ~ N(0, 2.8e4)
+    L["cb"], L["x"] = cb, x
+    ws = torch.zeros(64 * n * m, device=gpu, dtype=torch.float32)
+    sl = kernels.vq_slice_indices(L["packed"], L["bits"], n, k, 8, nc, device=gpu)
+    y = kernels.vq_linear_sliced(x.to(gpu), sl, cb.to(act).to(gpu), L["bias"].to(gpu), workspace=ws)
+    assert not ws.any()
+    code = orc.torch_dtype_code(act)
+    w = oracle_lib.vq_decode(L["packed"].numpy(), L["bits"], orc.to_bits(cb), n, k, code)
+    ref = oracle_lib.linear_f64(orc.to_bits(x), code, w, code, orc.to_bits(L["bias"]), code)
+    got = y.float().cpu().numpy().astype(np.float64)
+    lim = float(torch.finfo(act).max)
+    finite = np.abs(ref) < lim
+    assert np.abs(ref[finite]).max() > 2.0**15  # the case does leave the fixed-point range
+    assert np.all(np.abs(got[finite] - ref[finite]) <= 1e-2 + 1e-2 * np.abs(ref[finite]))
+    assert np.all(np.isinf(got[~finite]) & (np.sign(got[~finite]) == np.sign(ref[~finite])))
+    # NaN and infinity in the activations: the rows they reach are NaN / inf, as torch's would be.
+    x2 = L["x"].clone()
+    x2[0, 8] = float("nan")
+    y2 = kernels.vq_linear_sliced(x2.to(gpu), sl, cb.to(act).to(gpu), None, workspace=ws)
+    assert torch.isnan(y2[0]).any()
+    assert not ws.any()
+
+
+def test_sliced_gemv_two_kernel_finish(gpu, oracle_lib):
+    """A codebook of 2^20 rows has 256 slices: a row has more partial sums than the fused finish
+    counts, so the partial sums are written out and added by a second kernel."""
+    from neuropress_amd import kernels
+
+    n, k, nc, act = 40, 64, 1 << 20, torch.float16
+    L = cases.vq_layer(77, n, k, nc, bits=20, act=act, m=2, bias=True, std=0.05)
+    ws = torch.zeros(300 * n * 2 * 8, device=gpu, dtype=torch.float32)
+    y, sl = _run(gpu, L, act, workspace=ws)
+    assert sl.n_partials >= 256
+    _check(y, _vq_ref(oracle_lib, L, act))
+    assert not ws.any()
+    again, _ = _run(gpu, L, act, workspace=ws)
+    assert torch.equal(again, y)
 
 
 def test_sliced_wrapper_errors(gpu):
@@ -117,7 +154,7 @@ def test_sliced_wrapper_errors(gpu):
     with pytest.raises(RuntimeError, match="must be float16 or bfloat16"):
         kernels.vq_linear_sliced(x.float(), sl, cb.float())
     with pytest.raises(RuntimeError, match="workspace of"):
-        kernels.vq_linear_sliced(x, sl, cb, workspace=torch.empty(4, device=gpu))
+        kernels.vq_linear_sliced(x, sl, cb, workspace=torch.zeros(4, device=gpu))
     with pytest.raises(RuntimeError, match="VL = 8"):
         kernels.vq_slice_indices(L["packed"], L["bits"], 64, 64, 4, 20000, device=gpu)
 
