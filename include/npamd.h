@@ -213,6 +213,26 @@ int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
                          void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * npamd_vq_gemv_sliced for callers that cannot allocate device memory or pass a workspace along:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  The workspace is a device array inside this library,
+ * NPAMD_SLICED_STATIC_WORKSPACE_BYTES long, which every GPU the library runs on holds until the
+ * process ends; the call allocates and frees nothing (the array's address is looked up on the
+ * first call on each device, so make that call before a capture begins).  Requests whose
+ * npamd_vq_sliced_workspace_bytes() exceeds the array are rejected with NPAMD_ERR_INVALID.
+ * All calls on one GPU share the array: it starts zero-filled and every call hands it back
+ * zero-filled, so calls that follow each other (on one stream, or ordered by events) are
+ * fine, and calls that overlap on one GPU race.  Same arguments and results as
+ * npamd_vq_gemv_sliced otherwise.
+ */
+#define NPAMD_SLICED_STATIC_WORKSPACE_BYTES (4 * 1024 * 1024)
+int npamd_vq_gemv_sliced_static(const void* x, int64_t ldx, const int32_t* column_perm,
+                                const npamd_sliced_header* header_host,
+                                const void* blob, const void* codebook, int codebook_dtype,
+                                const float* bias, void* y, int64_t ldy, int M, int act_dtype,
+                                void* stream);
+
+/*
  * Decode GEMV over a prefix-coded index stream, read as it is stored (M <= NPAMD_GEMV_MAX_M):
  *   y[m, n] = sum_k x[m, k] * codebook[idx(n, k/VL), k%VL] (+ bias[n]).
  * Replaces vq_linear_tiered / vq_linear_ntier / vq_linear_zero_escape

@@ -15,7 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libnpamd.so"
 
 F16, BF16, F32 = 0, 1, 2
 GEMV_MAX_M = 32
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -45,6 +45,7 @@ SIGNATURES: dict[str, list] = {
                             _i64, _int, _int, _int, _int, _vp],  # fmt: skip
     "npamd_vq_sliced_workspace_bytes": [_vp, _int],
     "npamd_vq_gemv_sliced": [_vp, _i64, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _int, _int, _vp, _i64, _vp],
+    "npamd_vq_gemv_sliced_static": [_vp, _i64, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _int, _int, _vp],
     "npamd_rvq_dequant": [_vp, _i64, _int, _vp, _i64, _int, _vp, _int, _vp, _int, _vp, _vp, _int,
                           _int, _int, _vp, _int, _vp],  # fmt: skip
     "npamd_rvq_gemv": _RVQ_LINEAR,
@@ -61,6 +62,7 @@ SIGNATURES: dict[str, list] = {
 
 _RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64, "npamd_gemm_tile_workspace_bytes": _i64}
 SLICED_HEADER_BYTES = 128
+SLICED_STATIC_WORKSPACE_BYTES = 4 * 1024 * 1024
 
 _lib: ctypes.CDLL | None = None
 _load_error: str | None = None

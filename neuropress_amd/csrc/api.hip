@@ -121,7 +121,7 @@ int plan_tile_mw(int M) {
 
 }  // namespace npamd
 
-extern "C" int npamd_version(void) { return 2; }
+extern "C" int npamd_version(void) { return 3; }
 
 extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K < 64) return 0;

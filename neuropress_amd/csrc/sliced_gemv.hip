@@ -459,11 +459,11 @@ int launch_sliced(const npamd_sliced_header& h, const uint8_t* blob, const void*
 
 using namespace npamd;
 
-extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
-                                    const npamd_sliced_header* hp, const void* blob, const void* codebook,
-                                    int codebook_dtype, const float* bias, void* y, int64_t ldy, int M, int act_dtype,
-                                    void* workspace, int64_t workspace_bytes, void* stream) {
-  const char* what = "npamd_vq_gemv_sliced";
+// Argument checks shared by the two entry points.  `workspace` may be null on entry when the
+// caller fetches it afterwards (the entry point that brings its own): then only the rest is checked.
+static int check_sliced_call(const char* what, const void* x, int64_t ldx, const int32_t* column_perm,
+                             const npamd_sliced_header* hp, const void* blob, const void* codebook,
+                             int codebook_dtype, const void* y, int64_t ldy, int M, int act_dtype) {
   NPAMD_REQUIRE(hp != nullptr, "%s: header is null", what);
   const npamd_sliced_header h = *hp;
   NPAMD_REQUIRE(h.magic == kSlicedMagic && h.version == kSlicedVersion, "%s: not a slice-list header", what);
@@ -478,17 +478,79 @@ extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* c
   NPAMD_REQUIRE(h.n_workgroups >= 1 && h.n_partials >= 1, "%s: bad counts in header", what);
   NPAMD_REQUIRE(ldx >= h.k && ldy >= h.n, "%s: row stride smaller than the row", what);
   if (M == 0) return NPAMD_OK;
-  NPAMD_REQUIRE(x && blob && codebook && workspace && y, "%s: null pointer", what);
+  NPAMD_REQUIRE(x && blob && codebook && y, "%s: null pointer", what);
   NPAMD_REQUIRE(ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(codebook) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(blob) % 16) == 0 &&
-                    (reinterpret_cast<uintptr_t>(workspace) % 16) == 0 &&
                     (reinterpret_cast<uintptr_t>(column_perm) % 16) == 0,
-                "%s: x, column_perm, codebook, blob and workspace must be 16-byte aligned (ldx a multiple of 8)", what);
-  NPAMD_REQUIRE(workspace_bytes >= npamd_vq_sliced_workspace_bytes(&h, M), "%s: workspace of %lld bytes, %lld needed",
-                what, (long long)workspace_bytes, (long long)npamd_vq_sliced_workspace_bytes(&h, M));
+                "%s: x, column_perm, codebook and blob must be 16-byte aligned (ldx a multiple of 8)", what);
+  return NPAMD_OK;
+}
+
+static int run_sliced(const char* what, const void* x, int64_t ldx, const int32_t* column_perm,
+                      const npamd_sliced_header& h, const void* blob, const void* codebook, const float* bias,
+                      void* y, int64_t ldy, int M, int act_dtype, void* workspace, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == NPAMD_BF16)
     return launch_sliced<NPAMD_BF16>(h, (const uint8_t*)blob, x, ldx, codebook, column_perm, bias, y, ldy, M, (float*)workspace, st, what);
   return launch_sliced<NPAMD_F16>(h, (const uint8_t*)blob, x, ldx, codebook, column_perm, bias, y, ldy, M, (float*)workspace, st, what);
+}
+
+extern "C" int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
+                                    const npamd_sliced_header* hp, const void* blob, const void* codebook,
+                                    int codebook_dtype, const float* bias, void* y, int64_t ldy, int M, int act_dtype,
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
+  const char* what = "npamd_vq_gemv_sliced";
+  const int rc = check_sliced_call(what, x, ldx, column_perm, hp, blob, codebook, codebook_dtype, y, ldy, M, act_dtype);
+  if (rc != NPAMD_OK || M == 0) return rc;
+  NPAMD_REQUIRE(workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) % 16) == 0,
+                "%s: workspace must be a 16-byte aligned device pointer", what);
+  NPAMD_REQUIRE(workspace_bytes >= npamd_vq_sliced_workspace_bytes(hp, M), "%s: workspace of %lld bytes, %lld needed",
+                what, (long long)workspace_bytes, (long long)npamd_vq_sliced_workspace_bytes(hp, M));
+  return run_sliced(what, x, ldx, column_perm, *hp, blob, codebook, bias, y, ldy, M, act_dtype, workspace, stream);
+}
+
+// ---- the same call for callers that cannot allocate ---------------------------------------
+// The workspace lives in a device array of this library: every GPU the library runs on holds
+// its own copy at its own address, which is looked up once per device, with that device
+// current.  Static storage starts zero-filled, and every call hands the workspace back
+// zero-filled, which is all the kernels ask of it.
+static __device__ __align__(256) unsigned char scratch[NPAMD_SLICED_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_of_device[kMaxDevices];  // the device address of `scratch`, per device (null: not looked up yet)
+}  // namespace
+
+extern "C" int npamd_vq_gemv_sliced_static(const void* x, int64_t ldx, const int32_t* column_perm,
+                                           const npamd_sliced_header* hp, const void* blob, const void* codebook,
+                                           int codebook_dtype, const float* bias, void* y, int64_t ldy, int M,
+                                           int act_dtype, void* stream) {
+  const char* what = "npamd_vq_gemv_sliced_static";
+  const int rc = check_sliced_call(what, x, ldx, column_perm, hp, blob, codebook, codebook_dtype, y, ldy, M, act_dtype);
+  if (rc != NPAMD_OK || M == 0) return rc;
+  const int64_t need = npamd_vq_sliced_workspace_bytes(hp, M);
+  NPAMD_REQUIRE(need <= (int64_t)NPAMD_SLICED_STATIC_WORKSPACE_BYTES,
+                "%s: this layer and token count need %lld bytes of workspace, the built-in one holds %lld "
+                "(use npamd_vq_gemv_sliced with a workspace of your own)",
+                what, (long long)need, (long long)NPAMD_SLICED_STATIC_WORKSPACE_BYTES);
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(NPAMD_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  NPAMD_REQUIRE(device >= 0 && device < kMaxDevices, "%s: device %d outside the %d this library keeps track of", what,
+                device, kMaxDevices);
+  void* workspace = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_of_device[device] == nullptr) {
+      void* ptr = nullptr;
+      e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || ptr == nullptr)
+        return fail(NPAMD_ERR_LAUNCH, "%s: hipGetSymbolAddress: %s", what, hipGetErrorString(e));
+      scratch_of_device[device] = ptr;
+    }
+    workspace = scratch_of_device[device];
+  }
+  return run_sliced(what, x, ldx, column_perm, *hp, blob, codebook, bias, y, ldy, M, act_dtype, workspace, stream);
 }
