@@ -39,15 +39,34 @@ static int env_int(const char* name, int dflt) {
   return (v && *v) ? atoi(v) : dflt;
 }
 
+// The NPAMD_* tuning variables, read once per process (initialisation of a function-local
+// static is thread-safe); launches only read the table.
+const Tuning& tuning() {
+  static const Tuning table = [] {
+    Tuning t;
+    t.gemv_lds_cb = env_int("NPAMD_GEMV_LDS_CB", 1);
+    t.tile_lds_cb = env_int("NPAMD_TILE_LDS_CB", 1);
+    t.gemv_lds_x = env_int("NPAMD_GEMV_LDS_X", 0);
+    t.gemv_r = tuning().gemv_r;
+    t.gemv_spw = tuning().gemv_spw;
+    t.tile_splits = tuning().tile_splits;
+    t.tile_mw = tuning().tile_mw;
+    t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
+    t.q4_rowwise = env_int("NPAMD_Q4_ROWWISE", 1);
+    t.q4_rowwise_bf16 = env_int("NPAMD_Q4_ROWWISE_BF16", 0);
+    return t;
+  }();
+  return table;
+}
+
 static int device_cu_count() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
+  static const int cus = [] {
+    int dev = 0, n = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cus = prop.multiProcessorCount;
-    if (cus <= 0) cus = 256;
-  }
+      n = prop.multiProcessorCount;
+    return n > 0 ? n : 256;
+  }();
   return cus;
 }
 
@@ -55,9 +74,9 @@ static int device_cu_count() {
 // HBM round trip, so the plan aims at every job's packed bytes being requested
 // as soon as the grid starts: jobs per wave is kept near jobs / (16 waves * CUs).
 // NPAMD_GEMV_R / NPAMD_GEMV_SPW override the choice (tuning aid).
-bool gemv_lds_codebook_enabled() { return env_int("NPAMD_GEMV_LDS_CB", 1) != 0; }
-bool tile_lds_codebook_enabled() { return env_int("NPAMD_TILE_LDS_CB", 1) != 0; }
-bool gemv_lds_activations_forced() { return env_int("NPAMD_GEMV_LDS_X", 0) != 0; }
+bool gemv_lds_codebook_enabled() { return tuning().gemv_lds_cb != 0; }
+bool tile_lds_codebook_enabled() { return tuning().tile_lds_cb != 0; }
+bool gemv_lds_activations_forced() { return tuning().gemv_lds_x != 0; }
 
 GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {
   const int steps = (chunks + 3) / 4;
@@ -75,9 +94,9 @@ GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {
   p.R = (tiles * 10 >= cus * 24) ? 4 : (tiles * 10 >= cus * 12) ? 2 : 1;
   if (p.R > max_r) p.R = max_r;
   int spw = (jpw + p.R - 1) / p.R;
-  const int r_env = env_int("NPAMD_GEMV_R", 0);
+  const int r_env = tuning().gemv_r;
   if (r_env == 1 || r_env == 2 || r_env == 4) p.R = r_env;
-  const int spw_env = env_int("NPAMD_GEMV_SPW", 0);
+  const int spw_env = tuning().gemv_spw;
   if (spw_env > 0) spw = spw_env;
   int max_waves = p.R >= 4 ? 8 : 16;
   if (max_waves > max_waves_cap) max_waves = max_waves_cap;
@@ -98,7 +117,7 @@ bool gemv_perm_keeps_occupancy(int M, int N, int chunks, int cb_bytes) {
 }
 
 int plan_tile_splits(int M, int N, int chunks, int mw) {
-  const int env = env_int("NPAMD_TILE_SPLITS", 0);
+  const int env = tuning().tile_splits;
   const int cus = device_cu_count();
   const int blocks = ((N + 63) / 64) * ((M + 128 * mw - 1) / (128 * mw));
   int splits = 1;
@@ -113,7 +132,7 @@ int plan_tile_splits(int M, int N, int chunks, int mw) {
 extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K);
 
 int plan_tile_mw(int M) {
-  const int mw_env = env_int("NPAMD_TILE_MW", 0);
+  const int mw_env = tuning().tile_mw;
   if (mw_env >= 1 && mw_env <= 3) return mw_env;
   const int mw = (M + 127) / 128;
   return mw < 1 ? 1 : (mw > 3 ? 3 : mw);

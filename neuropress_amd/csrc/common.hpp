@@ -29,6 +29,13 @@ void set_error(const char* fmt, ...);
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 
+// Values of the NPAMD_* tuning environment variables, read once per process.
+struct Tuning {
+  int gemv_lds_cb, tile_lds_cb, gemv_lds_x, gemv_r, gemv_spw, tile_splits, tile_mw;
+  int q4_rows, q4_rowwise, q4_rowwise_bf16;
+};
+const Tuning& tuning();
+
 #define NPAMD_REQUIRE(cond, ...)                                  \
   do {                                                            \
     if (!(cond)) return ::npamd::fail(NPAMD_ERR_INVALID, __VA_ARGS__); \

@@ -40,6 +40,8 @@
 // bias, and rounds.
 #pragma once
 
+#include <atomic>
+
 #include "gemv.hpp"
 #include "providers.hpp"
 
@@ -280,6 +282,9 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   }
   const uint32_t xs_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)xs;
   const uint32_t wave_lds = xs_lds + (uint32_t)(wrow0 * XS::kXRowBytes);
+  // The statement writes m0, which the compiler does not let an asm statement declare as
+  // clobbered (a reserved register); it is sound as long as the compiler keeps nothing of its own
+  // in m0 in this kernel, which tests/test_tile_gemm_codegen.py checks on the generated code.
   auto fetch_piece = [&](int i, int buf, const uint8_t* src) {
     const uint32_t dst = __builtin_amdgcn_readfirstlane(wave_lds + (uint32_t)(buf * kXBufBytes + i * 1024));
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -444,14 +449,17 @@ int launch_tile_gemm_mw_cb(const GemmShape& s, const typename Provider::Args& pa
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
   const int lds = XStage<MW, CB_LDS>::kLdsBytes + (CB_LDS ? cb_bytes : 0);
-  static int reserved = 0;  // per instantiation: largest dynamic-LDS size enabled so far
-  if (lds > reserved) {
+  static std::atomic<int> reserved{0};  // per instantiation: largest dynamic-LDS size enabled so far (the
+  // attribute only ever grows; two threads enabling sizes at once both leave it large enough)
+  if (lds > reserved.load(std::memory_order_acquire)) {
     const hipError_t e = hipFuncSetAttribute(
         reinterpret_cast<const void*>(&tile_gemm_kernel<ACT, Provider, MW, CB_LDS>),
         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds,
                                      hipGetErrorString(e));
-    reserved = lds;
+    int seen = reserved.load(std::memory_order_relaxed);
+    while (seen < lds && !reserved.compare_exchange_weak(seen, lds, std::memory_order_release)) {
+    }
   }
   tile_gemm_kernel<ACT, Provider, MW, CB_LDS><<<grid, 512, lds, st>>>(s, pargs);
   if (s.splits > 1) {

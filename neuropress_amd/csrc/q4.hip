@@ -332,10 +332,6 @@ static bool q_fast_ok(const QCall& c) {
 }
 
 
-static int env_flag(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return (v && *v) ? atoi(v) : dflt;
-}
 
 template <int ACT, int M, int R>
 static int launch_q4_rowwise_r(const Q4RowArgs& a, hipStream_t st, const char* what) {
@@ -367,7 +363,7 @@ static int launch_q4_rowwise(const QCall& c) {
     cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
            prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
   }
-  const int r_env = env_flag("NPAMD_Q4_ROWS", 0);
+  const int r_env = tuning().q4_rows;
   const int r = r_env ? r_env : (c.N >= 16 * cus ? 2 : 1);
   if (r >= 4) return launch_q4_rowwise_r<ACT, M, 4>(a, c.st, c.what);
   if (r >= 2) return launch_q4_rowwise_r<ACT, M, 2>(a, c.st, c.what);
@@ -382,8 +378,8 @@ static int launch_q4_rowwise(const QCall& c) {
 // 13.5 vs 13.8 us on 14336 x 4096), x staged in at most 64 KiB of LDS.
 static bool q4_rowwise_ok(const QCall& c) {
   const int passes = (c.K / 32 + 63) / 64;
-  return (c.act == NPAMD_F16 || env_flag("NPAMD_Q4_ROWWISE_BF16", 0) != 0) && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4 * 2) <= 64 * 1024 &&
-         ptr_aligned(c.scale, 2) && env_flag("NPAMD_Q4_ROWWISE", 1) != 0;
+  return (c.act == NPAMD_F16 || tuning().q4_rowwise_bf16 != 0) && c.M == 1 && c.M * passes * (4 * 64 * 16 + 64 * 4 * 2) <= 64 * 1024 &&
+         ptr_aligned(c.scale, 2) && tuning().q4_rowwise != 0;
 }
 
 template <int ACT, bool ASYM>

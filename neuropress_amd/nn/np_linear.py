@@ -256,10 +256,17 @@ class NPLinear(nn.Module):
     def _bias_f32(self) -> torch.Tensor | None:
         if self.bias is None:
             return None
-        b = self._derived.get("bias_f32")
-        if b is None or b.device != self.bias.device:
-            b = self.bias.detach().to(torch.float32).contiguous()
-            self._derived["bias_f32"] = b
+        # Keyed on the buffer's device, address and version counter: load_state_dict or an in-place
+        # copy_ into `bias` makes a new fp32 copy.  Not stored inside a graph capture (a tensor made
+        # there holds data only after a replay).
+        src = self.bias
+        key = (src.device, src.data_ptr(), src._version)
+        hit = self._derived.get("bias_f32")
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        b = src.detach().to(torch.float32).contiguous()
+        if not (src.is_cuda and torch.cuda.is_current_stream_capturing()):
+            self._derived["bias_f32"] = (key, b)
         return b
 
     def _bias_as(self, dtype: torch.dtype) -> torch.Tensor | None:

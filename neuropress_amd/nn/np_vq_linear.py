@@ -48,6 +48,20 @@ from .backends import Backend, VQBackend, is_hip_backend_available, tile_band_ok
 
 log = logging.getLogger(__name__)
 
+_unprepared_warned = False
+
+
+def _warn_unprepared_once() -> None:
+    """One WARNING per process when a layer meant for the slice-list GEMV runs without its lists."""
+    global _unprepared_warned
+    if not _unprepared_warned:
+        _unprepared_warned = True
+        log.warning(
+            "NPVQLinear: a layer with a codebook of more than 4096 rows has no slice lists for its current "
+            "buffers (never prepared, or its indices were reloaded): decode steps run the slower fused GEMV.  "
+            "Call neuropress_amd.prepare_decode(model) once the model is on its GPU."
+        )
+
 
 def _env_int(names: tuple[str, ...], default: int) -> int:
     for name in names:
@@ -509,14 +523,35 @@ class NPVQLinear(nn.Module):
     def is_residual(self) -> bool:
         return self.residual_proxy is not None or self.row_scale is not None or self.row_bias is not None
 
+    def _derive(self, name: str, source: torch.Tensor, build):
+        """``build()`` cached under *name* until *source* moves, is replaced or is written to.
+
+        Every tensor derived from a buffer (a widened index stream, the slice lists, the fp32
+        bias, the int32 permutation) is keyed on the buffer's device, address and version
+        counter, so ``load_state_dict`` or an in-place ``copy_`` into the buffer invalidates it.
+        Inside a graph capture nothing is stored: a tensor made there lives in the graph's
+        private pool and holds data only after a replay, so a later eager call must make its own.
+        """
+        key = (source.device, source.data_ptr(), source._version)
+        hit = self._derived.get(name)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        value = build()
+        if not (source.is_cuda and torch.cuda.is_current_stream_capturing()):
+            self._derived[name] = (key, value)
+        return value
+
+    def _derived_hit(self, name: str, source: torch.Tensor):
+        """The cached value of :meth:`_derive`, or None when it is missing or stale."""
+        hit = self._derived.get(name)
+        if hit is not None and hit[0] == (source.device, source.data_ptr(), source._version):
+            return hit[1]
+        return None
+
     def _bias_f32(self) -> torch.Tensor | None:
         if self.bias is None:
             return None
-        b = self._derived.get("bias_f32")
-        if b is None or b.device != self.bias.device:
-            b = self.bias.detach().to(torch.float32).contiguous()
-            self._derived["bias_f32"] = b
-        return b
+        return self._derive("bias_f32", self.bias, lambda: self.bias.detach().to(torch.float32).contiguous())
 
     def _bias_as(self, dtype: torch.dtype) -> torch.Tensor | None:
         """Bias in the activation dtype for the torch GEMM (``F.linear`` wants one dtype)."""
@@ -533,12 +568,12 @@ class NPVQLinear(nn.Module):
         """
         if self.bits in _FAST_BITS or self.bits > 16:
             return self.packed_indices, self.bits
-        wide = self._derived.get("wide")
-        if wide is None or wide.device != self.packed_indices.device:
-            from .. import kernels
+        from .. import kernels
 
-            wide = kernels.widen_indices_u16(self.packed_indices, self.n_vectors, self.bits)
-            self._derived["wide"] = wide
+        wide = self._derive(
+            "wide", self.packed_indices,
+            lambda: kernels.widen_indices_u16(self.packed_indices, self.n_vectors, self.bits),
+        )  # fmt: skip
         return wide, 16
 
     # ------------------------------------------------------------------
@@ -549,12 +584,10 @@ class NPVQLinear(nn.Module):
         """Band dispatch by token count (reference: neuropress/nn/np_vq_linear.py:1014-1058)."""
         if self.backend in _FUSED_BACKENDS and x.dtype in (torch.float16, torch.bfloat16):
             m = x.numel() // self.in_features
-            if (
-                m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend))
-                and self._sliced_ready(x)
-                and m <= self._derived.get("sliced_max_tokens", _SLICED_MAX_TOKENS)
-            ):
-                return self._forward_sliced(x)  # applies column_perm inside the kernel
+            if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and x.is_cuda:
+                sliced = self._sliced_for(m)
+                if sliced is not None:
+                    return self._forward_sliced(x, sliced)  # applies column_perm inside the kernel
             if self.column_perm is not None and self._perm_fusable(x, m):
                 return self._fused(x, tile=False, perm=self._perm_i32(x.device))
         if self.column_perm is not None:
@@ -600,23 +633,46 @@ class NPVQLinear(nn.Module):
     def prepare_sliced(self) -> bool:
         """Build the slice-list form of the indices for the module's current device.
 
-        Called lazily by the first forward of at most ``_SLICED_MAX_TOKENS`` tokens; call it yourself before
-        capturing a HIP graph (the build copies the stream to the host and back).
-        Returns False when the layer does not use the path.
+        Host work (the stream is copied to the host, re-laid there and uploaded; then both decode
+        GEMVs are timed on the layer's own indices), so it is never done by ``forward``: call it --
+        or :func:`neuropress_amd.prepare_decode` for a whole model -- after the module has reached
+        its GPU and before the first decode step or graph capture.  Returns False when the layer
+        does not use the path.
         """
         if not (self._sliced_eligible() and self.packed_indices.is_cuda):
             return False
-        sl = self._derived.get("sliced")
-        if sl is None or sl.blob.device != self.packed_indices.device:
-            from .. import kernels
-
-            sl = kernels.vq_slice_indices(
-                self.packed_indices, self.bits, self.out_features, self.in_features,
-                self.vector_len, self.proxy.num_centroids,
-            )  # fmt: skip
-            self._derived["sliced"] = sl
-            self._derived["sliced_max_tokens"] = self._sliced_token_limit(sl)
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("NPVQLinear.prepare_sliced() copies to the host and back: call it before the capture")
+        self._derive("sliced", self.packed_indices, self._build_sliced)
+        self.prepare()
         return True
+
+    def prepare(self) -> None:
+        """Make every tensor the kernels derive from the module's buffers (widened index stream,
+        fp32 bias, int32 permutation, the codebook in the usual activation dtypes) for the current
+        device, so that a first call inside a graph capture finds them."""
+        if not self.packed_indices.is_cuda:
+            return
+        self._kernel_stream()
+        self._bias_f32()
+        if self.column_perm is not None:
+            self._perm_i32(self.packed_indices.device)
+        for dtype in (torch.float16, torch.bfloat16):
+            self.proxy.centroids_as(dtype)
+        if self.is_residual:
+            self._res_stream()
+            self._res_centroids()
+
+    def _build_sliced(self):
+        """(slice lists, most tokens for which they beat the fused GEMV on this layer)."""
+        from .. import kernels
+
+        sl = kernels.vq_slice_indices(
+            self.packed_indices, self.bits, self.out_features, self.in_features,
+            self.vector_len, self.proxy.num_centroids,
+        )  # fmt: skip
+        kernels.sliced_workspace(sl.blob.device, sl.workspace_bytes(_SLICED_MAX_TOKENS))
+        return sl, self._sliced_token_limit(sl)
 
     def _sliced_token_limit(self, sl) -> int:
         """Most tokens for which this layer's slice-list GEMV beats its fused GEMV.
@@ -625,10 +681,9 @@ class NPVQLinear(nn.Module):
         ``_SLICED_MAX_TOKENS`` by a wide margin.  A skewed index distribution (one codebook
         slice holding most of the indices) does two things: the hot slice's workgroups
         carry more of the work, or outnumber the compute units, and the fused GEMV's
-        lookups start hitting in L1.  Which one wins then depends on the layer (14336 x
-        4096, Zipf(0.7) / Zipf(1.1): one token 15.5 vs 30 / 17 vs 15 us, four tokens 29 vs
-        30 / 29 vs 16 us; 4096 x 4096, Zipf(1.1): 8.1 vs 5.7 us), so every layer of the
-        size the path is meant for is timed here, once, when its lists are built."""
+        lookups start hitting in L1.  Which one wins then depends on the layer, so every
+        layer of the size the path is meant for is timed here, once, when its lists are
+        built (by ``prepare_sliced``, never by ``forward``)."""
         if self.n_vectors < _SLICED_TUNE_MIN_INDICES:
             return _SLICED_MAX_TOKENS
         dev = sl.blob.device
@@ -665,7 +720,8 @@ class NPVQLinear(nn.Module):
                 if m > _SLICED_MAX_TOKENS:
                     break
                 x = torch.ones(m, self.in_features, dtype=dt, device=dev)
-                t_sliced = timed(lambda: kernels.vq_linear_sliced(x, sl, cb))
+                ws = torch.zeros(sl.workspace_bytes(m) // 4, dtype=torch.float32, device=dev)
+                t_sliced = timed(lambda: kernels.vq_linear_sliced(x, sl, cb, workspace=ws))
                 t_fused = timed(lambda: kernels.vq_linear(x, stream, cb, bits, self.vector_len, None, self.out_features))
                 if t_sliced >= t_fused:
                     break
@@ -675,23 +731,25 @@ class NPVQLinear(nn.Module):
             return _SLICED_MAX_TOKENS
         return limit
 
-    def _sliced_ready(self, x: torch.Tensor) -> bool:
-        if not (x.is_cuda and self._sliced_eligible()):
-            return False
-        sl = self._derived.get("sliced")
-        if sl is not None and sl.blob.device == x.device:
-            return True
-        if torch.cuda.is_current_stream_capturing():
-            return False  # no host work inside a capture: the fused GEMV runs instead
-        return self.prepare_sliced()
+    def _sliced_for(self, m: int):
+        """The slice lists when they exist for the buffer as it is now and win at *m* tokens, else None.
+
+        A lookup only: an eligible layer whose lists were never built (or whose indices were
+        reloaded since) runs the fused GEMV, and says so once."""
+        hit = self._derived_hit("sliced", self.packed_indices)
+        if hit is None:
+            if self._sliced_eligible():
+                _warn_unprepared_once()
+            return None
+        sl, limit = hit
+        return sl if m <= limit else None
 
     def _perm_i32(self, device: torch.device) -> torch.Tensor:
         """``column_perm`` as the int32 device tensor the kernels read (cached)."""
-        perm = self._derived.get("perm_i32")
-        if perm is None or perm.device != device:
-            perm = self.column_perm.to(device=device, dtype=torch.int32).contiguous()
-            self._derived["perm_i32"] = perm
-        return perm
+        return self._derive(
+            "perm_i32", self.column_perm,
+            lambda: self.column_perm.to(device=device, dtype=torch.int32).contiguous(),
+        )  # fmt: skip
 
     def _gemv_max_tokens(self, m: int) -> int:
         """End of band (a) for a call of *m* tokens: the fused limit, or 32 while x stays small."""
@@ -705,23 +763,23 @@ class NPVQLinear(nn.Module):
         """Whether the fused GEMV gathers ``x[..., column_perm]`` itself for this call."""
         if not x.is_cuda or self.is_residual or m > min(_fused_max_tokens(self.backend), 16):
             return False
-        if "perm_i32" not in self._derived and torch.cuda.is_current_stream_capturing():
-            return False  # the int32 copy is made outside a capture
+        if self.bits > 16 or not self._mfma_layer():
+            return False  # index widths the fused kernel does not stream (codebooks beyond 65536 rows)
         from .. import kernels
 
-        bits = self.bits if self.bits in _FAST_BITS else 16
+        bits = self.bits if self.bits in _FAST_BITS else 16  # as _kernel_stream
         return kernels.vq_linear_perm_supported(
             m, self.out_features, self.in_features, self.proxy.num_centroids, self.vector_len, bits
         )
 
-    def _forward_sliced(self, x: torch.Tensor) -> torch.Tensor:
+    def _forward_sliced(self, x: torch.Tensor, sliced) -> torch.Tensor:
         from .. import kernels
 
         *leading, _ = x.shape
         perm = self._perm_i32(x.device) if self.column_perm is not None else None
         try:
             y = kernels.vq_linear_sliced(
-                x.reshape(-1, self.in_features), self._derived["sliced"],
+                x.reshape(-1, self.in_features), sliced,
                 self.proxy.centroids_as(x.dtype), self._bias_f32(), column_perm=perm,
             )  # fmt: skip
         except RuntimeError as exc:
@@ -843,11 +901,8 @@ class NPVQLinear(nn.Module):
     def _res_stream(self) -> torch.Tensor:
         if self.packed_residual is not None:
             return self.packed_residual
-        z = self._derived.get("zero_res")
-        if z is None or z.device != self.packed_indices.device:
-            z = torch.zeros(self.n_vectors, dtype=torch.uint8, device=self.packed_indices.device)
-            self._derived["zero_res"] = z
-        return z
+        dev = self.packed_indices.device
+        return self._derive("zero_res", self.packed_indices, lambda: torch.zeros(self.n_vectors, dtype=torch.uint8, device=dev))
 
     def _res_bits(self) -> int:
         return self.residual_bits if self.packed_residual is not None else 8
@@ -855,13 +910,10 @@ class NPVQLinear(nn.Module):
     def _res_centroids(self) -> torch.Tensor:
         if self.residual_proxy is not None:
             return self.residual_proxy.centroids
-        z = self._derived.get("zero_cb")
-        if z is None or z.device != self.packed_indices.device:
-            z = torch.zeros(
-                (1, self.vector_len), dtype=torch.float16, device=self.packed_indices.device
-            )
-            self._derived["zero_cb"] = z
-        return z
+        dev = self.packed_indices.device
+        return self._derive(
+            "zero_cb", self.packed_indices, lambda: torch.zeros((1, self.vector_len), dtype=torch.float16, device=dev)
+        )
 
     def _fused(self, x: torch.Tensor, tile: bool, perm: torch.Tensor | None = None) -> torch.Tensor:
         from .. import kernels

@@ -12,9 +12,9 @@
  * Pinning status (what fixes each function independently of this file):
  *   np_oracle_unpack_indices / pack_indices  -- reference KAT [3,11]@4 bits ->
  *       0xB3, byte count ceil(n*b/8), max-index and odd-count round trips,
- *       and an independent big-integer packer (tests/test_oracle_packing.py).
+ *       and an independent big-integer packer (tests/test_oracle.py).
  *   np_oracle_vq_decode   -- numpy fancy indexing + torch .to(dtype)
- *       (tests/test_oracle_decode.py); dtype rule = IEEE RNE.
+ *       (tests/test_oracle.py); dtype rule = IEEE RNE.
  *   np_oracle_q_decode    -- closed form (q - zp) * scale, reference KAT
  *       code 15, zp 2, scale 1 -> 13 and underflowed block -> 0.
  *   np_oracle_rvq_decode  -- PARITY UNPINNED by the reference (it has no

@@ -149,7 +149,7 @@ def test_skewed_layers_time_the_sliced_gemv_against_the_fused_one(gpu):
         packed = idx.to(torch.int32).to(torch.int16).view(torch.uint8)
         layer = NPVQLinear(VQProxy(cb).to(gpu), packed, 16, n, k, 8, "cuda_wmma").to(gpu)
         assert layer.prepare_sliced()
-        limits[name] = layer._derived["sliced_max_tokens"]
+        limits[name] = layer._derived_hit("sliced", layer.packed_indices)[1]
         w = cb[idx].reshape(n, k).float()
         for m in (1, 4):
             _close(layer(x[:m].to(gpu)), x[:m].float() @ w.T)
@@ -236,7 +236,7 @@ def test_column_perm_is_folded_into_the_fused_gemv(gpu, act, monkeypatch):
         x = torch.randn(m, k, generator=cases.gen(m)).to(act)
         _close(layer(x.to(gpu)), torch.nn.functional.linear(x[:, perm].float(), w, L["bias"].float()))
     assert seen == [True, True, True]
-    assert layer._derived["perm_i32"].dtype == torch.int32
+    assert layer._perm_i32(gpu).dtype == torch.int32
 
 
 @pytest.mark.parametrize("kind", ["tiered", "ntier", "zero_escape"])
@@ -262,6 +262,9 @@ def test_prefix_coded_layers_run_the_hip_bands(gpu, kind, monkeypatch):
     model.to(gpu)
     AutoKernelLowering().apply(model)
     model.to(gpu)  # the weight container is not a parameter: the lowered module's buffers move here
+    import neuropress_amd
+
+    neuropress_amd.prepare_decode(model)  # slice lists for the buffers where they are now
     layer = model[0]
     assert layer.backend.value == {"tiered": "cuda_tiered", "ntier": "cuda_ntier", "zero_escape": "cuda_zero_escape"}[kind]
     assert layer.bits == 15 and layer.packed_indices.is_cuda

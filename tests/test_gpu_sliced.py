@@ -172,6 +172,7 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
     L = cases.vq_layer(41, n, k, nc, act=act, m=9, bias=True, std=0.05)
     proxy = mod.VQProxy(L["cb"]).to(gpu)
     layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], n, k, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
+    assert layer.prepare_sliced()  # forward never builds the lists itself
     calls = []
     real = kernels.vq_linear_sliced
     monkeypatch.setattr(kernels, "vq_linear_sliced", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
@@ -187,7 +188,6 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
     _check(y7, ref[:7])
     _check(y9, ref)
     # Graph capture: no host work may happen inside; the lists already exist.
-    assert layer.prepare_sliced()
     static_x = x[:1].clone()
     s = torch.cuda.Stream()
     with torch.cuda.stream(s):
@@ -203,27 +203,93 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
         assert torch.equal(static_y, layer(x[i : i + 1]))
 
 
-def test_module_without_prepared_lists_inside_capture_uses_fused_gemv(gpu, monkeypatch):
+def test_forward_never_builds_slice_lists(gpu, monkeypatch, caplog):
+    """An eligible layer that was not prepared runs the fused GEMV -- eagerly and when its very
+    first call is inside a graph capture -- without any host work (no build, no device-to-host
+    copy), and says so once; after prepare_sliced() the same calls take the slice lists."""
+    import logging
+
+    from neuropress_amd import kernels
     from neuropress_amd.nn import np_vq_linear as mod
 
     monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
-    L = cases.vq_layer(42, 128, 256, 20000, act=torch.float16, m=1, std=0.05)
+    monkeypatch.setattr(mod, "_unprepared_warned", False)
+    L = cases.vq_layer(42, 128, 256, 20000, bits=15, act=torch.float16, m=1, bias=True, std=0.05)  # 15 bits: widened stream
     proxy = mod.VQProxy(L["cb"]).to(gpu)
-    layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], 128, 256, 8, "cuda_wmma").to(gpu)
+    layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], 128, 256, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
     x = L["x"].to(gpu)
+
+    def no_build(*a, **kw):
+        raise AssertionError("forward() must not build slice lists")
+
+    monkeypatch.setattr(kernels, "vq_slice_indices", no_build)
+    caplog.set_level(logging.WARNING, logger=mod.__name__)
+    # First call of the module inside the capture: nothing it derives may be cached from there.
     s = torch.cuda.Stream()
     with torch.cuda.stream(s):
-        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 0)
-        layer(x)  # warm the fused path outside the capture
-        monkeypatch.setattr(mod, "_SLICED_MAX_TOKENS", 7)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=s):
             y = layer(x)
+    assert layer._derived_hit("sliced", layer.packed_indices) is None
+    assert not any(isinstance(v, tuple) for v in layer._derived.values())  # no tensor made inside the capture was kept
+    eager_before_replay = layer(x)  # must not read tensors that only exist inside the graph
     graph.replay()
     torch.cuda.synchronize()
-    assert "sliced" not in layer._derived
-    assert torch.equal(y, layer(x)) or (y.float() - layer(x).float()).abs().max().item() < 1e-2
+    assert torch.equal(y, eager_before_replay)
+    layer(x)
+    assert sum("prepare_decode" in r.getMessage() for r in caplog.records) == 1
+    monkeypatch.undo()
+    monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    assert layer.prepare_sliced()
+    seen = []
+    real = kernels.vq_linear_sliced
+    monkeypatch.setattr(kernels, "vq_linear_sliced", lambda *a, **kw: (seen.append(1), real(*a, **kw))[1])
+    y2 = layer(x)
+    assert seen == [1]
+    assert (y2.float() - y.float()).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("m", [1, 16, 64])
+def test_reloaded_buffers_invalidate_everything_derived_from_them(gpu, oracle_lib, monkeypatch, m):
+    """load_state_dict (an in-place copy into packed_indices and bias) after a first forward: the
+    slice lists, the widened stream and the fp32 bias made from the old buffers must not be
+    used again -- every band has to compute with the new indices and bias."""
+    from neuropress_amd.nn import np_vq_linear as mod
+
+    monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    act = torch.float16
+    n, k, nc = 192, 512, 20000
+    A = cases.vq_layer(71, n, k, nc, bits=15, act=act, m=m, bias=True, std=0.05)
+    B = cases.vq_layer(72, n, k, nc, bits=15, act=act, m=m, bias=True, std=0.05)
+    layer = mod.NPVQLinear(mod.VQProxy(A["cb"]).to(gpu), A["packed"], 15, n, k, 8, "cuda_wmma",
+                           bias=A["bias"].float()).to(gpu)
+    layer.prepare_sliced()
+    x = A["x"].to(gpu)
+    _check(layer(x), _vq_ref(oracle_lib, A, act))
+    state = {"packed_indices": B["packed"], "bias": B["bias"].float()}
+    layer.load_state_dict(state, strict=False)
+    Bx = dict(B, x=A["x"], cb=A["cb"])
+    _check(layer(x), _vq_ref(oracle_lib, Bx, act))  # unprepared: the fused paths, new buffers
+    layer.prepare_sliced()
+    _check(layer(x), _vq_ref(oracle_lib, Bx, act))  # and through the rebuilt lists at m <= 7
+
+
+@pytest.mark.parametrize("m", [1, 12])
+def test_column_permutation_with_indices_wider_than_16_bits(gpu, oracle_lib, m):
+    """A codebook of 70000 rows has 17-bit indices, which the fused GEMV with the permutation
+    folded in does not stream: the layer must permute with torch and take decode + GEMM, not fail."""
+    from neuropress_amd.nn import np_vq_linear as mod
+
+    act = torch.float16
+    n, k, nc = 64, 256, 70000
+    L = cases.vq_layer(81, n, k, nc, act=act, m=m, bias=True, std=0.05)
+    assert L["bits"] == 17
+    perm = torch.randperm(k, generator=cases.gen(82))
+    layer = mod.NPVQLinear(mod.VQProxy(L["cb"]).to(gpu), L["packed"], 17, n, k, 8, "cuda_wmma",
+                           bias=L["bias"].float(), column_perm=perm).to(gpu)
+    y = layer(L["x"].to(gpu))
+    _check(y, _vq_ref(oracle_lib, dict(L, x=L["x"][:, perm].contiguous()), act))
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
@@ -241,6 +307,7 @@ def test_column_permutation_is_applied_inside_the_sliced_kernel(gpu, oracle_lib,
     perm = torch.randperm(k, generator=cases.gen(52))
     layer = mod.NPVQLinear(mod.VQProxy(L["cb"]).to(gpu), L["packed"], L["bits"], n, k, 8, "cuda_wmma",
                            bias=L["bias"].float(), column_perm=perm).to(gpu)
+    assert layer.prepare_sliced()
     seen = []
     real = kernels.vq_linear_sliced
     monkeypatch.setattr(kernels, "vq_linear_sliced",
@@ -265,4 +332,5 @@ def test_prepare_decode_builds_the_lists_of_every_eligible_layer(gpu, monkeypatc
     assert neuropress_amd.prepare_decode(model) == 0  # still on the CPU
     model.to(gpu)
     assert neuropress_amd.prepare_decode(model) == 1
-    assert "sliced" in model[0]._derived and "sliced" not in model[1]._derived
+    assert model[0]._derived_hit("sliced", model[0].packed_indices) is not None
+    assert "sliced" not in model[1]._derived

@@ -19,9 +19,13 @@ import pytest
 from neuropress_amd import build
 
 
-def _assembly(tmp_path):
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    """The gfx950 assembly of the VQ tile GEMM, compiled once for the tests of this file."""
+    if shutil.which("hipcc") is None and not build.Path("/opt/rocm/bin/hipcc").exists():
+        pytest.skip("needs hipcc")
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    out = tmp_path / "vq_gemm.s"
+    out = tmp_path_factory.mktemp("codegen") / "vq_gemm.s"
     cmd = [hipcc, *build.CXXFLAGS, *build.DEVICE_FLAGS, "-S", "--cuda-device-only",
            str(build.CSRC / "vq_gemm.hip"), "-o", str(out)]  # fmt: skip
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -29,10 +33,8 @@ def _assembly(tmp_path):
     return out.read_text().split("\n")
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None and not build.Path("/opt/rocm/bin/hipcc").exists(),
-                    reason="needs hipcc")  # fmt: skip
-def test_relaxed_step_barriers_follow_stores_then_lookups(tmp_path):
-    lines = _assembly(tmp_path)
+def test_relaxed_step_barriers_follow_stores_then_lookups(assembly):
+    lines = assembly
     starts = [i for i, ln in enumerate(lines) if re.match(r"^_ZN5npamd16tile_gemm_kernel\S*: ;", ln)]
     assert len(starts) >= 100  # every (activation, width, vector length, tokens band, LDS) instantiation
     kernels_with_relaxed, relaxed = 0, 0
@@ -64,3 +66,26 @@ def test_relaxed_step_barriers_follow_stores_then_lookups(tmp_path):
             kernels_with_relaxed += 1
             relaxed += found
     assert kernels_with_relaxed >= 40 and relaxed == 8 * kernels_with_relaxed
+
+
+def test_nothing_but_the_lds_direct_loads_touches_m0(assembly):
+    """The x tile is fetched with ``s_mov_b32 m0, <LDS address>; global_load_lds_dwordx4`` in an asm
+    statement that cannot declare m0 as clobbered (the compiler reserves it).  That is sound only
+    while the compiler itself keeps nothing in m0 inside ``tile_gemm_kernel``: every instruction of
+    the generated kernels that names m0 must sit inside one of those asm statements."""
+    lines = assembly
+    starts = [i for i, ln in enumerate(lines) if re.match(r"^_ZN5npamd16tile_gemm_kernel\S*: ;", ln)]
+    assert starts
+    checked = 0
+    for i in starts:
+        end = next(j for j in range(i, len(lines)) if lines[j].startswith(".Lfunc_end"))
+        in_asm = False
+        for ln in lines[i:end]:
+            if "#ASMSTART" in ln:
+                in_asm = True
+            elif "#ASMEND" in ln:
+                in_asm = False
+            elif re.search(r"\bm0\b", ln.split(";")[0]):
+                assert in_asm, ln
+                checked += 1
+    assert checked > 0
