@@ -130,6 +130,17 @@ int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K);
 int npamd_vq_widen_u16(const uint8_t* packed, int64_t n_bytes, int bits,
                        int64_t n_indices, uint16_t* out, void* stream);
 
+/*
+ * Gather phase of the look-up-table formulation: y[m, j] = sum_g lut[m, g, idx(j, g)] in float32,
+ * where the caller built lut[m, g, c] = x[m, g*VL:(g+1)*VL] . codebook[c] with one matrix product.
+ * Replaces vq_lut_gather (neuropress/kernels/__init__.py:405-433, kernels/vq_linear_lut.cu:121-142).
+ * lut: f32 [M, groups, NC]; y: f32 [M, N]; bits in [4, 20]; indices beyond NC - 1 are clamped.
+ * The modules do not use this path (the table is M * K/VL * NC floats: 128 MiB per token for a
+ * 4096-wide layer with 65536 codebook rows); it is kept for callers of the reference's wrapper.
+ */
+int npamd_vq_lut_gather(const float* lut, const uint8_t* packed, int64_t n_bytes, int bits,
+                        float* y, int M, int N, int groups, int nc, void* stream);
+
 /* ------------------------------------- slice-list form of the indices ---- */
 /*
  * For codebooks too large for a compute unit's LDS (more than 4096 rows) the
@@ -374,7 +385,12 @@ int npamd_q_embedding(const int64_t* ids, int64_t n_ids, const uint8_t* w_pack,
  *   one 16-byte row of `table16` per index (index masked to `table_entries`, a
  *   power of two), from global memory or, with from_lds != 0, from an LDS copy
  *   of the table (at most 8192 rows).
+ *
+ * npamd_diag_reload_tuning: the NPAMD_* tuning environment variables are read once, at the first
+ *   launch; this reads them again.  For tests and tuning runs only: it must not run while
+ *   another thread launches.
  */
+void npamd_diag_reload_tuning(void);
 int npamd_diag_stream_read(const void* src, int64_t n_bytes, void* sink16, void* stream);
 int npamd_diag_gather(const void* idx_u16, int64_t n_indices, const void* table16,
                       int table_entries, int from_lds, void* sink16, void* stream);

@@ -36,6 +36,7 @@ SIGNATURES: dict[str, list] = {
     "npamd_vq_gemm_tile": _VQ_LINEAR[:-1] + _WS + [_vp],
     "npamd_gemm_tile_workspace_bytes": [_int, _int, _int],
     "npamd_vq_widen_u16": [_vp, _i64, _int, _i64, _vp, _vp],
+    "npamd_vq_lut_gather": [_vp, _vp, _i64, _int, _vp, _int, _int, _int, _int, _vp],
     "npamd_vq_sliced_build": [_vp, _i64, _int, _int, _int, _int, _int, _int, _vp, _i64,
                               ctypes.POINTER(_i64)],  # fmt: skip
     "npamd_vq_sliced_check": [_vp, _i64],
@@ -56,11 +57,13 @@ SIGNATURES: dict[str, list] = {
     "npamd_vq_embedding": [_vp, _i64, _vp, _i64, _int, _vp, _int, _int, _vp, ctypes.c_float, _vp, _int, _vp],
     "npamd_q_embedding": [_vp, _i64, _vp, _vp, _vp, _int, _int, _i64, _int, _i64, ctypes.c_float, _vp, _int, _vp],
     "npamd_q_gemm_tile": _Q_LINEAR[:-1] + _WS + [_vp],
+    "npamd_diag_reload_tuning": [],
     "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
     "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],
 }
 
-_RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64, "npamd_gemm_tile_workspace_bytes": _i64}
+_RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64, "npamd_gemm_tile_workspace_bytes": _i64,
+             "npamd_diag_reload_tuning": None}
 SLICED_HEADER_BYTES = 128
 SLICED_STATIC_WORKSPACE_BYTES = 4 * 1024 * 1024
 

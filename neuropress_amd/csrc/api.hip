@@ -40,33 +40,42 @@ static int env_int(const char* name, int dflt) {
 }
 
 // The NPAMD_* tuning variables, read once per process (initialisation of a function-local
-// static is thread-safe); launches only read the table.
-const Tuning& tuning() {
-  static const Tuning table = [] {
-    Tuning t;
-    t.gemv_lds_cb = env_int("NPAMD_GEMV_LDS_CB", 1);
-    t.tile_lds_cb = env_int("NPAMD_TILE_LDS_CB", 1);
-    t.gemv_lds_x = env_int("NPAMD_GEMV_LDS_X", 0);
-    t.gemv_r = tuning().gemv_r;
-    t.gemv_spw = tuning().gemv_spw;
-    t.tile_splits = tuning().tile_splits;
-    t.tile_mw = tuning().tile_mw;
-    t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
-    t.q4_rowwise = env_int("NPAMD_Q4_ROWWISE", 1);
-    t.q4_rowwise_bf16 = env_int("NPAMD_Q4_ROWWISE_BF16", 0);
-    return t;
-  }();
+// static is thread-safe); launches only read the table.  npamd_diag_reload_tuning() reads them
+// again, for tests and tuning runs that change them between launches.
+static Tuning read_tuning() {
+  Tuning t;
+  t.gemv_lds_cb = env_int("NPAMD_GEMV_LDS_CB", 1);
+  t.tile_lds_cb = env_int("NPAMD_TILE_LDS_CB", 1);
+  t.gemv_lds_x = env_int("NPAMD_GEMV_LDS_X", 0);
+  t.gemv_r = env_int("NPAMD_GEMV_R", 0);
+  t.gemv_spw = env_int("NPAMD_GEMV_SPW", 0);
+  t.tile_splits = env_int("NPAMD_TILE_SPLITS", 0);
+  t.tile_mw = env_int("NPAMD_TILE_MW", 0);
+  t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
+  t.q4_rowwise = env_int("NPAMD_Q4_ROWWISE", 1);
+  t.q4_rowwise_bf16 = env_int("NPAMD_Q4_ROWWISE_BF16", 0);
+  return t;
+}
+
+static Tuning& tuning_table() {
+  static Tuning table = read_tuning();
   return table;
 }
 
+const Tuning& tuning() { return tuning_table(); }
+
 static int device_cu_count() {
-  static const int cus = [] {
-    int dev = 0, n = 0;
+  // Looked up at most a few times per process (racing first callers all store the same value).
+  static std::atomic<int> cached{0};
+  int cus = cached.load(std::memory_order_relaxed);
+  if (cus == 0) {
+    int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      n = prop.multiProcessorCount;
-    return n > 0 ? n : 256;
-  }();
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+    cached.store(cus, std::memory_order_relaxed);
+  }
   return cus;
 }
 
@@ -141,6 +150,8 @@ int plan_tile_mw(int M) {
 }  // namespace npamd
 
 extern "C" int npamd_version(void) { return 3; }
+
+extern "C" void npamd_diag_reload_tuning(void) { npamd::tuning_table() = npamd::read_tuning(); }
 
 extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K < 64) return 0;

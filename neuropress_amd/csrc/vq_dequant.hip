@@ -254,6 +254,29 @@ static int launch_vq_dequant(const uint8_t* packed, int64_t n_bytes, int bits, c
   return check_launch("npamd_vq_dequant");
 }
 
+// LUT gather: y[m, j] = sum over groups g of lut[m, g, idx(j, g)], float32.
+// One wave per output row j: lane l takes groups l, l + 64, ... (consecutive indices of the
+// stream), the 64 partial sums are added pairwise across the wave in a fixed order.
+// blockIdx.y = token.
+__global__ void __launch_bounds__(256) vq_lut_gather_kernel(const float* __restrict__ lut,
+                                                             const uint8_t* __restrict__ packed, int64_t n_bytes,
+                                                             int bits, float* __restrict__ y, int N, int groups,
+                                                             int nc) {
+  const int lane = threadIdx.x & 63;
+  const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (j >= N) return;
+  const float* lut_m = lut + (int64_t)blockIdx.y * groups * nc;
+  float acc = 0.f;
+  for (int g = lane; g < groups; g += 64) {
+    uint32_t c = read_index(packed, n_bytes, (int64_t)j * groups + g, bits);
+    if (c > (uint32_t)nc - 1u) c = (uint32_t)nc - 1u;  // same clamp as the decode kernels
+    acc += lut_m[(int64_t)g * nc + c];
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (lane == 0) y[(int64_t)blockIdx.y * N + j] = acc;
+}
+
 }  // namespace npamd
 
 using namespace npamd;
@@ -289,6 +312,21 @@ extern "C" int npamd_vq_widen_u16(const uint8_t* packed, int64_t n_bytes, int bi
   const unsigned blocks = (unsigned)((n_indices + 255) / 256);
   vq_widen_u16_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(packed, n_bytes, bits, n_indices, out);
   return check_launch("npamd_vq_widen_u16");
+}
+
+extern "C" int npamd_vq_lut_gather(const float* lut, const uint8_t* packed, int64_t n_bytes, int bits,
+                                   float* y, int M, int N, int groups, int nc, void* stream) {
+  const char* what = "npamd_vq_lut_gather";
+  NPAMD_REQUIRE(bits >= 4 && bits <= 20, "%s: bits must be in [4, 20], got %d", what, bits);
+  NPAMD_REQUIRE(M >= 0 && N >= 0 && groups >= 1 && nc >= 1, "%s: bad shape M=%d N=%d groups=%d NC=%d", what, M, N,
+                groups, nc);
+  NPAMD_REQUIRE(((int64_t)N * groups * bits + 7) / 8 <= n_bytes, "%s: packed buffer too short", what);
+  NPAMD_REQUIRE(M <= 65535, "%s: at most 65535 tokens per call (got %d)", what, M);
+  if (M == 0 || N == 0) return NPAMD_OK;
+  NPAMD_REQUIRE(lut && packed && y, "%s: null pointer", what);
+  const dim3 grid((unsigned)((N + 3) / 4), (unsigned)M);
+  vq_lut_gather_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(lut, packed, n_bytes, bits, y, N, groups, nc);
+  return check_launch(what);
 }
 
 extern "C" int npamd_rvq_dequant(const uint8_t* packed_main, int64_t n_bytes_main, int bits_main,

@@ -517,6 +517,33 @@ def vq_linear_zero_escape(
                             [row_off_zero, row_off_hot, row_off_warm, row_off_cold], centroids, vector_len, bias)
 
 
+def vq_lut_gather(
+    lut: torch.Tensor,
+    packed_indices: torch.Tensor,
+    bits: int,
+    out_features: int,
+) -> torch.Tensor:
+    """LUT gather phase: ``y[m, j] = sum_g lut[m, g, idx[j, g]]`` (``npamd_vq_lut_gather``).
+
+    Same signature as the reference's wrapper (neuropress/kernels/__init__.py:405-433):
+    *lut* is the float32 ``[M, n_groups, NC]`` table the caller built as
+    ``(x.reshape(M * n_groups, VL) @ centroids.T).reshape(M, n_groups, NC)``, the index of
+    output ``j``, group ``g`` sits at position ``j * n_groups + g`` of the bit-stream;
+    returns float32 ``[M, N]``.
+    """
+    what = "vq_lut_gather"
+    _check_device(what, lut, packed_indices)
+    if lut.dim() != 3 or lut.dtype != torch.float32:
+        raise RuntimeError(f"{what}: lut must be a float32 [M, n_groups, NC] tensor, got {lut.dtype} {tuple(lut.shape)}")
+    lut = lut.contiguous()
+    packed = _packed_u8(packed_indices, what)
+    m, groups, nc = lut.shape
+    y = torch.empty((m, int(out_features)), device=lut.device, dtype=torch.float32)
+    _lib.call("npamd_vq_lut_gather", lut.data_ptr(), packed.data_ptr(), packed.numel(), int(bits), y.data_ptr(),
+              m, int(out_features), groups, nc, _stream(lut))  # fmt: skip
+    return y
+
+
 def vq_linear_wmma(
     x: torch.Tensor,
     packed_indices: torch.Tensor,

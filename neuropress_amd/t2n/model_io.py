@@ -354,7 +354,8 @@ def load_quantized_model(model: nn.Module, path: str | Path, kernel_lowering: st
     Regular tensors go through ``load_state_dict(strict=False)``; every quantized weight is rebuilt
     from its components and attached to its ``nn.Linear``; with ``kernel_lowering="auto"`` the
     model is then lowered (``AutoKernelLowering``).  Raises ``ValueError`` for a file without a
-    manifest or with a quantized-weight type this backend has no container for.
+    manifest, with a quantized-weight type this backend has no container for, or with a
+    ``mixed_precision_split`` transform (it changes the module tree; not replayed here).
     """
     from safetensors import safe_open
 
@@ -372,8 +373,18 @@ def load_quantized_model(model: nn.Module, path: str | Path, kernel_lowering: st
     manifest_dict = json.loads(manifest_str)
     manifest = QuantizationManifest(transforms=list(manifest_dict.get("transforms", [])))
     for t in manifest.transforms:
-        if t.get("type") not in ("qtensor_assignment",):
-            _log.warning("load_quantized_model: transform %r is not replayed by this backend", t.get("type"))
+        kind = t.get("type")
+        if kind == "mixed_precision_split":
+            # The reference replays this one before load_state_dict (t2n/model_io.py:367-420): it
+            # swaps nn.Linear modules for MixedPrecisionLinear ones whose sub-linears own the saved
+            # tensors.  Loading without it would drop those tensors silently (strict=False).
+            raise ValueError(
+                f"File {str(path)!r} records a 'mixed_precision_split' transform, which replaces the "
+                f"modules at {sorted(t.get('modules', {}))[:4]} ... by split mixed-precision linears; this "
+                "backend has no such module, so the checkpoint cannot be loaded here."
+            )
+        if kind != "qtensor_assignment":
+            _log.warning("load_quantized_model: transform %r is not replayed by this backend", kind)
     entries = manifest._assignment()
 
     regular = {k: v for k, v in all_tensors.items() if _QT_SEP not in k and k not in entries}

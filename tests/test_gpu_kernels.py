@@ -365,9 +365,10 @@ def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
     depends on its row count and the device's size, so every variant is forced here (tuning
     override NPAMD_GEMV_R) on ragged shapes: codebook in LDS, codebook gathered from memory,
     fused column permutation, int4, residual VQ."""
-    from neuropress_amd import kernels
+    from neuropress_amd import _lib, kernels
 
     monkeypatch.setenv("NPAMD_GEMV_R", str(rows))
+    _lib.load().npamd_diag_reload_tuning()  # the library reads its tuning variables once
     n, k = 200, 576  # 12.5 row tiles, 9 chunks of 64
     for bits, nc in ((8, 256), (16, 65536)):
         L = cases.vq_layer(900 + bits + m, n, k, nc, bits=bits, act=torch.bfloat16, m=m, bias=True, std=0.05)
@@ -386,6 +387,8 @@ def test_gemv_row_tiles_per_block(gpu, oracle_lib, monkeypatch, rows, m):
     y = kernels.rvq_linear(R["x"].to(gpu), R["pm"].to(gpu), R["bm"], R["pr"].to(gpu), R["br"], R["cbm"].to(gpu),
                            R["cbr"].to(gpu), R["scale"].to(gpu), R["wbias"].to(gpu), 80, None, tile=False)
     _check(y, _rvq_ref(oracle_lib, R, torch.float16))
+    monkeypatch.delenv("NPAMD_GEMV_R")
+    _lib.load().npamd_diag_reload_tuning()
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
@@ -539,3 +542,28 @@ def test_q4_and_rvq_gemm_tile_split_k(gpu, oracle_lib, m):
     y = kernels.rvq_linear(R["x"].to(gpu), R["pm"].to(gpu), R["bm"], R["pr"].to(gpu), R["br"], R["cbm"].to(gpu),
                            R["cbr"].to(gpu), R["scale"].to(gpu), R["wbias"].to(gpu), 80, None, tile=True)
     _check(y, _rvq_ref(oracle_lib, R, torch.float16))
+
+
+@pytest.mark.parametrize("bits,nc", [(8, 256), (12, 4096), (10, 600), (16, 65536)])
+@pytest.mark.parametrize("m", [1, 3])
+def test_vq_lut_gather_matches_a_float64_gather(gpu, oracle_lib, bits, nc, m):
+    """y[m, j] = sum_g lut[m, g, idx[j, g]] (reference: kernels/vq_linear_lut.cu:121-142), against the
+    same sum taken in float64 over oracle-unpacked indices; and, with the table the reference's
+    caller builds from x and the codebook, against the layer's output."""
+    from neuropress_amd import kernels
+
+    n, k, vl = 70, 8 * 37, 8
+    groups = k // vl
+    L = cases.vq_layer(300 + bits + m, n, k, nc, bits=bits, act=torch.float16, m=m, std=0.05)
+    idx = oracle_lib.unpack_indices(L["packed"].numpy(), bits, n * groups).reshape(n, groups)
+    assert np.array_equal(idx, L["idx"].reshape(n, groups).numpy())
+    lut = (L["x"].float().reshape(m * groups, vl) @ L["cb"].float().T).reshape(m, groups, nc)
+    y = kernels.vq_lut_gather(lut.to(gpu), L["packed"].to(gpu), bits, n)
+    assert y.shape == (m, n) and y.dtype == torch.float32
+    want = np.take_along_axis(lut.double().numpy()[:, None, :, :], idx[None, :, :, None], axis=3)[..., 0].sum(-1)
+    assert np.abs(y.cpu().numpy() - want).max() <= 1e-4
+    code = orc.DT_F16
+    w = oracle_lib.vq_decode(L["packed"].numpy(), bits, orc.to_bits(L["cb"]), n, k, code)
+    ref = oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code)
+    ok, max_abs, _ = cases.within_tol(y.cpu().numpy(), ref)
+    assert ok, max_abs

@@ -183,3 +183,45 @@ def test_load_errors(tmp_path):
         load_quantized_model(Net(), path)
     with pytest.raises(ValueError, match="kernel_lowering must be 'auto' or None"):
         load_quantized_model(Net(), path, kernel_lowering="fast")
+    split = {"format_version": "2", "recipe_config": None, "transforms": [
+        {"type": "mixed_precision_split", "modules": {"vq_a": {"out_features": 48, "split_sizes": [32, 32]}}}]}
+    save_file({"w": torch.zeros(2)}, str(path), metadata={"__neuropress_manifest__": json.dumps(split)})
+    with pytest.raises(ValueError, match="mixed_precision_split"):  # changes the module tree: refused, not skipped
+        load_quantized_model(Net(), path)
+
+
+@pytest.mark.gpu
+def test_checkpoint_loaded_onto_the_gpu_runs_the_hip_kernels(tmp_path):
+    """save_quantized_model -> load_quantized_model(kernel_lowering="auto") into a model that lives on
+    the GPU -> forward: every quantized layer computes with the HIP kernels and matches the
+    unlowered model's torch-op forward of the same checkpoint (fp16, 1 and 40 tokens)."""
+    from neuropress_amd import kernels
+
+    gpu = torch.device("cuda:0")
+    src = _quantized_net()
+    attach_manifest(src)
+    path = tmp_path / "net.safetensors"
+    save_quantized_model(src, path)
+    ref = Net()
+    load_quantized_model(ref, path, kernel_lowering=None)
+    AutoKernelLowering(vq_backend="default", linear_backend="compile").apply(ref)  # torch-op paths on the CPU
+    model = Net().half().to(gpu)
+    calls = []
+    patched = {}
+    for name in ("vq_linear", "q_linear", "vq_gemm_tile", "q_gemm_tile", "vq_dequant", "q_dequant"):
+        real = getattr(kernels, name)
+        patched[name] = real
+        setattr(kernels, name, lambda *a, _r=real, _n=name, **kw: (calls.append(_n), _r(*a, **kw))[1])
+    try:
+        load_quantized_model(model, path)  # kernel_lowering="auto"
+        assert is_lowered(model) and model.vq_a.packed_indices.is_cuda and model.q4.u8_blob.is_cuda
+        assert model.vq_a.backend.value.startswith("cuda") and model.q4.backend.value == "cuda"
+        for m in (1, 40):
+            x = torch.randn(m, 64, generator=torch.Generator().manual_seed(m))
+            y = model(x.half().to(gpu)).float().cpu()
+            want = ref.float()(x.half().float())
+            assert (y - want).abs().max().item() <= 1e-2 + 1e-2 * want.abs().max().item()
+    finally:
+        for name, real in patched.items():
+            setattr(kernels, name, real)
+    assert "vq_linear" in calls and "q_linear" in calls  # the HIP entry points did the work
