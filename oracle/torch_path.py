@@ -48,6 +48,26 @@ def unpack_fast(packed: torch.Tensor, bits: int, n_indices: int) -> torch.Tensor
     return unpack_bitloop(packed, bits, n_indices)
 
 
+def vq_decode_cpu(packed, centroids, bits, out_features, in_features, dtype, fast_unpack=True) -> torch.Tensor:
+    """The decode half of :func:`vq_linear_cpu`: unpack, gather codebook rows, cast."""
+    n_vec = out_features * in_features // centroids.shape[1]
+    idx = (unpack_fast if fast_unpack else unpack_bitloop)(packed, bits, n_vec)
+    return centroids[idx].reshape(out_features, in_features).to(dtype)
+
+
+def q_decode_cpu(u8_blob, scale, nbits, group_size, dtype, zero_point=None) -> torch.Tensor:
+    """The decode half of :func:`q_linear_cpu` (neuropress/nn/np_linear.py:333-353)."""
+    vpb = 8 // nbits
+    n, kp = u8_blob.shape
+    k = kp * vpb
+    shifts = torch.arange(vpb, dtype=torch.int32) * nbits
+    vals = ((u8_blob.to(torch.int32).unsqueeze(-1) >> shifts) & ((1 << nbits) - 1)).reshape(n, k)
+    vals_f = vals.to(torch.float32).reshape(n, k // group_size, group_size)
+    sc = scale.to(torch.float32).reshape(n, k // group_size, 1)
+    zp = zero_point.to(torch.float32).reshape(n, k // group_size, 1) if zero_point is not None else float(1 << (nbits - 1))
+    return ((vals_f - zp) * sc).reshape(n, k).to(dtype)
+
+
 def vq_linear_cpu(
     x: torch.Tensor,
     packed: torch.Tensor,
