@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
-    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "tile_m256", "tile_m384", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_tile_m128", "q4_tile_m256", "rvq_gemv_m1", "rvq_tile_m128",
+    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "gemv_cfg2_gateup_m1", "gemv_cfg2_down_m1", "tile_m256", "tile_m384", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_tile_m128", "q4_tile_m256", "rvq_gemv_m1", "rvq_tile_m128",
                                                     "rms_norm_m4096", "vq_embedding_m4096", "q4_embedding_m4096"],
                     help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
                          "on the config-3 / config-5 shape (rvq_*: the config-4 4096x4096 projection) and print a one-line JSON with its HIP-event time")
@@ -228,15 +228,20 @@ def main():
             alg, flops = n * k // 2 + n * k // 32 * 2 + m * k * 2 + m * n * 2, 2.0 * m * n * k
         else:
             nc, bits = (4096, 12) if args.case in ("gemv_nc4096_m1", "tile_nc4096_m128") else (65536, 16)
+            if args.case.startswith("gemv_cfg2"):  # config 2's own layers: 4096-row codebook, int16 stream
+                n, k = (8192, 2048) if args.case == "gemv_cfg2_gateup_m1" else (2048, 8192)
+                nc, bits, n_rot = 4096, 16, 160
             cb = (torch.randn(nc, 8, generator=g) * 0.02).to(torch.float16)
             if bits == 16:
-                base = torch.randint(0, 65536, (n * k // 8,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8)
+                base = torch.randint(0, nc, (n * k // 8,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8)
             else:
                 base = IndexPacking.pack(torch.randint(0, nc, (n * k // 8,), generator=g), bits)
             pool = [base.to(dev).clone() for _ in range(n_rot)]
             cb16, cbb = cb.to(dev), cb.to(torch.bfloat16).to(dev)
             m = 256 if args.case == "tile_m256" else 384 if args.case == "tile_m384" else 128 if args.case == "tile_nc4096_m128" else 1
             x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
+            if args.case.startswith("gemv_cfg2"):
+                x, cbb = x.to(torch.float16), cb16  # config 2 runs in fp16
             if args.case == "sliced_m1":
                 sl0 = kernels.vq_slice_indices(base, bits, n, k, 8, nc, device=dev)
                 n_rot = rot_for(sl0.total_bytes)  # more than L2 + Infinity Cache, as in the main run

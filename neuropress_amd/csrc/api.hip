@@ -54,6 +54,7 @@ static Tuning read_tuning() {
   t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
   t.q4_rowwise = env_int("NPAMD_Q4_ROWWISE", 1);
   t.q4_rowwise_bf16 = env_int("NPAMD_Q4_ROWWISE_BF16", 0);
+  t.q4_stream = env_int("NPAMD_Q4_STREAM", 1);
   return t;
 }
 

@@ -302,6 +302,186 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
     }
 }
 
+// ---------------------------------------------------------------------------
+// One token, whole layer streamed by one resident grid: at most one block per compute unit, no
+// LDS on the way in.  A lane owns two adjacent 32-k groups (32 bytes of a row, 64 values of x),
+// a wave 4096 columns ("pass" p of the row), a block's waves are arranged as (row lane j, pass
+// p).  In iteration `it` the grid contracts rows [it * row_stride, (it + 1) * row_stride), so
+// at any time it reads one contiguous window of the weights.  Every wave keeps its x values (in
+// the (k, k+4) pair order of the decoded nibbles) and their offsets in registers for its whole
+// life; x is requested first, then up to four rows' weights and scales, and each row is
+// contracted as it arrives.  A row's sum is reduced inside the wave with DPP adds and lane
+// reads; with more than one pass the parts meet in LDS and are added in pass order.
+// Same arithmetic as the kernel above (base + q nibbles, group offsets folded out, f32).
+// ---------------------------------------------------------------------------
+constexpr int kQ4StreamMaxWaves = 16;
+
+struct Q4StreamGeom {
+  int passes;           // ceil(K / 4096)
+  int waves;            // per block: row_lanes * passes
+  int row_lanes;        // L: rows a block works on at a time
+  int blocks;
+  int row_stride;       // blocks * L: rows the grid works on at a time
+  int iterations;       // ceil(N / row_stride)
+  int pairs;            // K / 64
+};
+
+struct Q4StreamItem {
+  u32x4 w[2];
+  uint32_t sc, zp;      // two fp16 values each: the lane's two groups
+};
+
+// A lane's two groups are 64 groups apart: each of the two weight loads of a wave covers one
+// contiguous KiB.
+template <bool ASYM>
+__device__ __forceinline__ void q4_stream_load(Q4StreamItem& it, const Q4RowArgs& a, int row, int g0, int g1) {
+  const uint8_t* w = a.w_pack + (int64_t)row * (a.K / 2);
+  it.w[0] = *reinterpret_cast<const u32x4*>(w + (int64_t)g0 * 16);
+  it.w[1] = *reinterpret_cast<const u32x4*>(w + (int64_t)g1 * 16);
+  const int64_t at = (int64_t)row * a.scales_per_row;
+  it.sc = a.scale[at + (g0 >> a.gs_shift)] | ((uint32_t)a.scale[at + (g1 >> a.gs_shift)] << 16);
+  if constexpr (ASYM) it.zp = a.zp[at + (g0 >> a.gs_shift)] | ((uint32_t)a.zp[at + (g1 >> a.gs_shift)] << 16);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+  return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over the 64 lanes, the same value in every lane: four rotations inside each row of 16
+// lanes, then the four row totals are read out and added in lane order.
+__device__ __forceinline__ float wave_total(float v) {
+  v = dpp_add<0x128>(v);  // row_ror:8
+  v = dpp_add<0x124>(v);  // row_ror:4
+  v = dpp_add<0x122>(v);  // row_ror:2
+  v = dpp_add<0x121>(v);  // row_ror:1
+  const int b = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+struct Q4StreamX {
+  u32x4 v[2][4];        // per group: four vectors of (k, k+4) pairs
+  float off[2], sum[2]; // per group: what base + 8 adds to the dot product; plain sum (zero points)
+};
+
+template <int ACT>
+__device__ __forceinline__ float q4_group_dot(const u32x4& w, const u32x4 (&xv)[4], float t) {
+  const uint32_t magic_lo = ACT == NPAMD_BF16 ? 0x43004300u : 0x64006400u, magic_hi = 0x54005400u;
+  const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t u = wd[q], u8 = u >> 8;
+    uint32_t p0, p1, p2, p3;
+    p0 = and_or(u, 0x000F000Fu, magic_lo);
+    p2 = and_or(u8, 0x000F000Fu, magic_lo);
+    if constexpr (ACT == NPAMD_BF16) {
+      p1 = and_or(u >> 4, 0x000F000Fu, magic_lo);
+      p3 = and_or(u >> 12, 0x000F000Fu, magic_lo);
+    } else {
+      p1 = and_or(u, 0x00F000F0u, magic_hi);
+      p3 = and_or(u8, 0x00F000F0u, magic_hi);
+    }
+    t = fdot2_act<ACT>(p0, xv[q].x, t);
+    t = fdot2_act<ACT>(p1, xv[q].y, t);
+    t = fdot2_act<ACT>(p2, xv[q].z, t);
+    t = fdot2_act<ACT>(p3, xv[q].w, t);
+  }
+  return t;
+}
+
+constexpr int kQ4StreamXStride = 80;   // bytes between the x values of two groups in LDS: 64 + 16, so
+                                       // that 16 lanes reading their own piece hit 16 different bank groups
+
+template <int ACT, bool ASYM>
+__device__ __forceinline__ void q4_stream_row(const Q4StreamItem& item, const Q4StreamX& x, bool live0, bool live1,
+                                              float* slot, int lane) {
+  float v = 0.f;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    float t = -x.off[h];
+    if constexpr (ASYM) t = __builtin_fmaf(8.0f - f16_bits_to_f32((item.zp >> (16 * h)) & 0xFFFFu), x.sum[h], t);
+    t = q4_group_dot<ACT>(item.w[h], x.v[h], t);
+    v = __builtin_fmaf((h ? live1 : live0) ? f16_bits_to_f32((item.sc >> (16 * h)) & 0xFFFFu) : 0.f, t, v);
+  }
+  const float total = wave_total(v);
+  // Parked in LDS: the bias load of a store issued here would have to wait for every weight
+  // request of the wave that is still under way (loads return in order).
+  if (lane == 0 && slot) *slot = total;
+}
+
+// The code is kept small on purpose (one row loop, two rows in flight per wave): a kernel that
+// lasts a few microseconds executes every instruction for the first time, and straight-line
+// code for many rows is paced by instruction-cache misses.
+template <int ACT, bool ASYM>
+__global__ void __launch_bounds__(kQ4StreamMaxWaves * 64) q4_stream_gemv_kernel(Q4RowArgs a, Q4StreamGeom geo) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint8_t* xs = smem;  // x: 80 bytes per 32-k group
+  float* part = reinterpret_cast<float*>(smem + geo.passes * 128 * kQ4StreamXStride);  // [iteration][row lane][pass]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int p = wave % geo.passes, j = wave / geo.passes;
+  const bool live0 = p * 128 + lane < a.groups32, live1 = p * 128 + 64 + lane < a.groups32;
+  const int g0 = min(p * 128 + lane, a.groups32 - 1), g1 = min(p * 128 + 64 + lane, a.groups32 - 1);
+  const int row_first = blockIdx.x * geo.row_lanes + j;
+  const int threads = geo.waves * 64, pieces = a.groups32 * 4;
+
+  // x is requested ahead of the weights (loads return in order: behind them it would hold the
+  // first row back) and goes through LDS once per block.
+  u32x4 piece[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+    if (tid + r * threads < pieces) piece[r] = reinterpret_cast<const u32x4*>(a.x)[tid + r * threads];
+  Q4StreamItem cur, nxt;
+  q4_stream_load<ASYM>(cur, a, min(row_first, a.N - 1), g0, g1);
+  q4_stream_load<ASYM>(nxt, a, min(row_first + geo.row_stride, a.N - 1), g0, g1);
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int q = tid + r * threads;
+    if (q < pieces) *reinterpret_cast<u32x4*>(xs + (q >> 2) * kQ4StreamXStride + (q & 3) * 16) = piece[r];
+  }
+  for (int q = tid + 2 * threads; q < pieces; q += threads)  // rows too few to fill the block with waves
+    *reinterpret_cast<u32x4*>(xs + (q >> 2) * kQ4StreamXStride + (q & 3) * 16) = reinterpret_cast<const u32x4*>(a.x)[q];
+  block_sync_lds();
+  Q4StreamX x;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    float sum_even = 0.f, sum_odd = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      x.v[h][q] = permute_a_0415(*reinterpret_cast<const u32x4*>(xs + (h ? g1 : g0) * kQ4StreamXStride + q * 16));
+      const uint32_t d[4] = {x.v[h][q].x, x.v[h][q].y, x.v[h][q].z, x.v[h][q].w};
+      sum_even += act_bits_to_f32<ACT>(d[0] & 0xFFFFu) + act_bits_to_f32<ACT>(d[0] >> 16) +
+                  act_bits_to_f32<ACT>(d[2] & 0xFFFFu) + act_bits_to_f32<ACT>(d[2] >> 16);
+      sum_odd += act_bits_to_f32<ACT>(d[1] & 0xFFFFu) + act_bits_to_f32<ACT>(d[1] >> 16) +
+                 act_bits_to_f32<ACT>(d[3] & 0xFFFFu) + act_bits_to_f32<ACT>(d[3] >> 16);
+    }
+    x.off[h] = ACT == NPAMD_BF16 ? 136.f * (sum_even + sum_odd) : 1032.f * sum_even + 72.f * sum_odd;
+    x.sum[h] = sum_even + sum_odd;
+  }
+
+  // Rows beyond the last iteration are clamped to the last row (cache hits) and not recorded.
+  for (int it = 0; it < geo.iterations; it += 2) {
+    q4_stream_row<ACT, ASYM>(cur, x, live0, live1, part + (it * geo.row_lanes + j) * geo.passes + p, lane);
+    q4_stream_load<ASYM>(cur, a, min(row_first + (it + 2) * geo.row_stride, a.N - 1), g0, g1);
+    q4_stream_row<ACT, ASYM>(nxt, x, live0, live1,
+                             it + 1 < geo.iterations ? part + ((it + 1) * geo.row_lanes + j) * geo.passes + p : nullptr, lane);
+    q4_stream_load<ASYM>(nxt, a, min(row_first + (it + 3) * geo.row_stride, a.N - 1), g0, g1);
+  }
+  __syncthreads();
+  for (int r = tid; r < geo.iterations * geo.row_lanes; r += geo.waves * 64) {
+    const int n = (r / geo.row_lanes) * geo.row_stride + blockIdx.x * geo.row_lanes + r % geo.row_lanes;
+    if (n >= a.N) continue;
+    float total = 0.f;
+    for (int q = 0; q < geo.passes; ++q) total += part[r * geo.passes + q];
+    store_from_f32<ACT>(a.y, n, total + (a.bias ? a.bias[n] : 0.f));
+  }
+}
+
 struct QCall {
   const void* x; int64_t ldx;
   const uint8_t* w_pack; const void* scale; const void* zp;
@@ -370,6 +550,60 @@ static int launch_q4_rowwise(const QCall& c) {
   return launch_q4_rowwise_r<ACT, M, 1>(a, c.st, c.what);
 }
 
+static int device_cus_q4() {
+  static std::atomic<int> cached{0};
+  int cus = cached.load(std::memory_order_relaxed);
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    cached.store(cus, std::memory_order_relaxed);
+  }
+  return cus;
+}
+
+// The resident-grid kernel takes one token of a layer with at most 16 passes (K <= 65536) whose
+// per-block tables fit 64 KiB of LDS, when every block has at least five rows per wave to go
+// through: it then streams at the rate of a plain read (28672 x 4096: 14.6 us against 17.7 us
+// for the kernel above, whose every block restages x), while its longer start (x through LDS
+// before the first row can be contracted, two rows in flight per wave) loses on fewer rows
+// (14336 x 4096: 9.6 us both, 4096 x 4096: 6.4 against 5.2 us).  NPAMD_Q4_STREAM=2 takes it
+// wherever it fits, 0 never.  Blocks are as many as give every block the same number of rows.
+static bool q4_stream_geometry(const QCall& c, Q4StreamGeom& geo) {
+  geo.pairs = c.K / 64;
+  geo.passes = (geo.pairs + 63) / 64;
+  if (c.M != 1 || geo.passes < 1 || geo.passes > kQ4StreamMaxWaves || tuning().q4_stream == 0) return false;
+  geo.row_lanes = kQ4StreamMaxWaves / geo.passes;
+  if (geo.row_lanes > c.N) geo.row_lanes = c.N;
+  const int row_groups = (c.N + geo.row_lanes - 1) / geo.row_lanes;
+  const int cus = device_cus_q4();
+  geo.iterations = (row_groups + cus - 1) / cus;
+  geo.blocks = (row_groups + geo.iterations - 1) / geo.iterations;
+  geo.row_stride = geo.blocks * geo.row_lanes;
+  geo.waves = geo.row_lanes * geo.passes;
+  if (geo.iterations < 5 && tuning().q4_stream < 2) return false;
+  return (int64_t)geo.iterations * geo.row_lanes * geo.passes * 4 + geo.passes * 128 * kQ4StreamXStride <= 64 * 1024;
+}
+
+template <int ACT>
+static int launch_q4_stream(const QCall& c, const Q4StreamGeom& geo) {
+  Q4RowArgs a;
+  a.x = (const uint16_t*)c.x; a.ldx = c.ldx;
+  a.w_pack = c.w_pack; a.scale = (const uint16_t*)c.scale; a.zp = (const uint16_t*)c.zp;
+  a.bias = c.bias; a.y = (uint16_t*)c.y; a.ldy = c.ldy;
+  a.N = c.N; a.K = c.K;
+  a.groups32 = c.K / 32;
+  a.passes = geo.passes;
+  a.scales_per_row = c.K / c.gs;
+  a.gs_shift = log2i(c.gs / 32);
+  const int lds = geo.passes * 128 * kQ4StreamXStride + geo.iterations * geo.row_lanes * geo.passes * 4;
+  const dim3 grid(geo.blocks), block(geo.waves * 64);
+  if (a.zp) q4_stream_gemv_kernel<ACT, true><<<grid, block, lds, c.st>>>(a, geo);
+  else q4_stream_gemv_kernel<ACT, false><<<grid, block, lds, c.st>>>(a, geo);
+  return check_launch(c.what);
+}
+
 // bf16: the row-wise kernel keeps the unrounded weight (q - 8) * s, while the dequant-then-matmul
 // path it is checked against rounds every weight to bf16 (8 bits); at K = 14336 the two differ by
 // up to 4.5e-2, more than the 1e-2 parity bound, so bf16 stays on the MFMA GEMV (which rounds the
@@ -410,7 +644,11 @@ template <int ACT>
 static int q_dispatch(const QCall& c, bool gemv) {
   if (q_fast_ok(c)) {
     if (c.nbits == 8) return c.zp ? q8_fused<ACT, true>(c, gemv) : q8_fused<ACT, false>(c, gemv);
-    if (gemv && q4_rowwise_ok(c)) return launch_q4_rowwise<ACT, 1>(c);
+    if (gemv && q4_rowwise_ok(c)) {
+      Q4StreamGeom geo;
+      if (q4_stream_geometry(c, geo)) return launch_q4_stream<ACT>(c, geo);
+      return launch_q4_rowwise<ACT, 1>(c);
+    }
     return c.zp ? q4_fused<ACT, true>(c, gemv) : q4_fused<ACT, false>(c, gemv);
   }
   const QElem e{c.w_pack, (const uint16_t*)c.scale, (const uint16_t*)c.zp, c.K, c.nbits, c.gs, c.act};

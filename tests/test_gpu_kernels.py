@@ -324,6 +324,35 @@ def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m, asym):
     _check(y, _q_ref(oracle_lib, L, act))
 
 
+@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 128), (4200, 256), (13000, 128),
+                                 (20000, 64)])
+@pytest.mark.parametrize("gs", [32, 64])
+@pytest.mark.parametrize("asym", [False, True])
+def test_q4_stream_gemv(gpu, oracle_lib, monkeypatch, n, k, gs, asym):
+    """The resident-grid int4 GEMV (one fp16 token; taken by itself only for layers with many
+    rows, forced here with NPAMD_Q4_STREAM=2): K of one partial pass, of one and of several whole
+    passes and of a partial last pass; rows fewer than the row lanes of a block; one, two, an even
+    and an odd number of iterations; rows that do not fill the last iteration."""
+    from neuropress_amd import _lib, kernels
+
+    if k % gs:
+        pytest.skip("K not a multiple of the group size")
+    L = cases.q4_layer(800 + n, n, k, gs=gs, act=torch.float16, m=1, bias=True, asym=asym)
+    zp = None if L["zp"] is None else L["zp"].to(gpu)
+    monkeypatch.setenv("NPAMD_Q4_STREAM", "2")
+    _lib.load().npamd_diag_reload_tuning()  # the library reads its tuning variables once
+    try:
+        y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, zp, L["bias"].to(gpu))
+        torch.cuda.synchronize()
+    finally:
+        monkeypatch.delenv("NPAMD_Q4_STREAM")
+        _lib.load().npamd_diag_reload_tuning()
+    assert y.shape == (1, n) and y.dtype == torch.float16
+    _check(y, _q_ref(oracle_lib, L, torch.float16))
+    y_rowwise = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, gs, zp, L["bias"].to(gpu))
+    assert (y.float() - y_rowwise.float()).abs().max().item() <= 2e-3 * max(1.0, y.float().abs().max().item())
+
+
 @pytest.mark.parametrize("asym", [False, True])
 def test_q4_rowwise_gemv_large_activations(gpu, asym):
     """Activations of a few hundred: the folded-out offset (72 * sum x) is then far larger than
