@@ -285,6 +285,7 @@ class SlicedIndices:
         for name, value in zip(self._FIELDS, values):
             setattr(self, name, value)
         self.wave_quads = struct.unpack("<16H", header[96:128])
+        self._workspace_bytes: dict[int, int] = {}  # per token count (asked on every call)
 
     @property
     def header_ptr(self) -> int:
@@ -293,7 +294,10 @@ class SlicedIndices:
         return ctypes.addressof(self._header_buf)
 
     def workspace_bytes(self, m: int) -> int:
-        return int(_lib.load().npamd_vq_sliced_workspace_bytes(self.header_ptr, int(m)))
+        need = self._workspace_bytes.get(m)
+        if need is None:
+            need = self._workspace_bytes[m] = int(_lib.load().npamd_vq_sliced_workspace_bytes(self.header_ptr, int(m)))
+        return need
 
     def to(self, device) -> "SlicedIndices":
         return SlicedIndices(self.blob.to(device), self.header)
@@ -347,14 +351,16 @@ def vq_slice_indices(
 _SLICED_WORKSPACES: dict = {}
 
 
-def sliced_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+def sliced_workspace(device: torch.device, nbytes: int, stream: int | None = None) -> torch.Tensor:
     """The zero-filled scratch of :func:`vq_linear_sliced` for the current stream of *device*.
 
     Every call hands its workspace back zero-filled, so one buffer per (device, stream) serves
     all layers whose calls follow each other on that stream.  Grown (and zero-filled again) on
     demand; allocate it before a graph capture starts, e.g. through ``NPVQLinear.prepare_sliced``.
     """
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    if stream is None:
+        stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device.index, stream)
     ws = _SLICED_WORKSPACES.get(key)
     if ws is None or ws.numel() * 4 < nbytes:
         ws = torch.zeros(max(nbytes, 1 << 20) // 4 + 4, device=device, dtype=torch.float32)
@@ -394,17 +400,26 @@ def vq_linear_sliced(
         _check_device(what, x, column_perm)
     if k != sliced.k or cb.shape[0] != sliced.nc or cb.shape[1] != sliced.vl:
         raise RuntimeError(f"{what}: slice lists were built for K={sliced.k}, codebook [{sliced.nc}, {sliced.vl}]")
-    need = sliced.workspace_bytes(max(m, 1))
-    if workspace is None:
-        workspace = sliced_workspace(x.device, need)
-    elif workspace.dtype != torch.float32 or not workspace.is_contiguous():
+    if workspace is not None and (workspace.dtype != torch.float32 or not workspace.is_contiguous()):
         raise RuntimeError(f"{what}: workspace must be a contiguous float32 tensor")
+    return vq_linear_sliced_checked(x, sliced, cb, _bias_f32(bias), column_perm, workspace)
+
+
+def vq_linear_sliced_checked(x, sliced, cb, bias_f32, column_perm, workspace=None) -> torch.Tensor:
+    """:func:`vq_linear_sliced` without the argument checks, for callers that have made them
+    (``NPVQLinear``, whose tensors come out of its own caches): *x* 2-D with unit inner stride,
+    fp16 / bf16, *cb* in ``x.dtype``, *bias_f32* float32 or None, *column_perm* int32 or None, all
+    on ``x``'s device.  The library still validates sizes and pointers."""
+    m = x.shape[0]
+    stream = _stream(x)
+    if workspace is None:
+        workspace = sliced_workspace(x.device, sliced.workspace_bytes(max(m, 1)), stream)
     y = torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
-    b32 = _bias_f32(bias)
+    dt = _DT[x.dtype]
     _lib.call(
         "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), _ptr(column_perm), sliced.header_ptr, sliced.blob.data_ptr(),
-        cb.data_ptr(), _DT[cb.dtype], _ptr(b32), _ptr(y), sliced.n, m, _DT[x.dtype],
-        workspace.data_ptr(), workspace.numel() * 4, _stream(x),
+        cb.data_ptr(), dt, _ptr(bias_f32), y.data_ptr(), sliced.n, m, dt,
+        workspace.data_ptr(), workspace.numel() * 4, stream,
     )  # fmt: skip
     return y
 

@@ -90,11 +90,11 @@ _GEMV_KERNEL_MAX_TOKENS: int = 32  # what the GEMV entry points accept (NPAMD_GE
 # compute unit's LDS next to the GEMV's buffers (more than 4096 rows): the fused
 # GEMV then pays one L2 lookup per index (34-35 us on a 14336 x 4096 layer with a
 # 65536-row codebook, any token count up to 16), while the slice-list GEMV
-# (kernels.vq_linear_sliced) keeps 8192-row codebook slices in LDS: 12.8 / 15.5 /
-# 21.3 / 24.1 / 29.2 / 32.0 us at 1 / 2 / 4 / 5 / 6 / 7 tokens; an eighth token needs
-# a second pass over the entries (40.8 us vs 36.4 us fused).  The slice lists are
-# built on the host at first use (about 25 MB per such layer, on top of the packed
-# stream the other bands keep reading).  0 disables the path.
+# (kernels.vq_linear_sliced) keeps 4096-row codebook slices in LDS: 10.3-10.9 / 14.2 /
+# 20.3 / 30.9 us at 1 / 2 / 4 / 7 tokens; an eighth token needs a second pass over the
+# entries.  The slice lists are built on the host by prepare_sliced() / prepare_decode(),
+# never by forward() (about 26 MB per such layer, on top of the packed stream the other
+# bands keep reading).  0 disables the path.
 _SLICED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_SLICED_MAX_TOKENS",), 7)
 _SLICED_MIN_CENTROIDS: int = 4097
 _SLICED_MIN_INDICES: int = _env_int(("NEUROPRESS_VQ_SLICED_MIN_INDICES",), 1 << 20)
@@ -777,11 +777,17 @@ class NPVQLinear(nn.Module):
 
         *leading, _ = x.shape
         perm = self._perm_i32(x.device) if self.column_perm is not None else None
+        if x.device != self.packed_indices.device:
+            raise RuntimeError(f"NPVQLinear: input on {x.device}, weights on {self.packed_indices.device}")
+        x2d = x.reshape(-1, self.in_features)
+        if x2d.stride(1) != 1:
+            x2d = x2d.contiguous()
         try:
-            y = kernels.vq_linear_sliced(
-                x.reshape(-1, self.in_features), sliced,
-                self.proxy.centroids_as(x.dtype), self._bias_f32(), column_perm=perm,
-            )  # fmt: skip
+            # forward() has checked x's dtype and device; the other tensors come out of this
+            # module's caches in the form the kernel reads.
+            y = kernels.vq_linear_sliced_checked(
+                x2d, sliced, self.proxy.centroids_as(x.dtype), self._bias_f32(), perm
+            )
         except RuntimeError as exc:
             self._fallback("vq_linear_sliced", "decode + GEMM", exc)
             if self.column_perm is not None:

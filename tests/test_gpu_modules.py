@@ -269,14 +269,14 @@ def test_prefix_coded_layers_run_the_hip_bands(gpu, kind, monkeypatch):
     assert layer.backend.value == {"tiered": "cuda_tiered", "ntier": "cuda_ntier", "zero_escape": "cuda_zero_escape"}[kind]
     assert layer.bits == 15 and layer.packed_indices.is_cuda
     calls = []
-    for name in ("vq_linear_sliced", "vq_linear", "vq_gemm_tile", "vq_dequant"):
+    for name in ("vq_linear_sliced_checked", "vq_linear", "vq_gemm_tile", "vq_dequant"):
         real = getattr(kernels, name)
         monkeypatch.setattr(kernels, name, lambda *a, _r=real, _n=name, **kw_: (calls.append(_n), _r(*a, **kw_))[1])
     w = cb[idx].reshape(n, k).float()
     for m in (1, 12, 40, 100):
         x = torch.randn(m, k, generator=cases.gen(m)).half()
         _close(layer(x.to(gpu)), torch.nn.functional.linear(x.float(), w, bias.float()))
-    assert calls == ["vq_linear_sliced", "vq_linear", "vq_gemm_tile", "vq_dequant"]
+    assert calls == ["vq_linear_sliced_checked", "vq_linear", "vq_gemm_tile", "vq_dequant"]
 
 
 # ------------------------------------------------------ benchmark full sizes ---

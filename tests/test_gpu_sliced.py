@@ -174,8 +174,8 @@ def test_module_routes_decode_steps_through_the_slice_lists(gpu, oracle_lib, act
     layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], n, k, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
     assert layer.prepare_sliced()  # forward never builds the lists itself
     calls = []
-    real = kernels.vq_linear_sliced
-    monkeypatch.setattr(kernels, "vq_linear_sliced", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
+    real = kernels.vq_linear_sliced_checked
+    monkeypatch.setattr(kernels, "vq_linear_sliced_checked", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
     x = L["x"].to(gpu)
     ref = _vq_ref(oracle_lib, L, act)
     y1 = layer(x[:1])
@@ -243,8 +243,8 @@ def test_forward_never_builds_slice_lists(gpu, monkeypatch, caplog):
     monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
     assert layer.prepare_sliced()
     seen = []
-    real = kernels.vq_linear_sliced
-    monkeypatch.setattr(kernels, "vq_linear_sliced", lambda *a, **kw: (seen.append(1), real(*a, **kw))[1])
+    real = kernels.vq_linear_sliced_checked
+    monkeypatch.setattr(kernels, "vq_linear_sliced_checked", lambda *a, **kw: (seen.append(1), real(*a, **kw))[1])
     y2 = layer(x)
     assert seen == [1]
     assert (y2.float() - y.float()).abs().max().item() < 1e-2
@@ -309,9 +309,9 @@ def test_column_permutation_is_applied_inside_the_sliced_kernel(gpu, oracle_lib,
                            bias=L["bias"].float(), column_perm=perm).to(gpu)
     assert layer.prepare_sliced()
     seen = []
-    real = kernels.vq_linear_sliced
-    monkeypatch.setattr(kernels, "vq_linear_sliced",
-                        lambda *a, **kw: (seen.append(kw.get("column_perm") is not None), real(*a, **kw))[1])
+    real = kernels.vq_linear_sliced_checked
+    monkeypatch.setattr(kernels, "vq_linear_sliced_checked",
+                        lambda *a, **kw: (seen.append(a[4] is not None), real(*a, **kw))[1])
     y = layer(L["x"].to(gpu))
     assert seen == ([True] if m <= 7 else [])
     Lp = dict(L, x=L["x"][:, perm].contiguous())
