@@ -395,3 +395,83 @@ def test_cfg4_residual_full_size(gpu):
         y = kernels.rvq_linear(x, dev["pm"], L["bm"], dev["pr"], L["br"], dev["cbm"], dev["cbr"], dev["scale"],
                                dev["wbias"], 1024, None, tile=tile)
         _close(y, x.float() @ w.float().T)
+
+
+# Full sizes anchored in the oracle itself (the C restatement decodes a few million vectors and
+# contracts one or two tokens in well under a second), not in the HIP decode.
+
+
+@pytest.mark.parametrize("name,n,k", [("q/o", 2048, 2048), ("k/v", 512, 2048), ("gate/up", 8192, 2048), ("down", 2048, 8192)])
+@pytest.mark.parametrize("bits", [12, 16])
+def test_cfg2_layers_full_size_against_the_oracle(gpu, oracle_lib, name, n, k, bits):
+    """Config 2's own four layers (4096 x 8 fp16 codebook, fp16, one and two tokens), with the
+    index stream as the 12-bit bit stream and as int16: decode bit-exact against the oracle's
+    decode, the LDS-codebook GEMV within the bound of the oracle's double-accumulated product."""
+    from neuropress_amd import kernels
+
+    from oracle import oracle as orc
+
+    lib = oracle_lib
+    L = cases.vq_layer(1002, n, k, 4096, bits=bits, act=torch.float16, m=2, bias=True)
+    code = orc.torch_dtype_code(torch.float16)
+    w_ref = lib.vq_decode(L["packed"].numpy(), bits, orc.to_bits(L["cb"]), n, k, code)
+    dev = {key: L[key].to(gpu) for key in ("x", "packed", "cb", "bias")}
+    w = kernels.vq_dequant(dev["packed"], dev["cb"], bits, n, k, torch.float16)
+    assert np.array_equal(orc.to_bits(w.cpu()), w_ref)
+    for m in (1, 2):
+        x = L["x"][:m].contiguous()
+        ref = lib.linear_f64(orc.to_bits(x), code, w_ref, code, orc.to_bits(L["bias"]), code)
+        y = kernels.vq_linear(x.to(gpu), dev["packed"], dev["cb"], bits, 8, dev["bias"], n)
+        ok, max_abs, excess = cases.within_tol(y.float().cpu().numpy(), ref)
+        assert ok, f"{name} M={m}: max abs err {max_abs:.3e} = {excess:.2f}x the 1e-2 bound"
+
+
+def test_cfg4_q_proj_full_size_against_the_oracle(gpu, oracle_lib):
+    """Config 4's q/o projection (4096 x 4096, residual VQ, Zipf(1.1) indices): decode bit-exact
+    against the oracle, one token through the fused GEMV against the oracle's product, 384 tokens
+    through the tile GEMM against the dense product of the (now anchored) decoded weight."""
+    from neuropress_amd import kernels
+
+    from oracle import oracle as orc
+
+    lib = oracle_lib
+    L = cases.rvq_layer(1004, 4096, 4096)
+    code = orc.torch_dtype_code(torch.float16)
+    w_ref = lib.rvq_decode(L["pm"].numpy(), L["bm"], L["pr"].numpy(), L["br"], orc.to_bits(L["cbm"]),
+                           orc.to_bits(L["cbr"]), orc.to_bits(L["scale"]), orc.to_bits(L["wbias"]), 4096, 4096, code)
+    dev = {k: (v.to(gpu) if isinstance(v, torch.Tensor) else v) for k, v in L.items()}
+    w = kernels.rvq_dequant(dev["pm"], L["bm"], dev["pr"], L["br"], dev["cbm"], dev["cbr"], dev["scale"],
+                            dev["wbias"], 4096, 4096, torch.float16)
+    assert np.array_equal(orc.to_bits(w.cpu()), w_ref)
+    ref = lib.linear_f64(orc.to_bits(L["x"]), code, w_ref, code)
+    y = kernels.rvq_linear(dev["x"], dev["pm"], L["bm"], dev["pr"], L["br"], dev["cbm"], dev["cbr"], dev["scale"],
+                           dev["wbias"], 4096, None, tile=False)
+    ok, max_abs, excess = cases.within_tol(y.float().cpu().numpy(), ref)
+    assert ok, f"max abs err {max_abs:.3e} = {excess:.2f}x the 1e-2 bound"
+    x = torch.randn(384, 4096, generator=cases.gen(384)).half().to(gpu)
+    y = kernels.rvq_linear(x, dev["pm"], L["bm"], dev["pr"], L["br"], dev["cbm"], dev["cbr"], dev["scale"],
+                           dev["wbias"], 4096, None, tile=True)
+    _close(y, x.float() @ w.float().T)
+
+
+def test_cfg5_square_layer_full_size_against_the_oracle(gpu, oracle_lib):
+    """Config 5's 4096 x 4096 layer: int4 decode bit-exact against the oracle, one token (the
+    row-wise kernel) against the oracle's product, 16 and 256 tokens against the dense product."""
+    from neuropress_amd import kernels
+
+    from oracle import oracle as orc
+
+    lib = oracle_lib
+    Q = cases.q4_layer(1005, 4096, 4096, bias=True)
+    code = orc.torch_dtype_code(torch.float16)
+    w_ref = lib.q_decode(Q["blob"].numpy(), orc.to_bits(Q["scale"]), None, 4, 32, code)
+    blob, sc, bias = Q["blob"].to(gpu), Q["scale"].to(gpu), Q["bias"].to(gpu)
+    w = kernels.q_dequant(blob, sc, 4, 32, None, torch.float16)
+    assert np.array_equal(orc.to_bits(w.cpu()), w_ref)
+    ref = lib.linear_f64(orc.to_bits(Q["x"]), code, w_ref, code, orc.to_bits(Q["bias"]), code)
+    y = kernels.q_linear(Q["x"].to(gpu), blob, sc, 4, 32, None, bias)
+    ok, max_abs, excess = cases.within_tol(y.float().cpu().numpy(), ref)
+    assert ok, f"max abs err {max_abs:.3e} = {excess:.2f}x the 1e-2 bound"
+    for m in (16, 256):
+        x = torch.randn(m, 4096, generator=cases.gen(m)).half().to(gpu)
+        _close(kernels.q_linear(x, blob, sc, 4, 32, None, bias), x.float() @ w.float().T + bias.float())
