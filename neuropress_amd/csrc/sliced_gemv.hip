@@ -76,9 +76,11 @@ struct Quad {
 
 // Entry quads a lane keeps requested ahead of the one it works on.
 constexpr int kDepth = 3;
-// Straight-line code exists for strips of up to this many quads, at up to kStraightTokens tokens.
+// Straight-line code exists for strips of up to this many quads, at the token counts where it
+// measured faster than the loops (config 3: 1 / 2 tokens, and 6 / 7 tokens 26.9 -> 25.1 / 29.9 -> 28.4 us;
+// no difference at 3-5 tokens, which keep the smaller code).
 constexpr int kMaxStraightQuads = 16;
-constexpr int kStraightTokens = 2;
+constexpr bool straight_tokens(int m) { return m <= 2 || m >= 6; }
 // LDS map: activations of the group range, then the slice, then the zero row that
 // padding entries select.  Both bases fit the 16-bit offset field of an LDS read.
 constexpr int kMaxTokens = 7;  // tokens per pass over the entries (an eighth token's activations would not fit in LDS)
@@ -279,7 +281,7 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
   float acc[M][2];
 #pragma unroll
   for (int m = 0; m < M; ++m) acc[m][0] = acc[m][1] = 0.f;
-  if (M <= kStraightTokens && nq <= kMaxStraightQuads) {
+  if (straight_tokens(M) && nq <= kMaxStraightQuads) {
     // Strips of up to kMaxStraightQuads quads (all of them, unless a row's indices crowd into one
     // slice) are walked by straight-line code picked by the strip's length: no loop carries a
     // register that is being loaded (a loop drains the quads in flight at every back-edge to
