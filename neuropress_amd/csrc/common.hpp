@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/npamd.h"
 
 namespace npamd {
@@ -35,6 +37,27 @@ struct Tuning {
   int q4_rows, q4_rowwise, q4_rowwise_bf16, q4_stream;
 };
 const Tuning& tuning();
+
+// Dynamic LDS beyond 64 KiB has to be enabled per kernel and per device (hipFuncSetAttribute).
+// One latch per kernel instantiation (a function-local static of its launcher) holds the largest
+// size enabled so far on each device; the attribute only ever grows, and two threads enabling
+// sizes at once both leave it large enough.  Devices past the table are enabled on every launch.
+constexpr int kLdsLatchDevices = 64;
+struct LdsLatch {
+  std::atomic<int> reserved[kLdsLatchDevices];
+};
+inline hipError_t enable_dynamic_lds(LdsLatch& latch, const void* kernel, int bytes) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+  std::atomic<int>* slot = (dev >= 0 && dev < kLdsLatchDevices) ? &latch.reserved[dev] : nullptr;
+  if (slot && bytes <= slot->load(std::memory_order_acquire)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess || !slot) return e;
+  int seen = slot->load(std::memory_order_relaxed);
+  while (seen < bytes && !slot->compare_exchange_weak(seen, bytes, std::memory_order_release)) {
+  }
+  return hipSuccess;
+}
 
 #define NPAMD_REQUIRE(cond, ...)                                  \
   do {                                                            \

@@ -87,12 +87,10 @@ extern "C" int npamd_diag_gather(const void* idx_u16, int64_t n_indices, const v
   }
   NPAMD_REQUIRE(table_entries <= 8192, "npamd_diag_gather: an LDS table holds at most 8192 rows");
   const int lds = table_entries * 16;
-  static int reserved = 0;
-  if (lds > 64 * 1024 && lds > reserved) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&diag_gather_lds_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (lds > 64 * 1024) {
+    static LdsLatch latch;
+    const hipError_t e = enable_dynamic_lds(latch, reinterpret_cast<const void*>(&diag_gather_lds_kernel), lds);
     if (e != hipSuccess) return fail(NPAMD_ERR_LAUNCH, "npamd_diag_gather: %s", hipGetErrorString(e));
-    reserved = lds;
   }
   const int blocks = 512;
   const int64_t per_block = (n8 + blocks - 1) / blocks;

@@ -449,18 +449,11 @@ int launch_tile_gemm_mw_cb(const GemmShape& s, const typename Provider::Args& pa
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
   const int lds = XStage<MW, CB_LDS>::kLdsBytes + (CB_LDS ? cb_bytes : 0);
-  static std::atomic<int> reserved{0};  // per instantiation: largest dynamic-LDS size enabled so far (the
-  // attribute only ever grows; two threads enabling sizes at once both leave it large enough)
-  if (lds > reserved.load(std::memory_order_acquire)) {
-    const hipError_t e = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&tile_gemm_kernel<ACT, Provider, MW, CB_LDS>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds,
-                                     hipGetErrorString(e));
-    int seen = reserved.load(std::memory_order_relaxed);
-    while (seen < lds && !reserved.compare_exchange_weak(seen, lds, std::memory_order_release)) {
-    }
-  }
+  static LdsLatch latch;  // per instantiation
+  const hipError_t e =
+      enable_dynamic_lds(latch, reinterpret_cast<const void*>(&tile_gemm_kernel<ACT, Provider, MW, CB_LDS>), lds);
+  if (e != hipSuccess)
+    return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
   tile_gemm_kernel<ACT, Provider, MW, CB_LDS><<<grid, 512, lds, st>>>(s, pargs);
   if (s.splits > 1) {
     const int64_t quads = (int64_t)s.M * ((s.N + 3) / 4);

@@ -246,18 +246,11 @@ int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const
                       : red_bytes + x_bytes +
                             ((X_LDS && s.perm) ? (cb_lds_bytes > x_bytes ? cb_lds_bytes : x_bytes) : cb_lds_bytes);
   if (lds > 64 * 1024) {
-    static std::atomic<int> reserved{0};  // per instantiation: largest dynamic-LDS size enabled so far (the
-  // attribute only ever grows; two threads enabling sizes at once both leave it large enough)
-    if (lds > reserved.load(std::memory_order_acquire)) {
-      const hipError_t e = hipFuncSetAttribute(
-          reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT>),
-          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      if (e != hipSuccess)
-        return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
-      int seen = reserved.load(std::memory_order_relaxed);
-    while (seen < lds && !reserved.compare_exchange_weak(seen, lds, std::memory_order_release)) {
-    }
-    }
+    static LdsLatch latch;  // per instantiation
+    const hipError_t e = enable_dynamic_lds(
+        latch, reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT>), lds);
+    if (e != hipSuccess)
+      return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
   }
   fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);

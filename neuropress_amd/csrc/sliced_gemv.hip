@@ -374,14 +374,10 @@ __global__ void __launch_bounds__(256) sliced_reduce_kernel(float* __restrict__ 
 
 template <int ACT, int M, bool PERM>
 int launch_sliced_tokens_p(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
-  static std::once_flag once;
-  static hipError_t reserve_error = hipSuccess;
-  std::call_once(once, [] {
-    reserve_error = hipFuncSetAttribute(reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M, PERM>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  });
-  if (reserve_error != hipSuccess)
-    return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(reserve_error));
+  static LdsLatch latch;  // per instantiation
+  const hipError_t e = enable_dynamic_lds(latch, reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M, PERM>), kLdsBytes);
+  if (e != hipSuccess)
+    return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(e));
   sliced_gemv_kernel<ACT, M, PERM><<<n_workgroups, kSlicedTasks, kLdsBytes, st>>>(a);
   return check_launch(what);
 }
