@@ -145,7 +145,7 @@ int npamd_vq_lut_gather(const float* lut, const uint8_t* packed, int64_t n_bytes
 /*
  * For codebooks too large for a compute unit's LDS (more than 4096 rows) the
  * decode GEMV is bound by random 16-byte codebook lookups in L2.  The slice-list
- * form files every index under the 8192-row codebook slice it points into, so a
+ * form files every index under the 4096-row codebook slice it points into, so a
  * workgroup that holds one slice in LDS only sees the lookups that hit it; every
  * lane sums the entries of one output row in a register.  It is
  * built once per layer from the packed stream (a construction-time re-layout,
