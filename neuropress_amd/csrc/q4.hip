@@ -156,7 +156,7 @@ __device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t m
   return r;
 }
 
-constexpr int kQ4RowWaves = 4;   // waves per block; a wave owns R consecutive rows
+// The row-wise kernel's blocks have W = 4 or 8 waves; a wave owns R consecutive rows.
 
 template <int R>
 struct Q4RowItem {   // one pass (64 groups of 32 k) of R rows
@@ -236,8 +236,8 @@ __device__ __forceinline__ void q4_row_compute(const Q4RowItem<R>& it, const Q4R
   }
 }
 
-template <int ACT, int M, int R, bool ASYM>
-__global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4RowArgs a) {
+template <int ACT, int M, int R, bool ASYM, int W>
+__global__ void __launch_bounds__(W * 64) q4_rowwise_gemv_kernel(Q4RowArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // xs[m][pass][piece 0..3][lane] (16-byte vectors), then off[m][pass][lane] (floats), then
   // (ASYM) sumx[m][pass][lane].
@@ -246,7 +246,7 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
   float* sumx = off + (size_t)M * a.passes * 64;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r0 = (blockIdx.x * kQ4RowWaves + wave) * R;
+  const int r0 = (blockIdx.x * W + wave) * R;
 
   // The first pass of weights is requested before x is staged (requesting two here is
   // slower: 11.5 vs 9.2 us on 14336 x 4096).
@@ -255,7 +255,7 @@ __global__ void __launch_bounds__(kQ4RowWaves * 64) q4_rowwise_gemv_kernel(Q4Row
 
   // Stage x: one thread per (token, 32-k group): its four vectors go to the lane-major
   // layout in (k, k+4) pair order, sum (b[k] + 8) * x[k] to the offset table.
-  for (int i = tid; i < M * a.passes * 64; i += kQ4RowWaves * 64) {
+  for (int i = tid; i < M * a.passes * 64; i += W * 64) {
     const int m = i / (a.passes * 64), g = i % (a.passes * 64);
     const u32x4* xg = reinterpret_cast<const u32x4*>(a.x + (int64_t)m * a.ldx) + (size_t)g * 4;
     float sum_even = 0.f, sum_odd = 0.f;  // over even / odd k of the group
@@ -513,14 +513,32 @@ static bool q_fast_ok(const QCall& c) {
 
 
 
-template <int ACT, int M, int R>
-static int launch_q4_rowwise_r(const Q4RowArgs& a, hipStream_t st, const char* what) {
-  const int rows_per_block = R * kQ4RowWaves;
+static int device_cus_q4() {
+  static std::atomic<int> cached{0};
+  int cus = cached.load(std::memory_order_relaxed);
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    cached.store(cus, std::memory_order_relaxed);
+  }
+  return cus;
+}
+
+template <int ACT, int M, int R, int W>
+static int launch_q4_rowwise_rw(const Q4RowArgs& a, hipStream_t st, const char* what) {
+  const int rows_per_block = R * W;
   const int blocks = (a.N + rows_per_block - 1) / rows_per_block;
   const int lds = M * a.passes * (4 * 64 * 16 + 64 * 4 * 2);
-  if (a.zp) q4_rowwise_gemv_kernel<ACT, M, R, true><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
-  else q4_rowwise_gemv_kernel<ACT, M, R, false><<<blocks, kQ4RowWaves * 64, lds, st>>>(a);
+  if (a.zp) q4_rowwise_gemv_kernel<ACT, M, R, true, W><<<blocks, W * 64, lds, st>>>(a);
+  else q4_rowwise_gemv_kernel<ACT, M, R, false, W><<<blocks, W * 64, lds, st>>>(a);
   return check_launch(what);
+}
+
+template <int ACT, int M, int R>
+static int launch_q4_rowwise_r(const Q4RowArgs& a, int waves, hipStream_t st, const char* what) {
+  return waves >= 8 ? launch_q4_rowwise_rw<ACT, M, R, 8>(a, st, what) : launch_q4_rowwise_rw<ACT, M, R, 4>(a, st, what);
 }
 
 template <int ACT, int M>
@@ -534,33 +552,18 @@ static int launch_q4_rowwise(const QCall& c) {
   a.passes = (a.groups32 + 63) / 64;
   a.scales_per_row = c.K / c.gs;
   a.gs_shift = log2i(c.gs / 32);
-  // Rows per wave: 2 when that still leaves at least eight waves per compute unit (measured
-  // on 14336 x 4096: 1 row 12.0 us, 2 rows 10.4 us, 4 rows 10.8 us).
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-  }
+  // Rows per wave: 2 when that still leaves sixteen waves per compute unit, else 1; waves per
+  // block (x is staged once per block): 8 from four passes up, else 4.  Measured (us, 4 / 8 / 16
+  // waves): 14336 x 4096 one row 11.6 / 10.9 / 11.2, two rows 9.7 / 10.7 / 10.6, four 10.2 / 10.3 / 10.1;
+  // 4096 x 4096 one row 5.07 / 5.0 / 5.05, two 5.3 / 5.3 / 5.9; 4096 x 14336 one row 10.5 / 9.3 / 9.2,
+  // two 10.0 / 9.6 / 11.3.
+  const int cus = device_cus_q4();
   const int r_env = tuning().q4_rows;
-  const int r = r_env ? r_env : (c.N >= 16 * cus ? 2 : 1);
-  if (r >= 4) return launch_q4_rowwise_r<ACT, M, 4>(a, c.st, c.what);
-  if (r >= 2) return launch_q4_rowwise_r<ACT, M, 2>(a, c.st, c.what);
-  return launch_q4_rowwise_r<ACT, M, 1>(a, c.st, c.what);
-}
-
-static int device_cus_q4() {
-  static std::atomic<int> cached{0};
-  int cus = cached.load(std::memory_order_relaxed);
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-    cached.store(cus, std::memory_order_relaxed);
-  }
-  return cus;
+  const int r = r_env ? r_env : (c.N >= 32 * cus ? 2 : 1);
+  const int waves = a.passes >= 4 ? 8 : 4;
+  if (r >= 4) return launch_q4_rowwise_r<ACT, M, 4>(a, waves, c.st, c.what);
+  if (r >= 2) return launch_q4_rowwise_r<ACT, M, 2>(a, waves, c.st, c.what);
+  return launch_q4_rowwise_r<ACT, M, 1>(a, waves, c.st, c.what);
 }
 
 // The resident-grid kernel takes one token of a layer with at most 16 passes (K <= 65536) whose

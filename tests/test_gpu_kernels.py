@@ -306,15 +306,15 @@ def _q_ref(oracle_lib, L, act):
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 128), (4200, 256)])
+@pytest.mark.parametrize("n,k", [(301, 384), (64, 4096), (37, 14336), (5, 2048 + 128), (4200, 256), (8300, 256)])
 @pytest.mark.parametrize("gs", [32, 128])
 @pytest.mark.parametrize("m", [1, 2])
 @pytest.mark.parametrize("asym", [False, True])
 def test_q4_rowwise_gemv(gpu, oracle_lib, act, n, k, gs, m, asym):
     """One fp16 token takes the row-wise kernel (nibbles read as base + q, group offsets folded
     out), two tokens and bf16 the MFMA GEMV.  Row counts that are not a multiple of the rows per wave
-    (and enough rows for two per wave), K of one partial pass, of several passes and of a
-    partial last pass."""
+    (8300 rows: two per wave), K of one partial pass, of several passes (14336: eight waves per
+    block) and of a partial last pass."""
     from neuropress_amd import kernels
 
     L = cases.q4_layer(700 + n + m, n, k, gs=gs, act=act, m=m, bias=True, asym=asym)
