@@ -248,7 +248,8 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
       perm_hi = reinterpret_cast<const u32x4*>(a.column_perm)[2 * xvec + 1];
     } else {
 #pragma unroll
-      for (int i = 0; i < kXLoads; ++i) xt[i] = reinterpret_cast<const u32x4*>(xrow[i])[xvec];
+      for (int i = 0; i < kXLoads; ++i)
+        if (xm + 2 * i < M) xt[i] = reinterpret_cast<const u32x4*>(xrow[i])[xvec];  // wave-uniform: xm = tid / 512
     }
     __builtin_amdgcn_sched_barrier(0);  // keep the entry requests behind the slice's
     // The first quads (past the strip's end: its last quad again; no branch around a load).
