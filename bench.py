@@ -325,6 +325,7 @@ def main():
     alg = vq_alg_bytes(c3, 1)
     gbs = alg / us / 1e3
     host_us, wall_us = time_eager(step, s_rot, 200, dev)
+    us_warm = time_graph(lambda i: step(0), 1, max(args.steps, 20), 2, dev)  # one blob, no flush: served by the Infinity Cache
 
     # correctness gate on the timed configuration (decode bit-exact, output within 1e-2 + 1e-2 |ref|)
     w_gpu = kernels.vq_dequant(c3["pool"][0], c3["d_cb"], 16, n, k, torch.bfloat16)
@@ -365,6 +366,7 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(us / 1e3, 6),
         "us_per_call": round(us, 3),
+        "cache_warm_us_per_call": round(us_warm, 3),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -418,47 +420,67 @@ def main():
     del xm2, y2
 
     # ---------------- sweep over the other bands / configs ----------------------
+    # Every row: the call timed as above, and the same call's output checked against the dense
+    # product of the decoded weight in f32 (the decode kernels are bit-exact against the oracle,
+    # tested): max abs error, its largest ratio to the bound 1e-2 + 1e-2 |ref|, and the verdict.
     sweep = []
     if not args.no_sweep:
-        def add(name, band, m, us_, alg_bytes, flops):
-            sweep.append({"case": name, "band": band, "M": m, "us": round(us_, 2),
-                          "GBps": round(alg_bytes / us_ / 1e3, 1), "hbm_frac": round(alg_bytes / us_ / 1e3 / HBM_PEAK_GBS, 4),
-                          "TFLOPs": round(flops / us_ / 1e6, 1), "mfma_frac": round(flops / us_ / 1e6 / MFMA_PEAK_TFLOPS, 4)})
+        def check(y, ref):
+            err = (y.float() - ref).abs()
+            bound = 1e-2 + 1e-2 * ref.abs()
+            return {"max_abs_err": round(float(err.max()), 6), "err_over_bound": round(float((err / bound).max()), 3),
+                    "ok": bool((err <= bound).all())}
+
+        def run(name, band, m, f, rot, alg_bytes, flops, ref=None, steps=None, warm=3):
+            us_ = timed(f, rot, steps, warm)
+            row = {"case": name, "band": band, "M": m, "us": round(us_, 2),
+                   "GBps": round(alg_bytes / us_ / 1e3, 1), "hbm_frac": round(alg_bytes / us_ / 1e3 / HBM_PEAK_GBS, 4),
+                   "TFLOPs": round(flops / us_ / 1e6, 1), "mfma_frac": round(flops / us_ / 1e6 / MFMA_PEAK_TFLOPS, 4)}
+            if ref is not None:
+                row.update(check(f(0), ref()))
+            sweep.append(row)
 
         def xpair(m, kk, seed, act):
             return [torch.randn(m, kk, generator=gen(seed + j)).to(act).to(dev) for j in range(2)]
 
+        w32 = w_gpu.float()  # config 3 up/gate, decoded above and found bit-exact
+        name = "cfg3 14336x4096 bf16"
         for m in (2, 4, 7):
-            xm2 = xpair(m, k, 50 + m, torch.bfloat16)
+            xm = xpair(m, k, 50 + m, torch.bfloat16)
             ws2 = torch.zeros(sl0.workspace_bytes(m) // 4, device=dev, dtype=torch.float32)
-            t = timed(lambda i: kernels.vq_linear_sliced(xm2[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2), s_rot)
-            add("cfg3 14336x4096 bf16", "a:sliced-gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+            run(name, "a:sliced-gemv", m,
+                lambda i: kernels.vq_linear_sliced(xm[i % 2], spool[i], c3["d_cb_act"], None, workspace=ws2), s_rot,
+                vq_alg_bytes(c3, m), 2.0 * m * n * k, ref=lambda: xm[0].float() @ w32.T)
         del spool[1:]
         torch.cuda.empty_cache()
         for m in (1, 2, 16, 32):  # 32: two 16-token tiles per decoded operand
             xm = xpair(m, k, 50 + m, torch.bfloat16)
-            t = timed(lambda i: kernels.vq_linear(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n), n_rot)
-            add("cfg3 14336x4096 bf16", "a:fused-gemv", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+            run(name, "a:fused-gemv", m, lambda i: kernels.vq_linear(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, 8, None, n),
+                n_rot, vq_alg_bytes(c3, m), 2.0 * m * n * k, ref=lambda: xm[0].float() @ w32.T)
         for m in (64, 384, 1024, 4096):
             xm = xpair(m, k, 60 + m, torch.bfloat16)
-            steps_m = n_rot if m <= 1024 else 12
-            t = timed(lambda i: kernels.vq_gemm_tile(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, n, None), n_rot, steps_m, 2)
-            add("cfg3 14336x4096 bf16", "b:tile-gemm", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
-            t = timed(lambda i: torch.nn.functional.linear(
-                xm[i % 2], kernels.vq_dequant(c3["pool"][i], c3["d_cb"], 16, n, k, torch.bfloat16)), n_rot, steps_m, 2)
-            add("cfg3 14336x4096 bf16", "c:decode+gemm", m, t, vq_alg_bytes(c3, m), 2.0 * m * n * k)
+            steps_m = None if m <= 1024 else 12
+            ref = lambda: xm[0].float() @ w32.T
+            run(name, "b:tile-gemm", m, lambda i: kernels.vq_gemm_tile(xm[i % 2], c3["pool"][i], c3["d_cb_act"], 16, n, None),
+                n_rot, vq_alg_bytes(c3, m), 2.0 * m * n * k, ref=ref, steps=steps_m, warm=2)
+            run(name, "c:decode+gemm", m, lambda i: torch.nn.functional.linear(
+                xm[i % 2], kernels.vq_dequant(c3["pool"][i], c3["d_cb"], 16, n, k, torch.bfloat16)),
+                n_rot, vq_alg_bytes(c3, m), 2.0 * m * n * k, ref=ref, steps=steps_m, warm=2)
             del xm
-        del c3["pool"][1:]
+        del c3["pool"][1:], w32
         torch.cuda.empty_cache()
         # config 3 down-proj shape
+        name = "cfg3 4096x14336 bf16"
         c3d = vq_case(dev, 1003, 4096, 14336, 65536, 16, torch.bfloat16, n_rot)
+        w32 = kernels.vq_dequant(c3d["pool"][0], c3d["d_cb"], 16, 4096, 14336, torch.bfloat16).float()
         sld = kernels.vq_slice_indices(c3d["packed"], 16, 4096, 14336, 8, 65536, device=dev)
         sdpool = [sld] + [kernels.SlicedIndices(sld.blob.clone(), sld.header) for _ in range(rot_for(sld.total_bytes) - 1)]
         for m in (1, 2):
             wsd = torch.zeros(sld.workspace_bytes(m) // 4, device=dev, dtype=torch.float32)
-            xd = xpair(m, 14336, 70 + m, torch.bfloat16)
-            t = timed(lambda i: kernels.vq_linear_sliced(xd[i % 2], sdpool[i], c3d["d_cb_act"], None, workspace=wsd), len(sdpool))
-            add("cfg3 4096x14336 bf16", "a:sliced-gemv", m, t, vq_alg_bytes(c3d, m), 2.0 * m * 4096 * 14336)
+            xm = xpair(m, 14336, 70 + m, torch.bfloat16)
+            run(name, "a:sliced-gemv", m,
+                lambda i: kernels.vq_linear_sliced(xm[i % 2], sdpool[i], c3d["d_cb_act"], None, workspace=wsd), len(sdpool),
+                vq_alg_bytes(c3d, m), 2.0 * m * 4096 * 14336, ref=lambda: xm[0].float() @ w32.T)
         del sdpool, sld
         torch.cuda.empty_cache()
         for m, band in ((1, "a:fused-gemv"), (16, "a:fused-gemv"), (64, "b:tile-gemm"), (384, "b:tile-gemm"),
@@ -468,50 +490,57 @@ def main():
                 f = lambda i: kernels.vq_linear(xm[i % 2], c3d["pool"][i], c3d["d_cb_act"], 16, 8, None, 4096)
             else:
                 f = lambda i: kernels.vq_gemm_tile(xm[i % 2], c3d["pool"][i], c3d["d_cb_act"], 16, 4096, None)
-            t = timed(f, n_rot, n_rot if m <= 1024 else 12, 2)
-            add("cfg3 4096x14336 bf16", band, m, t, vq_alg_bytes(c3d, m), 2.0 * m * 4096 * 14336)
+            run(name, band, m, f, n_rot, vq_alg_bytes(c3d, m), 2.0 * m * 4096 * 14336,
+                ref=lambda: xm[0].float() @ w32.T, steps=None if m <= 1024 else 12, warm=2)
             del xm
-        del c3d
+        del c3d, w32
         torch.cuda.empty_cache()
         # config 2: 4096-entry codebook, fp16.  Every shape with the index stream as int16 (the bytes the
         # configuration is quoted on); gate/up also with the 12-bit stream and a column permutation.
         for label, nn_, kk in (("q/o", 2048, 2048), ("k/v", 512, 2048), ("gate/up", 8192, 2048), ("down", 2048, 8192)):
             rot = rot_for(nn_ * kk // 8 * 2)
             cc = vq_case(dev, 1002, nn_, kk, 4096, 16, torch.float16, rot)
+            w32 = kernels.vq_dequant(cc["pool"][0], cc["d_cb"], 16, nn_, kk, torch.float16).float()
             for m in (1, 2):
                 xm = xpair(m, kk, 80 + m, torch.float16)
-                t = timed(lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], 16, 8, None, nn_), rot)
-                add(f"cfg2 {label} {nn_}x{kk} f16 int16 stream", "a:gemv", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
-            del cc
+                run(f"cfg2 {label} {nn_}x{kk} f16 int16 stream", "a:gemv", m,
+                    lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], 16, 8, None, nn_), rot,
+                    vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk, ref=lambda: xm[0].float() @ w32.T)
+            del cc, w32
             torch.cuda.empty_cache()
         for name, (nn_, kk, nc, bits), ms in (("cfg2 gate/up 8192x2048 f16 12-bit stream", (8192, 2048, 4096, 12), (1, 2, 32)),
                                               ("cfg1 2048x640 f16 8-bit", (2048, 640, 256, 8), (1, 16))):
             rot = rot_for(nn_ * kk // 8 * bits // 8)
             cc = vq_case(dev, 1002 if bits == 12 else 1001, nn_, kk, nc, bits, torch.float16, rot)
+            w32 = kernels.vq_dequant(cc["pool"][0], cc["d_cb"], bits, nn_, kk, torch.float16).float()
             for m in ms:
                 xm = xpair(m, kk, 80 + m, torch.float16)
-                t = timed(lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_), rot)
-                add(name, "a:gemv", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
+                ref = lambda: xm[0].float() @ w32.T
+                run(name, "a:gemv", m, lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_),
+                    rot, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk, ref=ref)
                 if m == 1 and bits == 12:
                     # the same call with a column permutation: gathered inside the GEMV, or by torch in front of it
                     perm = torch.randperm(kk, generator=gen(90)).to(dev)
                     p32 = perm.to(torch.int32)
-                    t = timed(lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_,
-                                                          column_perm=p32), rot)
-                    add(name + " column_perm", "a:gemv, gather fused", m, t, vq_alg_bytes(cc, m) + kk * 4, 2.0 * m * nn_ * kk)
-                    t = timed(lambda i: kernels.vq_linear(xm[i % 2][:, perm], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_), rot)
-                    add(name + " column_perm", "a:torch gather + gemv", m, t, vq_alg_bytes(cc, m) + kk * 8, 2.0 * m * nn_ * kk)
+                    refp = lambda: xm[0][:, perm].float() @ w32.T
+                    run(name + " column_perm", "a:gemv, gather fused", m,
+                        lambda i: kernels.vq_linear(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_, column_perm=p32),
+                        rot, vq_alg_bytes(cc, m) + kk * 4, 2.0 * m * nn_ * kk, ref=refp)
+                    run(name + " column_perm", "a:torch gather + gemv", m,
+                        lambda i: kernels.vq_linear(xm[i % 2][:, perm], cc["pool"][i], cc["d_cb"], bits, 8, None, nn_),
+                        rot, vq_alg_bytes(cc, m) + kk * 8, 2.0 * m * nn_ * kk, ref=refp)
             if bits == 12:
                 # the same layer in the token bands the configuration itself does not list: tile GEMM with the
                 # 4096-row codebook looked up in LDS, against decode + GEMM
                 for m in (64, 256):
                     xm = xpair(m, kk, 80 + m, torch.float16)
-                    t = timed(lambda i: kernels.vq_gemm_tile(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, nn_, None), rot)
-                    add(name, "b:tile-gemm", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
-                    t = timed(lambda i: torch.nn.functional.linear(
-                        xm[i % 2], kernels.vq_dequant(cc["pool"][i], cc["d_cb"], bits, nn_, kk, torch.float16)), rot)
-                    add(name, "c:decode+gemm", m, t, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk)
-            del cc
+                    ref = lambda: xm[0].float() @ w32.T
+                    run(name, "b:tile-gemm", m, lambda i: kernels.vq_gemm_tile(xm[i % 2], cc["pool"][i], cc["d_cb"], bits, nn_, None),
+                        rot, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk, ref=ref)
+                    run(name, "c:decode+gemm", m, lambda i: torch.nn.functional.linear(
+                        xm[i % 2], kernels.vq_dequant(cc["pool"][i], cc["d_cb"], bits, nn_, kk, torch.float16)),
+                        rot, vq_alg_bytes(cc, m), 2.0 * m * nn_ * kk, ref=ref)
+            del cc, w32
             torch.cuda.empty_cache()
         # config 4: residual VQ (65536 + 256 entry codebooks, Zipf(1.1) indices, per-row scale / bias), fp16
         def zipf(gq, nc, count):
@@ -530,6 +559,7 @@ def main():
             rot = rot_for(pm.numel() + pr.numel(), cap=128)
             pms = [pm.to(dev).clone() for _ in range(rot)]
             prs = [pr.to(dev).clone() for _ in range(rot)]
+            w32 = kernels.rvq_dequant(pms[0], 16, prs[0], 8, cbm, cbr, rsc, rbi, nn_, kk, torch.float16).float()
             alg4 = lambda m: cnt * 3 + (65536 + 256) * 16 + nn_ * 4 + m * kk * 2 + m * nn_ * 2
             for m, band in ((1, "a:fused-gemv"), (32, "a:fused-gemv"), (128, "b:tile-gemm"), (384, "b:tile-gemm"),
                             (384, "c:decode+gemm")):
@@ -541,9 +571,8 @@ def main():
                 else:
                     f = lambda i: torch.nn.functional.linear(
                         xm[i % 2], kernels.rvq_dequant(pms[i], 16, prs[i], 8, cbm, cbr, rsc, rbi, nn_, kk, torch.float16))
-                t = timed(f, rot)
-                add(f"cfg4 rvq {nn_}x{kk} f16", band, m, t, alg4(m), 2.0 * m * nn_ * kk)
-            del pms, prs
+                run(f"cfg4 rvq {nn_}x{kk} f16", band, m, f, rot, alg4(m), 2.0 * m * nn_ * kk, ref=lambda: xm[0].float() @ w32.T)
+            del pms, prs, w32
             torch.cuda.empty_cache()
         # config 5: int4 group-affine, fp16, both shapes
         from neuropress_amd.t2n.packing import BitPacking4
@@ -555,33 +584,37 @@ def main():
             rot = rot_for(blob.numel(), cap=128)
             blobs = [blob.to(dev)]
             blobs += [blobs[0].clone() for _ in range(rot - 1)]
+            w32 = kernels.q_dequant(blobs[0], sc, 4, 32, None, torch.float16).float()
             for m in (1, 16, 32, 256):
                 xm = xpair(m, kk, 90 + m, torch.float16)
-                t = timed(lambda i: kernels.q_linear(xm[i % 2], blobs[i], sc, 4, 32), rot)
                 algq = nn_ * kk // 2 + nn_ * kk // 32 * 2 + m * kk * 2 + m * nn_ * 2
-                add(f"cfg5 int4 {nn_}x{kk} f16", "a:gemv" if m <= 32 else "b:tile-gemm", m, t, algq, 2.0 * m * nn_ * kk)
+                run(f"cfg5 int4 {nn_}x{kk} f16", "a:gemv" if m <= 32 else "b:tile-gemm", m,
+                    lambda i: kernels.q_linear(xm[i % 2], blobs[i], sc, 4, 32), rot, algq, 2.0 * m * nn_ * kk,
+                    ref=lambda: xm[0].float() @ w32.T)
             if nn_ == 14336:
                 q5 = {"blob": blob, "scale": sc.cpu(), "x": xpair(1, kk, 91, torch.float16)[0].cpu(), "n": nn_, "k": kk,
                       "y": kernels.q_linear(xpair(1, kk, 91, torch.float16)[0], blobs[0], sc, 4, 32).cpu()}
-            del blobs
+            del blobs, w32
             torch.cuda.empty_cache()
         # neighbours of the linear on a decode step: RMSNorm and the embedding lookups (Llama-3-8B sizes)
         hdim, vocab = 4096, 128256
         wn = (torch.rand(hdim, generator=g) + 0.5).to(torch.bfloat16).to(dev)
         for m in (1, 4096):
             xn = [torch.randn(m, hdim, generator=gen(95 + i)).to(torch.bfloat16).to(dev) for i in range(8 if m > 1 else 2)]
-            t = timed(lambda i: kernels.rms_norm(xn[i % len(xn)], wn, 1e-6), len(xn), 20, 3)
-            add("rms_norm H=4096 bf16", "aux", m, t, 2 * m * hdim * 2 + hdim * 2, 0.0)
+            run("rms_norm H=4096 bf16", "aux", m, lambda i: kernels.rms_norm(xn[i % len(xn)], wn, 1e-6), len(xn),
+                2 * m * hdim * 2 + hdim * 2, 0.0, steps=20)
         cbe = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.float16).to(dev)
         tab = torch.randint(0, 65536, (vocab, hdim // 8), generator=g, dtype=torch.int32).to(torch.int16).to(dev)
         qblob = torch.randint(0, 256, (vocab, hdim // 2), generator=g, dtype=torch.int32).to(torch.uint8).to(dev)
         qsc = (torch.rand(vocab * hdim // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
         for m in (1, 4096):
             ids = [torch.randint(0, vocab, (m,), generator=gen(97 + i)).to(dev) for i in range(4)]
-            t = timed(lambda i: kernels.vq_embedding(ids[i % 4], tab, cbe, 64.0, None, torch.bfloat16), 4, 20, 3)
-            add("vq_embedding 128256x4096 -> bf16", "aux", m, t, m * (8 + hdim // 8 * 2 + hdim // 8 * 16 + hdim * 2), 0.0)
-            t = timed(lambda i: kernels.q_embedding(ids[i % 4], qblob, qsc, 4, 32, None, None, 64.0, torch.bfloat16), 4, 20, 3)
-            add("int4 embedding 128256x4096 -> bf16", "aux", m, t, m * (8 + hdim // 2 + hdim // 32 * 2 + hdim * 2), 0.0)
+            run("vq_embedding 128256x4096 -> bf16", "aux", m,
+                lambda i: kernels.vq_embedding(ids[i % 4], tab, cbe, 64.0, None, torch.bfloat16), 4,
+                m * (8 + hdim // 8 * 2 + hdim // 8 * 16 + hdim * 2), 0.0, steps=20)
+            run("int4 embedding 128256x4096 -> bf16", "aux", m,
+                lambda i: kernels.q_embedding(ids[i % 4], qblob, qsc, 4, 32, None, None, 64.0, torch.bfloat16), 4,
+                m * (8 + hdim // 2 + hdim // 32 * 2 + hdim * 2), 0.0, steps=20)
         del tab, qblob, qsc
         torch.cuda.empty_cache()
     result["sweep"] = sweep
