@@ -161,7 +161,12 @@ __device__ __forceinline__ void finish_row(const SlicedArgs& a, int m, uint32_t 
   if (fits) {
     add += (unsigned long long)(long long)__float2ll_rn(v * kFixedOne) << 16;
   } else {
-    __hip_atomic_fetch_add(a.spill + cell, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // returns: done before the count
+    // The addition must have been performed before this lane's arrival is counted (the lane that
+    // completes the count reads the accumulator): its result is asked for and waited for -- an
+    // atomic without a use of its result is issued as fire-and-forget, and nothing orders it
+    // against the atomic on the row's word, which may live in another L2 channel.
+    const float before = __hip_atomic_fetch_add(a.spill + cell, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("" ::"v"(before) : "memory");
     add += 0x100ull;
   }
   const unsigned long long old = __hip_atomic_fetch_add(a.sums + cell, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
