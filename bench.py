@@ -42,7 +42,7 @@ POOL_BYTES = 640 << 20         # rotate through more than L2 (32 MB) + Infinity 
 # counters read for a plain copy of known size).  Not measured in this run: the profile summary named
 # in `source` holds the command, the raw counter values and the date they were taken.
 TRAFFIC = {
-    "sliced_m1": {"bytes": 13581 * 1024 * 2 + 1932 * 1024, "source": "profiles/vq_sliced_gemv_cfg3_14336x4096_m1.md"},
+    "sliced_m1": {"bytes": 13577 * 1024 * 2 + 1932 * 1024, "source": "profiles/vq_sliced_gemv_cfg3_14336x4096_m1.md"},
     "tile_m384": {"bytes": 60422 * 1024 * 2 + 11670 * 1024, "source": "profiles/vq_tile_gemm_cfg3_14336x4096_m384.md"},
 }
 FLUSH_BYTES = 512 << 20        # written before every timed replay: nothing a replay reads is still cached
