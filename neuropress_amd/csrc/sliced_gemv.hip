@@ -154,7 +154,7 @@ __device__ __forceinline__ void run_quad(const QuadAddr& ad, const uint8_t* lds,
 constexpr float kFixedOne = 16777216.f;     // 2^24
 constexpr float kFixedLimit = 32768.f;      // 2^15: 255 such sums stay inside 47 bits
 template <int ACT>
-__device__ __forceinline__ void finish_row(const SlicedArgs& a, int m, uint32_t row, float v) {
+__device__ __forceinline__ void finish_row(const SlicedArgs& a, int m, uint32_t row, float v, float bias) {
   const size_t cell = (size_t)m * a.n + row;
   const bool fits = fabsf(v) < kFixedLimit;  // false for NaN and infinities
   unsigned long long add = 1ull;
@@ -174,7 +174,7 @@ __device__ __forceinline__ void finish_row(const SlicedArgs& a, int m, uint32_t 
   const unsigned long long total = old + add;
   float sum = (float)((double)((long long)total >> 16) * (1.0 / 16777216.0));  // exact product, one rounding
   if ((total >> 8) & 0xFFull) sum += __hip_atomic_exchange(a.spill + cell, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (a.bias) sum += a.bias[row];
+  sum += bias;  // requested before the atomic: a load issued here would add a memory round trip to the call's tail
   store_from_f32<ACT>((uint16_t*)a.y + (size_t)m * a.ldy, row, sum);
   __hip_atomic_store(a.sums + cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -340,8 +340,9 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     }
     __syncthreads();
     if ((uint32_t)tid < row_count) {
+      const float bias = a.bias ? a.bias[row_begin + (uint32_t)tid] : 0.f;
 #pragma unroll
-      for (int m = 0; m < M; ++m) finish_row<ACT>(a, m, row_begin + (uint32_t)tid, stage[m * kSlicedTasks + tid]);
+      for (int m = 0; m < M; ++m) finish_row<ACT>(a, m, row_begin + (uint32_t)tid, stage[m * kSlicedTasks + tid], bias);
     }
   } else if (row != kSlicedNoRow) {
 #pragma unroll
