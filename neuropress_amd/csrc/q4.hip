@@ -567,12 +567,14 @@ static int launch_q4_rowwise(const QCall& c) {
 }
 
 // The resident-grid kernel takes one token of a layer with at most 16 passes (K <= 65536) whose
-// per-block tables fit 64 KiB of LDS, when every block has at least five rows per wave to go
-// through: it then streams at the rate of a plain read (28672 x 4096: 14.6 us against 17.7 us
-// for the kernel above, whose every block restages x), while its longer start (x through LDS
-// before the first row can be contracted, two rows in flight per wave) loses on fewer rows
-// (14336 x 4096: 9.6 us both, 4096 x 4096: 6.4 against 5.2 us).  NPAMD_Q4_STREAM=2 takes it
-// wherever it fits, 0 never.  Blocks are as many as give every block the same number of rows.
+// per-block tables fit 64 KiB of LDS, from 64 Mi weights (32 MiB packed) up: it then streams at
+// the rate of a plain read, while the kernel above restages x in every block, and its longer
+// start (x through LDS before the first row can be contracted, two rows in flight per wave)
+// loses on less.  Measured, us per call, row-wise / resident: 11008 x 4096 8.6 / 9.3,
+// 16384 x 2048 8.4 / 8.7, 14336 x 4096 9.75 / 9.8, 8192 x 8192 10.8 / 10.7, 16384 x 4096
+// 11.9 / 10.2, 32768 x 2048 13.3 / 12.8, 24576 x 4096 15.6 / 12.7, 28672 x 4096 17.7 / 14.6.
+// NPAMD_Q4_STREAM=2 takes it wherever it fits, 0 never.  Blocks are as many as give every block
+// the same number of rows.
 static bool q4_stream_geometry(const QCall& c, Q4StreamGeom& geo) {
   geo.pairs = c.K / 64;
   geo.passes = (geo.pairs + 63) / 64;
@@ -585,7 +587,7 @@ static bool q4_stream_geometry(const QCall& c, Q4StreamGeom& geo) {
   geo.blocks = (row_groups + geo.iterations - 1) / geo.iterations;
   geo.row_stride = geo.blocks * geo.row_lanes;
   geo.waves = geo.row_lanes * geo.passes;
-  if (geo.iterations < 5 && tuning().q4_stream < 2) return false;
+  if ((int64_t)c.N * c.K < ((int64_t)64 << 20) && tuning().q4_stream < 2) return false;
   return (int64_t)geo.iterations * geo.row_lanes * geo.passes * 4 + geo.passes * 128 * kQ4StreamXStride <= 64 * 1024;
 }
 

@@ -353,6 +353,17 @@ def test_q4_stream_gemv(gpu, oracle_lib, monkeypatch, n, k, gs, asym):
     assert (y.float() - y_rowwise.float()).abs().max().item() <= 2e-3 * max(1.0, y.float().abs().max().item())
 
 
+@pytest.mark.parametrize("n,k", [(16384, 4096), (8192, 8192)])
+def test_q4_one_token_at_the_size_where_the_launcher_changes_kernel(gpu, oracle_lib, n, k):
+    """64 Mi weights: the smallest layers the launcher gives to the resident-grid kernel with
+    no variable set; one fp16 token against the oracle."""
+    from neuropress_amd import kernels
+
+    L = cases.q4_layer(77, n, k, gs=32, act=torch.float16, m=1, bias=True)
+    y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), 4, 32, None, L["bias"].to(gpu))
+    _check(y, _q_ref(oracle_lib, L, torch.float16))
+
+
 @pytest.mark.parametrize("asym", [False, True])
 def test_q4_rowwise_gemv_large_activations(gpu, asym):
     """Activations of a few hundred: the folded-out offset (72 * sum x) is then far larger than
