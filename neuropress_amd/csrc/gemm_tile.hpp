@@ -107,13 +107,14 @@ struct XStage {
   static constexpr int kLdsBytes = kBufs * kBufBytes + kWRing * kWBufBytes;  // the codebook copy follows
 };
 constexpr int kTileLdsCodebookMax = 64 * 1024;
+constexpr int kTileLdsResidualMax = 16 * 1024;
 constexpr int kLdsPerBlockMax = 160 * 1024;
 
 template <int ACT, class Provider, int MW, bool CB_LDS = false>
 __global__ void __launch_bounds__(512)
 tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  using XS = XStage<MW, CB_LDS>;
+  using XS = XStage<MW, CB_LDS && !Provider::kLdsResidual>;  // a residual table is small: no x tile given up
   constexpr int BM = 128 * MW;
   constexpr int kXBufBytes = XS::kBufBytes;
   uint8_t* const xs = lds;                             // [XS::kBufs][BM][XS::kXRowBytes]
@@ -235,7 +236,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
         // at its top, and with it their waits, the last of which is for the gathers issued one
         // step earlier.  (With the codebook in LDS the free schedule already waits for the
         // oldest load only, and is the faster one at 128 tokens.)
-        if constexpr (!CB_LDS) __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!CB_LDS || Provider::kLdsResidual) __builtin_amdgcn_sched_barrier(0);
       }
     }
     return;
@@ -448,7 +449,7 @@ int launch_tile_gemm_mw_cb(const GemmShape& s, const typename Provider::Args& pa
                            const char* what) {
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kTileCols - 1) / kTileCols, (s.M + BM - 1) / BM, s.splits);
-  const int lds = XStage<MW, CB_LDS>::kLdsBytes + (CB_LDS ? cb_bytes : 0);
+  const int lds = XStage<MW, CB_LDS && !Provider::kLdsResidual>::kLdsBytes + (CB_LDS ? cb_bytes : 0);
   static LdsLatch latch;  // per instantiation
   const hipError_t e =
       enable_dynamic_lds(latch, reinterpret_cast<const void*>(&tile_gemm_kernel<ACT, Provider, MW, CB_LDS>), lds);
@@ -467,6 +468,13 @@ int launch_tile_gemm_mw_cb(const GemmShape& s, const typename Provider::Args& pa
 template <int ACT, class Provider, int MW>
 int launch_tile_gemm_mw(const GemmShape& s, const typename Provider::Args& pargs, int cb_bytes, hipStream_t st,
                         const char* what) {
+  if constexpr (Provider::kLdsResidual) {
+    // Residual VQ: cb_bytes is the residual codebook; behind the tiles it takes half of the
+    // producers' lookups off the vector memory path at every token count.
+    if (cb_bytes > 0 && cb_bytes <= kTileLdsResidualMax && cb_bytes % 16 == 0 &&
+        XStage<MW, false>::kLdsBytes + cb_bytes <= kLdsPerBlockMax && tile_lds_codebook_enabled())
+      return launch_tile_gemm_mw_cb<ACT, Provider, MW, true>(s, pargs, cb_bytes, st, what);
+  }
   if constexpr (Provider::kLdsCodebook && MW < 3) {
     // At 129..256 tokens the copy costs the third x tile: worth it only for tables the vector L1
     // does not hold anyway (14336 x 4096 at 256 tokens: 4096 rows 64 -> 57 us, 256 rows 49 -> 53 us).

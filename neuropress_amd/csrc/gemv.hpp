@@ -230,6 +230,7 @@ GemvPlan plan_gemv(int N, int chunks, int max_r = 4, int max_waves_cap = 16);
 
 // Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
+constexpr int kGemvLdsResidualMax = 16 * 1024;   // residual codebooks of up to 1024 rows
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
 bool gemv_lds_activations_forced();  // NPAMD_GEMV_LDS_X=1: stage x in LDS also without a permutation (tuning aid)
 
@@ -266,6 +267,21 @@ template <int ACT, class Provider>
 int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStream_t st,
                       const char* what, int cb_bytes = 0) {
   s.steps = (s.chunks + 3) / 4;
+  if constexpr (Provider::kLdsResidual) {
+    // Residual VQ: cb_bytes is the residual codebook.  In LDS its lookups leave the vector memory
+    // path to the main codebook's; row tiles per block stay at two, as for every provider that
+    // looks up in memory.
+    if (cb_bytes > 0 && cb_bytes <= kGemvLdsResidualMax && gemv_lds_codebook_enabled()) {
+      if (s.M > 16) {
+        const GemvPlan plan = plan_gemv(s.N, s.chunks, 2, 8);
+        if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
+        return launch_fused_gemv_r<ACT, Provider, 1, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
+      }
+      const GemvPlan plan = plan_gemv(s.N, s.chunks, 2);
+      if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true>(s, pargs, plan, cb_bytes, st, what);
+      return launch_fused_gemv_r<ACT, Provider, 1, true>(s, pargs, plan, cb_bytes, st, what);
+    }
+  }
   bool cb_in_lds = false;
   if constexpr (Provider::kLdsCodebook)
     cb_in_lds = cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled();

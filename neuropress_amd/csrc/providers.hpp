@@ -57,6 +57,7 @@ struct VqProvider {
     u32x4 idx_hi;  // indices 8..15 (VL = 4 only)
   };
   static constexpr bool kLdsCodebook = true;  // the codebook may be staged in LDS (use_codebook)
+  static constexpr bool kLdsResidual = false;
   static constexpr bool kGathers = true;  // operands are codebook lookups, not arithmetic on the packed bytes
   const Args& a;
   const u32x4* cb;  // where operands are gathered from: global memory, or an LDS copy
@@ -151,9 +152,17 @@ struct RvqProvider {
     uint32_t s2, b2;  // scale / bias replicated in both halves
   };
   static constexpr bool kLdsCodebook = false;
+  // The GEMV can keep the residual codebook (4 KiB at 256 rows) in LDS: lookups through the
+  // vector memory path cost one cache-tag cycle per lane whether they hit or not, and the
+  // residual's are half of them.  The main codebook stays in memory.
+  static constexpr bool kLdsResidual = true;
   static constexpr bool kGathers = true;  // operands are codebook lookups, not arithmetic on the packed bytes
   const Args& a;
-  __device__ explicit RvqProvider(const Args& args) : a(args) {}
+  const u32x4* cbr;  // where residual rows are looked up: global memory, or an LDS copy
+  __device__ explicit RvqProvider(const Args& args) : a(args), cbr(args.cb_r) {}
+  __device__ __forceinline__ void use_codebook(const u32x4* p) { cbr = p; }
+  __device__ __forceinline__ const u32x4* global_codebook() const { return a.cb_r; }
+  __device__ __forceinline__ int codebook_vec16() const { return (int)a.ncr_minus_1 + 1; }
 
   __device__ __forceinline__ void load(Raw& r, int n, int kc) const {
     const int64_t i0 = ((int64_t)n * a.chunks + kc) * 8;
@@ -187,14 +196,14 @@ struct RvqProvider {
   struct PairOps {
     u32x4 cm0, cr0, cm1, cr1;  // main and residual rows of the two operands, as gathered
   };
-  static constexpr int kLdsOpsPerGather = 0;  // both codebooks are gathered from memory
+  static constexpr int kLdsOpsPerGather = 2;  // with the residual codebook in LDS: its two lookups
   __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o) const {
     const uint32_t pm = select_dword(extract_idx8<BITS_M>(r.wm), jp);
     const uint32_t pr = select_dword(extract_idx8<BITS_R>(r.wr), jp);
     o.cm0 = a.cb_m[min(pm & 0xFFFFu, a.ncm_minus_1)];
-    o.cr0 = a.cb_r[min(pr & 0xFFFFu, a.ncr_minus_1)];
     o.cm1 = a.cb_m[min(pm >> 16, a.ncm_minus_1)];
-    o.cr1 = a.cb_r[min(pr >> 16, a.ncr_minus_1)];
+    o.cr0 = cbr[min(pr & 0xFFFFu, a.ncr_minus_1)];
+    o.cr1 = cbr[min(pr >> 16, a.ncr_minus_1)];
   }
   __device__ __forceinline__ void finish_pair(const PairOps& o, u32x4& b0, u32x4& b1) const {
     b0 = combine_rows(o.cm0, o.cr0, s2, b2);
@@ -202,7 +211,7 @@ struct RvqProvider {
   }
 
   __device__ __forceinline__ u32x4 combine(uint32_t im, uint32_t ir, uint32_t s2, uint32_t b2) const {
-    return combine_rows(a.cb_m[min(im, a.ncm_minus_1)], a.cb_r[min(ir, a.ncr_minus_1)], s2, b2);
+    return combine_rows(a.cb_m[min(im, a.ncm_minus_1)], cbr[min(ir, a.ncr_minus_1)], s2, b2);
   }
   __device__ __forceinline__ u32x4 combine_rows(const u32x4& cm, const u32x4& cr, uint32_t s2, uint32_t b2) const {
 #pragma clang fp contract(off)
@@ -252,6 +261,7 @@ struct Q4Provider {
     uint32_t z_lo, z_hi;  // zero points (fp16 bits) of the same two groups (ASYM only)
   };
   static constexpr bool kLdsCodebook = false;
+  static constexpr bool kLdsResidual = false;
   static constexpr bool kGathers = false;  // operands are codebook lookups, not arithmetic on the packed bytes
   const Args& a;
   __device__ explicit Q4Provider(const Args& args) : a(args) {}
@@ -368,6 +378,7 @@ struct Q8Provider {
     uint32_t z_lo, z_hi;  // zero points (fp16 bits), ASYM only
   };
   static constexpr bool kLdsCodebook = false;
+  static constexpr bool kLdsResidual = false;
   static constexpr bool kGathers = false;  // operands are arithmetic on the packed bytes
   const Args& a;
   __device__ explicit Q8Provider(const Args& args) : a(args) {}

@@ -41,7 +41,7 @@ int run_rvq(const VqCall& c, const GemmShape& s) {
   typename P::Args a{c.packed, c.packed_r, (const u32x4*)c.cb, (const u32x4*)c.cb_r,
                      (const uint16_t*)c.row_scale, (const uint16_t*)c.row_bias,
                      (uint32_t)c.nc - 1u, (uint32_t)c.nc_r - 1u, s.chunks};
-  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
+  return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes, c.nc_r * 16);
 }
 
 template <int ACT>

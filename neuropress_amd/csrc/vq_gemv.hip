@@ -40,7 +40,7 @@ int run_rvq(const VqCall& c, const GemvShape& s) {
   typename P::Args a{c.packed, c.packed_r, (const u32x4*)c.cb, (const u32x4*)c.cb_r,
                      (const uint16_t*)c.row_scale, (const uint16_t*)c.row_bias,
                      (uint32_t)c.nc - 1u, (uint32_t)c.nc_r - 1u, s.chunks};
-  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what);
+  return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, c.nc_r * 16);
 }
 
 template <int ACT>

@@ -297,6 +297,19 @@ def test_rvq_linear(gpu, oracle_lib, act, m, tile):
     _check(y, _rvq_ref(oracle_lib, L, act))
 
 
+@pytest.mark.parametrize("nc_main,nc_res", [(65536, 200), (65536, 40000), (4096, 256), (256, 130)])
+@pytest.mark.parametrize("m", [1, 20])
+def test_rvq_gemv_residual_table_sizes(gpu, oracle_lib, nc_main, nc_res, m):
+    """The fused GEMV keeps a small residual codebook in LDS (a table that is not a power of two
+    long included) and looks a large one up in memory; both against the oracle."""
+    from neuropress_amd import kernels
+
+    L = cases.rvq_layer(400 + nc_res, 96, 512, nc_main=nc_main, nc_res=nc_res, act=torch.float16, m=m)
+    y = kernels.rvq_linear(L["x"].to(gpu), L["pm"].to(gpu), L["bm"], L["pr"].to(gpu), L["br"], L["cbm"].to(gpu),
+                           L["cbr"].to(gpu), L["scale"].to(gpu), L["wbias"].to(gpu), 96, None, tile=False)
+    _check(y, _rvq_ref(oracle_lib, L, torch.float16))
+
+
 def _q_ref(oracle_lib, L, act):
     code = orc.torch_dtype_code(act)
     w = oracle_lib.q_decode(L["blob"].numpy(), orc.to_bits(L["scale"]),
