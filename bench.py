@@ -424,7 +424,7 @@ def main():
     # ---------------- sweep over the other bands / configs ----------------------
     # Every row: the call timed as above, and the same call's output checked against the dense
     # product of the decoded weight in f32 (the decode kernels are bit-exact against the oracle,
-    # tested): max abs error, its largest ratio to the bound 1e-2 + 1e-2 |ref|, and the verdict.
+    # tested): max abs error, its largest ratio to the bound 1e-2 + 1e-2 |ref|, and whether it holds.
     sweep = []
     if not args.no_sweep:
         def check(y, ref):
