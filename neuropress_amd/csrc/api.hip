@@ -49,6 +49,7 @@ static Tuning read_tuning() {
   t.gemv_lds_x = env_int("NPAMD_GEMV_LDS_X", 0);
   t.gemv_r = env_int("NPAMD_GEMV_R", 0);
   t.gemv_spw = env_int("NPAMD_GEMV_SPW", 0);
+  t.gemv_parts = env_int("NPAMD_GEMV_PARTS", 0);
   t.tile_splits = env_int("NPAMD_TILE_SPLITS", 0);
   t.tile_mw = env_int("NPAMD_TILE_MW", 0);
   t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
@@ -111,6 +112,43 @@ GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {
   int max_waves = p.R >= 4 ? 8 : 16;
   if (max_waves > max_waves_cap) max_waves = max_waves_cap;
   if ((steps + spw - 1) / spw > max_waves) spw = (steps + max_waves - 1) / max_waves;
+  p.steps_per_wave = spw;
+  p.waves = (steps + spw - 1) / spw;
+  return p;
+}
+
+// Measured, one token, 16 rows per block against 8 / 4 (us): residual VQ 1024 x 4096 7.7 -> 4.4,
+// 65536-row codebook 1024 x 4096 8.4 -> 4.8 and 2048 x 4096 9.2 -> 7.1, int4 1024 x 4096 at two
+// tokens 5.8 -> 3.8, 2048 x 8192 with a 4096-row table in LDS 6.5 -> 5.4; but 2048 x 2048 and
+// 512 x 2048 with that table 4.5 -> 5.2 and 4.4 -> 6.7 (every block copies the 64 KiB first, and
+// there are then two or four times as many), 2048 x 640 3.2 -> 3.3.  Hence: K of at least 1024
+// per part, and a block must keep at least two lookups per row of the table it copies.
+int plan_gemv_parts(int M, int N, int chunks, int lds_rows) {
+  const int env = tuning().gemv_parts;
+  const int cus = device_cu_count();
+  int h = 1;
+  while (h < 4) {
+    const int next = 2 * h;
+    const int tiles = (N + 16 / h - 1) / (16 / h);
+    const bool fits = M <= 16 / next && chunks >= 16 * next;
+    const bool wanted = tiles * 4 < cus * 3;
+    const bool pays = (int64_t)(16 / next) * chunks * 8 >= 2 * (int64_t)lds_rows;
+    if (!(fits && wanted && pays)) break;
+    h = next;
+  }
+  if (env == 1 || env == 2 || env == 4) h = (M <= 16 / env) ? env : 1;
+  return h;
+}
+
+GemvPlan plan_gemv_rows(int N, int rows, int steps) {
+  const int tiles = (N + rows - 1) / rows;
+  const int64_t jobs = (int64_t)tiles * steps;
+  const int64_t target_waves = (int64_t)device_cu_count() * 16;
+  int spw = (int)((jobs + target_waves - 1) / target_waves);
+  if (spw < 1) spw = 1;
+  if ((steps + spw - 1) / spw > 16) spw = (steps + 15) / 16;
+  GemvPlan p;
+  p.R = 1;
   p.steps_per_wave = spw;
   p.waves = (steps + spw - 1) / spw;
   return p;

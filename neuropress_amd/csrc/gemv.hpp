@@ -13,7 +13,8 @@
 //
 // Work split: a "chunk" is 64 k of one row (8 operands); one "step" is the 4
 // k-slots of a wave = 256 k.  A block owns 16*R rows and all of K; its S waves
-// split the steps and their partial tiles are summed through LDS.
+// split the steps and their partial tiles are summed through LDS.  (Layers of
+// few rows: 16 / H rows per block and H parts of k per k-slot, see the kernel.)
 #pragma once
 
 #include <atomic>
@@ -55,9 +56,16 @@ constexpr int kGemvMaxWaves = (R >= 4 || MT >= 2) ? 8 : 16;
 // column permutation s.perm on the way when there is one, and reads its A
 // operands from there: the gather x[m, perm[k]] costs K element loads per block
 // instead of a kernel of its own in front of this one.
-template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS, int MT = 1>
+// H > 1 (layers of few rows, at most 16 / H tokens): the 16 columns of the MFMA tile are 16 / H
+// weight rows x H parts of k, and A carries the matching part of x in the row of the same
+// number, so D[m'][n'] is a wanted partial sum where m' and n' name the same part and is
+// ignored elsewhere.  A block then owns 16 / H rows: H times the blocks, each with 1 / H of the
+// lookups, for layers that would leave most compute units without a block.
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS, int MT = 1, int H = 1>
 __global__ void __launch_bounds__((kGemvMaxWaves<R, MT> * 64))
 fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
+  static_assert(H == 1 || ((H == 2 || H == 4) && R == 1 && MT == 1), "k parts only with one row tile and one token tile");
+  constexpr int RT = 16 / H;  // weight rows (and tokens) per MFMA tile
   extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][M][16*R] (+ codebook copy)
   Provider prov(pargs);
   const int lane = threadIdx.x & 63;
@@ -118,7 +126,8 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   if constexpr (CB_LDS || X_LDS) __syncthreads();
   const int c = lane & 15;
   const int q = lane >> 4;
-  const int row0 = blockIdx.x * (16 * R);
+  const int cr = c & (RT - 1), part = c / RT;  // H = 1: cr = c, part = 0
+  const int row0 = blockIdx.x * (RT * R);
 
   f32x4 acc[R][MT];
 #pragma unroll
@@ -135,21 +144,21 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   bool x_lane[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int x_row = min(16 * t + c, s.M - 1);
+    const int x_row = min(16 * t + cr, s.M - 1);
     xrow[t] = X_LDS ? x_lds + (int64_t)x_row * (s.chunks * 64)
                     : reinterpret_cast<const uint16_t*>(s.x) + (int64_t)x_row * s.ldx;
-    x_lane[t] = 16 * t + c < s.M;
+    x_lane[t] = 16 * t + cr < s.M;
   }
   const u32x4 zero4{0, 0, 0, 0};
 
   for (int step = step_begin; step < step_end; ++step) {
-    const int kc_raw = step * 4 + q;
+    const int kc_raw = (step * 4 + q) * H + part;
     const bool kvalid = kc_raw < s.chunks;
     const int kc = min(kc_raw, s.chunks - 1);
 
     typename Provider::Raw raw[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) prov.load(raw[r], min(row0 + 16 * r + c, s.N - 1), kc);
+    for (int r = 0; r < R; ++r) prov.load(raw[r], min(row0 + 16 * r + cr, s.N - 1), kc);
 
     u32x4 xa[MT][8];
 #pragma unroll
@@ -175,7 +184,7 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
       b[r][6] = prov.template operand<6>(raw[r]);
       b[r][7] = prov.template operand<7>(raw[r]);
     }
-    if (s.chunks & 3) {  // uniform: only shapes with a ragged last step pay for the select
+    if (s.chunks % (4 * H)) {  // uniform: only shapes with a ragged last step pay for the select
 #pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -191,15 +200,19 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
 
   if constexpr (kRedOverCodebook) __syncthreads();  // every wave is done with the codebook
   // D layout: lane (c, q) holds D[m = 16t + 4q + i][n = c], i = 0..3, for token tile t.
-  const int cols = 16 * R;
+  // With k parts: D row m' = 4q + i is token m' % RT of part m' / RT, wanted where that is the
+  // lane's own part; every (wave, part) files its sums as one more partial tile.
+  const int cols = RT * R;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int m = 16 * t + 4 * q + i;
-        if (m < s.M) red[((int64_t)wave * s.M + m) * cols + r * 16 + c] = acc[r][t][i];
+        const int mp = 4 * q + i;
+        const int m = 16 * t + (mp & (RT - 1));
+        if (m < s.M && mp / RT == part)
+          red[((int64_t)(wave * H + part) * s.M + m) * cols + r * 16 + cr] = acc[r][t][i];
       }
   }
   __syncthreads();
@@ -209,7 +222,7 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
     const int n = row0 + col;
     if (n >= s.N) continue;
     float v = 0.f;
-    for (int w = 0; w < n_waves; ++w) v += red[((int64_t)w * s.M + m) * cols + col];
+    for (int w = 0; w < n_waves * H; ++w) v += red[((int64_t)w * s.M + m) * cols + col];
     if (s.bias) v += s.bias[n];
     store_from_f32<ACT>(s.y, (int64_t)m * s.ldy + n, v);
   }
@@ -227,6 +240,12 @@ struct GemvPlan {
 // max_r: most row tiles per block the caller wants (4, or 2 for lookups served by L2);
 // max_waves_cap: most waves per block its kernel variant is built for.
 GemvPlan plan_gemv(int N, int chunks, int max_r = 4, int max_waves_cap = 16);
+// k parts per MFMA tile (1, 2 or 4) for M tokens on an N-row layer: more than one only where
+// whole 16-row tiles would leave most compute units without a block.  NPAMD_GEMV_PARTS overrides.
+// lds_rows: rows of the table every block copies into LDS first (0: none).
+int plan_gemv_parts(int M, int N, int chunks, int lds_rows);
+// One row tile of `rows` rows per block, `steps` steps to split over its waves.
+GemvPlan plan_gemv_rows(int N, int rows, int steps);
 
 // Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
@@ -234,11 +253,11 @@ constexpr int kGemvLdsResidualMax = 16 * 1024;   // residual codebooks of up to 
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
 bool gemv_lds_activations_forced();  // NPAMD_GEMV_LDS_X=1: stage x in LDS also without a permutation (tuning aid)
 
-template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false, int MT = 1>
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false, int MT = 1, int H = 1>
 int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const GemvPlan& plan,
                         int cb_bytes, hipStream_t st, const char* what) {
   s.steps_per_wave = plan.steps_per_wave;
-  const int blocks = (s.N + 16 * R - 1) / (16 * R);
+  const int blocks = (s.N + 16 / H * R - 1) / (16 / H * R);
   const int red_bytes = ((plan.waves * s.M * 16 * R + 3) & ~3) * (int)sizeof(float);
   const int x_bytes = X_LDS ? s.M * s.chunks * 64 * 2 : 0;
   const int cb_lds_bytes = CB_LDS ? cb_bytes : 0;
@@ -249,11 +268,11 @@ int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const
   if (lds > 64 * 1024) {
     static LdsLatch latch;  // per instantiation
     const hipError_t e = enable_dynamic_lds(
-        latch, reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT>), lds);
+        latch, reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H>), lds);
     if (e != hipSuccess)
       return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
   }
-  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
+  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);
 }
 
@@ -267,6 +286,25 @@ template <int ACT, class Provider>
 int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStream_t st,
                       const char* what, int cb_bytes = 0) {
   s.steps = (s.chunks + 3) / 4;
+  // Layers of few rows, few tokens: 16 / H rows x H parts of k per tile (see the kernel).
+  bool lds_table = false;
+  if constexpr (Provider::kLdsResidual)
+    lds_table = cb_bytes > 0 && cb_bytes <= kGemvLdsResidualMax && gemv_lds_codebook_enabled();
+  if constexpr (Provider::kLdsCodebook)
+    lds_table = cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled();
+  if (const int h = plan_gemv_parts(s.M, s.N, s.chunks, lds_table ? cb_bytes / 16 : 0);
+      h > 1 && !s.perm && !gemv_lds_activations_forced()) {
+    s.steps = (s.chunks + 4 * h - 1) / (4 * h);
+    const GemvPlan plan = plan_gemv_rows(s.N, 16 / h, s.steps);
+    if constexpr (Provider::kLdsResidual || Provider::kLdsCodebook) {
+      if (lds_table) {
+        if (h == 4) return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 4>(s, pargs, plan, cb_bytes, st, what);
+        return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 2>(s, pargs, plan, cb_bytes, st, what);
+      }
+    }
+    if (h == 4) return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 4>(s, pargs, plan, 0, st, what);
+    return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 2>(s, pargs, plan, 0, st, what);
+  }
   if constexpr (Provider::kLdsResidual) {
     // Residual VQ: cb_bytes is the residual codebook.  In LDS its lookups leave the vector memory
     // path to the main codebook's; row tiles per block stay at two, as for every provider that

@@ -491,6 +491,91 @@ def test_fused_kernels_decode_bit_exactly(gpu, act, kind):
     assert torch.equal(tile(eye[100:330]), wt[100:330]), "tile GEMM, 230 tokens"
 
 
+@pytest.fixture
+def gemv_parts(monkeypatch):
+    """Sets NPAMD_GEMV_PARTS (rows of an MFMA tile traded for parts of k) for one test; the
+    library reads its tuning variables once, so they are re-read on the way in and out."""
+    from neuropress_amd import _lib
+
+    def force(parts: int):
+        monkeypatch.setenv("NPAMD_GEMV_PARTS", str(parts))
+        _lib.load().npamd_diag_reload_tuning()
+
+    yield force
+    monkeypatch.delenv("NPAMD_GEMV_PARTS", raising=False)
+    _lib.load().npamd_diag_reload_tuning()
+
+
+@pytest.mark.parametrize("parts,m", [(2, 1), (2, 5), (2, 8), (4, 1), (4, 3), (4, 4), (4, 7), (2, 12)])
+@pytest.mark.parametrize("n,k", [(37, 192), (100, 1088), (8, 64), (260, 4160)])
+@pytest.mark.parametrize("kind", ["vq8", "vq12", "vq16_bf16", "vq12_vl4", "rvq", "q4", "q4_asym", "q8"])
+def test_gemv_rows_traded_for_k_parts(gpu, oracle_lib, gemv_parts, kind, n, k, parts, m):
+    """The fused GEMV with 8 or 4 rows x 2 or 4 parts of k per MFMA tile (taken by itself for
+    layers of few rows; forced here): row counts that do not fill a tile, K of one chunk, K whose
+    chunks do not fill the last step, every token count a tile holds — and one above
+    (7 tokens at four parts, 12 at two), which must fall back to whole tiles.  Table in LDS
+    (256 and 4096 rows, the residual's 256) and in memory (65536 rows)."""
+    from neuropress_amd import kernels
+
+    gemv_parts(parts)
+    if kind.startswith("vq"):
+        bits = int(kind[2:].split("_")[0])
+        act = torch.bfloat16 if kind.endswith("bf16") else torch.float16
+        vl = 4 if kind.endswith("vl4") else 8
+        L = cases.vq_layer(300 + bits + m, n, k, 1 << bits, vl=vl, bits=bits, act=act, m=m, bias=True)
+        y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, vl, L["bias"].to(gpu), n)
+        ref = _vq_ref(oracle_lib, L, act)
+    elif kind == "rvq":
+        L = cases.rvq_layer(310 + m, n, k, act=torch.float16, m=m)
+        y = kernels.rvq_linear(L["x"].to(gpu), L["pm"].to(gpu), L["bm"], L["pr"].to(gpu), L["br"], L["cbm"].to(gpu),
+                               L["cbr"].to(gpu), L["scale"].to(gpu), L["wbias"].to(gpu), n, None, tile=False)
+        ref = _rvq_ref(oracle_lib, L, torch.float16)
+    else:
+        nbits = int(kind[1])
+        L = cases.q4_layer(320 + m, n, k, nbits=nbits, gs=32, act=torch.float16, m=m, asym="asym" in kind, bias=True)
+        zp = None if L["zp"] is None else L["zp"].to(gpu)
+        y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), nbits, 32, zp, L["bias"].to(gpu))
+        ref = _q_ref(oracle_lib, L, torch.float16)
+    assert y.shape == (m, n)
+    _check(y, ref)
+
+
+@pytest.mark.parametrize("parts", [2, 4])
+@pytest.mark.parametrize("kind", ["vq12", "vq16", "rvq", "q4"])
+def test_gemv_k_parts_decode_bit_exactly(gpu, gemv_parts, kind, parts):
+    """One-hot activations through the k-parts GEMV: y[m, n] is the single product 1 * W[n, k_m],
+    so every (row, part, k slot) of the tile layout must land where the one-pass decode has it."""
+    from neuropress_amd import kernels
+
+    n, k, act = 45, 1024, torch.float16
+    if kind.startswith("vq"):
+        bits = int(kind[2:])
+        L = cases.vq_layer(340 + bits, n, k, 1 << bits, bits=bits, act=act, m=1, std=0.05)
+        pk, cb = L["packed"].to(gpu), L["cb"].to(gpu)
+        w = kernels.vq_dequant(pk, cb, bits, n, k, act)
+        gemv = lambda x: kernels.vq_linear(x, pk, cb, bits, 8, None, n)
+    elif kind == "rvq":
+        L = cases.rvq_layer(341, n, k, act=act, m=1)
+        d = {key: (v.to(gpu) if torch.is_tensor(v) else v) for key, v in L.items()}
+        args = (d["pm"], L["bm"], d["pr"], L["br"], d["cbm"], d["cbr"], d["scale"], d["wbias"], n)
+        w = kernels.rvq_dequant(*args, k, act)
+        gemv = lambda x: kernels.rvq_linear(x, *args, None, tile=False)
+    else:
+        L = cases.q4_layer(342, n, k, act=act, m=1)
+        blob, sc = L["blob"].to(gpu), L["scale"].to(gpu)
+        w = kernels.q_dequant(blob, sc, 4, 32, None, act)
+        gemv = lambda x: kernels.q_linear(x, blob, sc, 4, 32, None)
+    gemv_parts(parts)
+    eye = torch.eye(k, dtype=act, device=gpu)
+    wt = w.t().contiguous()
+    tokens = 16 // parts
+    for k0 in range(0, k, 8 * tokens // 2 + 24):  # windows that straddle chunks and steps
+        k1 = min(k0 + tokens, k)
+        if kind == "q4" and k1 - k0 < 2:
+            continue  # one token of int4 takes the row-wise kernel
+        assert torch.equal(gemv(eye[k0:k1]), wt[k0:k1]), f"tokens one-hot at {k0}..{k1}"
+
+
 @pytest.mark.parametrize("nbits,gs,asym", [(4, 32, True), (8, 32, False), (2, 16, True), (1, 8, False), (4, 24, False)])
 @pytest.mark.parametrize("m", [2, 20])
 def test_q_linear_generic_path(gpu, oracle_lib, nbits, gs, asym, m):
