@@ -118,11 +118,13 @@ GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {
 }
 
 // Measured, one token, 16 rows per block against 8 / 4 (us): residual VQ 1024 x 4096 7.7 -> 4.4,
-// 65536-row codebook 1024 x 4096 8.4 -> 4.8 and 2048 x 4096 9.2 -> 7.1, int4 1024 x 4096 at two
-// tokens 5.8 -> 3.8, 2048 x 8192 with a 4096-row table in LDS 6.5 -> 5.4; but 2048 x 2048 and
-// 512 x 2048 with that table 4.5 -> 5.2 and 4.4 -> 6.7 (every block copies the 64 KiB first, and
-// there are then two or four times as many), 2048 x 640 3.2 -> 3.3.  Hence: K of at least 1024
-// per part, and a block must keep at least two lookups per row of the table it copies.
+// 65536-row codebook 1024 x 4096 8.4 -> 4.8, 2048 x 4096 9.2 -> 7.1 and 1024 x 1024 3.8 -> 3.3,
+// int4 1024 x 4096 at two tokens 5.8 -> 3.8, 2048 x 8192 with a 4096-row table in LDS 6.5 -> 5.5,
+// 2048 x 4096 with it 5.0 -> 4.5; but 2048 x 2048 and 512 x 2048 with that table 4.2 -> 4.4 and
+// 4.15 -> 4.9 (every block copies the 64 KiB first, and there are then two or four times as
+// many), 4096 x 4096 (whole tiles cover the compute units) 5.3 -> 5.5.  Hence: K of at least 512
+// per part, whole tiles leave a quarter of the compute units empty, and a block keeps at least
+// one lookup per row of the table it copies.
 int plan_gemv_parts(int M, int N, int chunks, int lds_rows) {
   const int env = tuning().gemv_parts;
   const int cus = device_cu_count();
@@ -130,9 +132,9 @@ int plan_gemv_parts(int M, int N, int chunks, int lds_rows) {
   while (h < 4) {
     const int next = 2 * h;
     const int tiles = (N + 16 / h - 1) / (16 / h);
-    const bool fits = M <= 16 / next && chunks >= 16 * next;
+    const bool fits = M <= 16 / next && chunks >= 8 * next;
     const bool wanted = tiles * 4 < cus * 3;
-    const bool pays = (int64_t)(16 / next) * chunks * 8 >= 2 * (int64_t)lds_rows;
+    const bool pays = (int64_t)(16 / next) * chunks * 8 >= (int64_t)lds_rows;
     if (!(fits && wanted && pays)) break;
     h = next;
   }

@@ -118,9 +118,21 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
     x_lds = xs;
   }
   if constexpr (CB_LDS) {
+    // Four requests per thread in flight: a block of few waves (short K) would otherwise copy
+    // the table one round trip per 16 bytes and thread.
     u32x4* cb_lds = reinterpret_cast<u32x4*>(lds0);
     const u32x4* src = prov.global_codebook();
-    for (int i = threadIdx.x; i < prov.codebook_vec16(); i += blockDim.x) cb_lds[i] = src[i];
+    const int n16 = prov.codebook_vec16();
+    constexpr int kBatch = 4;
+    for (int base = threadIdx.x; base < n16; base += (int)blockDim.x * kBatch) {
+      u32x4 t[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j)
+        if (base + j * (int)blockDim.x < n16) t[j] = src[base + j * (int)blockDim.x];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j)
+        if (base + j * (int)blockDim.x < n16) cb_lds[base + j * (int)blockDim.x] = t[j];
+    }
     prov.use_codebook(cb_lds);
   }
   if constexpr (CB_LDS || X_LDS) __syncthreads();
@@ -292,8 +304,22 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
     lds_table = cb_bytes > 0 && cb_bytes <= kGemvLdsResidualMax && gemv_lds_codebook_enabled();
   if constexpr (Provider::kLdsCodebook)
     lds_table = cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled();
-  if (const int h = plan_gemv_parts(s.M, s.N, s.chunks, lds_table ? cb_bytes / 16 : 0);
-      h > 1 && !s.perm && !gemv_lds_activations_forced()) {
+  int h = plan_gemv_parts(s.M, s.N, s.chunks, lds_table ? cb_bytes / 16 : 0);
+  bool whole_codebook_in_lds = lds_table && Provider::kLdsCodebook;
+  if (whole_codebook_in_lds && s.M <= 16 && !s.perm && !gemv_lds_activations_forced()) {
+    // A block that has few lookups to make does them in memory rather than copy the table first:
+    // with as many parts as the layer admits when nothing is copied, up to 2048 lookups per
+    // block.  One token, 4096-row table, copy / memory at the parts each admits (us): 512 x 2048
+    // 4.15 / 3.0, 2048 x 2048 4.2 / 3.85, 1024 x 1024 4.2 / 3.05, 1024 x 4096 4.4 / 3.95; above the
+    // limit 2048 x 4096 4.5 / 5.3, 2048 x 8192 5.5 / 8.6, 512 x 8192 4.5 / 4.8; 1024-row table
+    // 1024 x 2048 3.5 / 3.0; 256-row table 1024 x 4096 3.5 / 3.4, 512 x 512 2.95 / 2.7.
+    const int h_mem = plan_gemv_parts(s.M, s.N, s.chunks, 0);
+    if ((int64_t)16 * s.chunks * 8 / h_mem <= 2048) {
+      h = h_mem;
+      lds_table = whole_codebook_in_lds = false;
+    }
+  }
+  if (h > 1 && !s.perm && !gemv_lds_activations_forced()) {
     s.steps = (s.chunks + 4 * h - 1) / (4 * h);
     const GemvPlan plan = plan_gemv_rows(s.N, 16 / h, s.steps);
     if constexpr (Provider::kLdsResidual || Provider::kLdsCodebook) {
@@ -320,9 +346,7 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
       return launch_fused_gemv_r<ACT, Provider, 1, true>(s, pargs, plan, cb_bytes, st, what);
     }
   }
-  bool cb_in_lds = false;
-  if constexpr (Provider::kLdsCodebook)
-    cb_in_lds = cb_bytes > 0 && cb_bytes <= kGemvLdsCodebookMax && gemv_lds_codebook_enabled();
+  const bool cb_in_lds = whole_codebook_in_lds;
   // Lookups that go to L2 want many waves in flight more than they want shared x operands
   // (14336 x 4096, 65536-row codebook, one token: 34.6 us with two row tiles, 37.2 with four).
   if (s.M > 16) {
