@@ -50,6 +50,7 @@ static Tuning read_tuning() {
   t.gemv_r = env_int("NPAMD_GEMV_R", 0);
   t.gemv_spw = env_int("NPAMD_GEMV_SPW", 0);
   t.gemv_parts = env_int("NPAMD_GEMV_PARTS", 0);
+  t.gemv_xstage = env_int("NPAMD_GEMV_XSTAGE", 1);
   t.tile_splits = env_int("NPAMD_TILE_SPLITS", 0);
   t.tile_mw = env_int("NPAMD_TILE_MW", 0);
   t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
@@ -88,6 +89,14 @@ static int device_cu_count() {
 bool gemv_lds_codebook_enabled() { return tuning().gemv_lds_cb != 0; }
 bool tile_lds_codebook_enabled() { return tuning().tile_lds_cb != 0; }
 bool gemv_lds_activations_forced() { return tuning().gemv_lds_x != 0; }
+// One token tile, one row tile, us, straight from memory / staged: int4 4096 x 4096 7.75 / 7.1 at 8
+// tokens, 9.2 / 7.8 at 16, 13.2 / 10.8 at 32; 4096 x 14336 27.5 / 19.7 at 16, 38.7 / 27.6 at 32;
+// 65536-row codebook 4096 x 14336 42.4 / 38.4 at 16, 52 / 42 at 32; but int4 1024 x 4096 5.8 / 6.2
+// at 8 tokens.  With more row tiles per block (14336 x 4096) or the table in LDS it does not pay.
+bool gemv_stage_activations(int M) {
+  const int mode = tuning().gemv_xstage;
+  return mode >= 2 || (mode == 1 && M >= 9);
+}
 
 GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {
   const int steps = (chunks + 3) / 4;

@@ -36,6 +36,7 @@ struct GemvShape {
   // Optional gather of the activation columns: the kernel contracts x[m, perm[k]] with W[n, k].
   // Only with the X_LDS variant (every block first copies the permuted rows of x into LDS).
   const int32_t* perm = nullptr;
+  int stage_offset = 0;  // XS kernels: byte offset of the waves' activation staging areas in LDS
 };
 
 // Largest M * K (elements) whose activations the GEMV stages in LDS (32 KiB; the unpermuted
@@ -61,10 +62,19 @@ constexpr int kGemvMaxWaves = (R >= 4 || MT >= 2) ? 8 : 16;
 // number, so D[m'][n'] is a wanted partial sum where m' and n' name the same part and is
 // ignored elsewhere.  A block then owns 16 / H rows: H times the blocks, each with 1 / H of the
 // lookups, for layers that would leave most compute units without a block.
-template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS, int MT = 1, int H = 1>
+// XS (one row tile per block, from about nine tokens): a step's activations -- 16 * MT rows x 256
+// k -- are loaded 512 contiguous bytes per row, two rows per instruction, parked in an LDS area
+// of the wave's own (rows 528 bytes apart: a 16-lane read of one k-slot then touches every
+// 16-byte bank group once) and read back in operand layout.  Straight from memory every x load
+// instruction touches 64 cache lines at 16 tokens (a lane's 16 bytes lie in a line only the
+// lanes of its token and k-slot share), eight times per step, and with one row tile nothing
+// shares that cost.
+constexpr int kStageRowBytes = 528;
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS, int MT = 1, int H = 1, bool XS = false>
 __global__ void __launch_bounds__((kGemvMaxWaves<R, MT> * 64))
 fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   static_assert(H == 1 || ((H == 2 || H == 4) && R == 1 && MT == 1), "k parts only with one row tile and one token tile");
+  static_assert(!XS || (R == 1 && H == 1 && !X_LDS), "staged activations: one row tile, whole tiles, x not already in LDS");
   constexpr int RT = 16 / H;  // weight rows (and tokens) per MFMA tile
   extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][M][16*R] (+ codebook copy)
   Provider prov(pargs);
@@ -173,13 +183,38 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
     for (int r = 0; r < R; ++r) prov.load(raw[r], min(row0 + 16 * r + cr, s.N - 1), kc);
 
     u32x4 xa[MT][8];
+    if constexpr (XS) {
+      // LDS operations of a wave complete in order, so the reads below see the stores above
+      // them without a barrier; rows past M repeat row M - 1 and are zeroed after the read.
+      uint8_t* const mine = reinterpret_cast<uint8_t*>(red) + s.stage_offset + wave * (MT * 16 * kStageRowBytes);
+      const int piece = lane & 31;  // 16 bytes of the row's 512
+      const int kcp = min(step * 4 + (piece >> 3), s.chunks - 1);
+      u32x4 tmp[8 * MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        xa[t][j] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kc * 64 + j * 8);
-        xa[t][j] = (x_lane[t] && kvalid) ? xa[t][j] : zero4;
+      for (int i = 0; i < 8 * MT; ++i) {
+        const int row = min(2 * i + (lane >> 5), s.M - 1);
+        tmp[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(s.x) + (int64_t)row * s.ldx +
+                                                 (int64_t)kcp * 64 + (piece & 7) * 8);
       }
+#pragma unroll
+      for (int i = 0; i < 8 * MT; ++i)
+        *reinterpret_cast<u32x4*>(mine + (2 * i + (lane >> 5)) * kStageRowBytes + piece * 16) = tmp[i];
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          xa[t][j] = *reinterpret_cast<const u32x4*>(mine + (16 * t + c) * kStageRowBytes + q * 128 + j * 16);
+          xa[t][j] = (x_lane[t] && kvalid) ? xa[t][j] : zero4;
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          xa[t][j] = *reinterpret_cast<const u32x4*>(xrow[t] + (int64_t)kc * 64 + j * 8);
+          xa[t][j] = (x_lane[t] && kvalid) ? xa[t][j] : zero4;
+        }
+    }
 
     // Rows past N are computed on a clamped row and never stored; a k-slot past
     // K must contribute exactly zero, so its operands are zeroed (x is zero
@@ -262,10 +297,14 @@ GemvPlan plan_gemv_rows(int N, int rows, int steps);
 // Codebooks up to this many bytes are staged in LDS by the GEMV (64 KiB = 4096 x 8 fp16).
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
 constexpr int kGemvLdsResidualMax = 16 * 1024;   // residual codebooks of up to 1024 rows
+constexpr int kGemvLdsPerBlockMax = 160 * 1024;
+// Whether a one-row-tile launch of M tokens stages its activations (XS kernels): from nine tokens
+// (NPAMD_GEMV_XSTAGE: 0 never, 2 at every token count).
+bool gemv_stage_activations(int M);
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
 bool gemv_lds_activations_forced();  // NPAMD_GEMV_LDS_X=1: stage x in LDS also without a permutation (tuning aid)
 
-template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false, int MT = 1, int H = 1>
+template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS = false, int MT = 1, int H = 1, bool XS = false>
 int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const GemvPlan& plan,
                         int cb_bytes, hipStream_t st, const char* what) {
   s.steps_per_wave = plan.steps_per_wave;
@@ -273,18 +312,24 @@ int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const
   const int red_bytes = ((plan.waves * s.M * 16 * R + 3) & ~3) * (int)sizeof(float);
   const int x_bytes = X_LDS ? s.M * s.chunks * 64 * 2 : 0;
   const int cb_lds_bytes = CB_LDS ? cb_bytes : 0;
-  const int lds = (CB_LDS && !X_LDS)
+  int lds = (CB_LDS && !X_LDS)
                       ? (red_bytes > cb_lds_bytes ? red_bytes : cb_lds_bytes)
                       : red_bytes + x_bytes +
                             ((X_LDS && s.perm) ? (cb_lds_bytes > x_bytes ? cb_lds_bytes : x_bytes) : cb_lds_bytes);
+  if constexpr (XS) {
+    s.stage_offset = (lds + 15) & ~15;
+    lds = s.stage_offset + plan.waves * MT * 16 * kStageRowBytes;
+    if (lds > kGemvLdsPerBlockMax)  // no room for the staging areas: the same kernel without them
+      return launch_fused_gemv_r<ACT, Provider, R, CB_LDS, X_LDS, MT, H, false>(s, pargs, plan, cb_bytes, st, what);
+  }
   if (lds > 64 * 1024) {
     static LdsLatch latch;  // per instantiation
     const hipError_t e = enable_dynamic_lds(
-        latch, reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H>), lds);
+        latch, reinterpret_cast<const void*>(&fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H, XS>), lds);
     if (e != hipSuccess)
       return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
   }
-  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
+  fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H, XS><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);
 }
 
@@ -339,10 +384,14 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
       if (s.M > 16) {
         const GemvPlan plan = plan_gemv(s.N, s.chunks, 2, 8);
         if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
+        if (gemv_stage_activations(s.M))
+          return launch_fused_gemv_r<ACT, Provider, 1, true, false, 2, 1, true>(s, pargs, plan, cb_bytes, st, what);
         return launch_fused_gemv_r<ACT, Provider, 1, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
       }
       const GemvPlan plan = plan_gemv(s.N, s.chunks, 2);
       if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true>(s, pargs, plan, cb_bytes, st, what);
+      if (gemv_stage_activations(s.M))
+        return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 1, true>(s, pargs, plan, cb_bytes, st, what);
       return launch_fused_gemv_r<ACT, Provider, 1, true>(s, pargs, plan, cb_bytes, st, what);
     }
   }
@@ -364,6 +413,8 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
     if constexpr (!Provider::kGathers)
       if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, false, false, 2>(s, pargs, plan, 0, st, what);
     if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, false, false, 2>(s, pargs, plan, 0, st, what);
+    if (gemv_stage_activations(s.M))
+      return launch_fused_gemv_r<ACT, Provider, 1, false, false, 2, 1, true>(s, pargs, plan, 0, st, what);
     return launch_fused_gemv_r<ACT, Provider, 1, false, false, 2>(s, pargs, plan, 0, st, what);
   }
   const GemvPlan plan = plan_gemv(s.N, s.chunks, (Provider::kGathers && !cb_in_lds) ? 2 : 4);
@@ -387,6 +438,8 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
   }
   if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, false>(s, pargs, plan, 0, st, what);
   if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, false>(s, pargs, plan, 0, st, what);
+  if (gemv_stage_activations(s.M))
+    return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 1, true>(s, pargs, plan, 0, st, what);
   return launch_fused_gemv_r<ACT, Provider, 1, false>(s, pargs, plan, 0, st, what);
 }
 

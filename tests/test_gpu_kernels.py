@@ -540,6 +540,93 @@ def test_gemv_rows_traded_for_k_parts(gpu, oracle_lib, gemv_parts, kind, n, k, p
     _check(y, ref)
 
 
+@pytest.fixture
+def gemv_tuning(monkeypatch):
+    """Sets NPAMD_* tuning variables for one test (the library reads them once: they are re-read on
+    the way in and out)."""
+    from neuropress_amd import _lib
+
+    names = []
+
+    def force(**variables):
+        for name, value in variables.items():
+            monkeypatch.setenv(name, str(value))
+            names.append(name)
+        _lib.load().npamd_diag_reload_tuning()
+
+    yield force
+    for name in names:
+        monkeypatch.delenv(name, raising=False)
+    _lib.load().npamd_diag_reload_tuning()
+
+
+@pytest.mark.parametrize("m", [1, 9, 16, 17, 25, 32])
+@pytest.mark.parametrize("n,k", [(37, 192), (100, 1088), (260, 4160)])
+@pytest.mark.parametrize("kind", ["vq16", "vq16_bf16", "vq12_mem", "vq12_vl4_mem", "rvq", "q4", "q4_asym", "q8"])
+def test_gemv_staged_activations(gpu, oracle_lib, gemv_tuning, kind, n, k, m):
+    """The fused GEMV with a step's activations staged through a per-wave LDS area (taken by itself
+    from nine tokens on layers of one row tile per block; forced here at every token count, whole
+    tiles): token counts on both sides of a token tile, rows past M, K whose chunks do not fill
+    the last step, lookups from memory and (residual VQ) with a table in LDS next to the staging
+    areas."""
+    from neuropress_amd import kernels
+
+    tuning = {"NPAMD_GEMV_XSTAGE": 2, "NPAMD_GEMV_PARTS": 1}
+    if kind.endswith("_mem"):
+        tuning["NPAMD_GEMV_LDS_CB"] = 0
+    gemv_tuning(**tuning)
+    if kind.startswith("vq"):
+        bits = int(kind[2:4])
+        act = torch.bfloat16 if "bf16" in kind else torch.float16
+        vl = 4 if "vl4" in kind else 8
+        L = cases.vq_layer(500 + bits + m, n, k, 1 << bits, vl=vl, bits=bits, act=act, m=m, bias=True)
+        y = kernels.vq_linear(L["x"].to(gpu), L["packed"].to(gpu), L["cb"].to(gpu), bits, vl, L["bias"].to(gpu), n)
+        ref = _vq_ref(oracle_lib, L, act)
+    elif kind == "rvq":
+        L = cases.rvq_layer(510 + m, n, k, act=torch.float16, m=m)
+        y = kernels.rvq_linear(L["x"].to(gpu), L["pm"].to(gpu), L["bm"], L["pr"].to(gpu), L["br"], L["cbm"].to(gpu),
+                               L["cbr"].to(gpu), L["scale"].to(gpu), L["wbias"].to(gpu), n, None, tile=False)
+        ref = _rvq_ref(oracle_lib, L, torch.float16)
+    else:
+        nbits = int(kind[1])
+        L = cases.q4_layer(520 + m, n, k, nbits=nbits, gs=32, act=torch.float16, m=m, asym="asym" in kind, bias=True)
+        zp = None if L["zp"] is None else L["zp"].to(gpu)
+        y = kernels.q_linear(L["x"].to(gpu), L["blob"].to(gpu), L["scale"].to(gpu), nbits, 32, zp, L["bias"].to(gpu))
+        ref = _q_ref(oracle_lib, L, torch.float16)
+    assert y.shape == (m, n)
+    _check(y, ref)
+
+
+@pytest.mark.parametrize("kind", ["vq16", "rvq", "q4"])
+def test_gemv_staged_activations_decode_bit_exactly(gpu, gemv_tuning, kind):
+    """One-hot activations through the staged GEMV: every (token, k) must come back out of the
+    staging area where the MFMA operand layout expects it."""
+    from neuropress_amd import kernels
+
+    n, k, act = 45, 1088, torch.float16
+    if kind == "vq16":
+        L = cases.vq_layer(541, n, k, 65536, bits=16, act=act, m=1, std=0.05)
+        pk, cb = L["packed"].to(gpu), L["cb"].to(gpu)
+        w = kernels.vq_dequant(pk, cb, 16, n, k, act)
+        gemv = lambda x: kernels.vq_linear(x, pk, cb, 16, 8, None, n)
+    elif kind == "rvq":
+        L = cases.rvq_layer(542, n, k, act=act, m=1)
+        d = {key: (v.to(gpu) if torch.is_tensor(v) else v) for key, v in L.items()}
+        args = (d["pm"], L["bm"], d["pr"], L["br"], d["cbm"], d["cbr"], d["scale"], d["wbias"], n)
+        w = kernels.rvq_dequant(*args, k, act)
+        gemv = lambda x: kernels.rvq_linear(x, *args, None, tile=False)
+    else:
+        L = cases.q4_layer(543, n, k, act=act, m=1)
+        blob, sc = L["blob"].to(gpu), L["scale"].to(gpu)
+        w = kernels.q_dequant(blob, sc, 4, 32, None, act)
+        gemv = lambda x: kernels.q_linear(x, blob, sc, 4, 32, None)
+    gemv_tuning(NPAMD_GEMV_XSTAGE=2, NPAMD_GEMV_PARTS=1)
+    eye = torch.eye(k, dtype=act, device=gpu)
+    wt = w.t().contiguous()
+    for k0, count in ((0, 16), (250, 16), (k - 32, 32), (500, 21), (1020, 9)):
+        assert torch.equal(gemv(eye[k0:k0 + count]), wt[k0:k0 + count]), f"{count} tokens one-hot at {k0}"
+
+
 @pytest.mark.parametrize("parts", [2, 4])
 @pytest.mark.parametrize("kind", ["vq12", "vq16", "rvq", "q4"])
 def test_gemv_k_parts_decode_bit_exactly(gpu, gemv_parts, kind, parts):
