@@ -41,6 +41,7 @@ SIGNATURES: dict[str, list] = {
                               ctypes.POINTER(_i64)],  # fmt: skip
     "npamd_vq_sliced_check": [_vp, _i64],
     "npamd_vq_fused_supported": [_int, _int, _int],
+    "npamd_gemv_stages_activations": [_int, _int, _int, _int],
     "npamd_q_fused_supported": [_int, _int, _int],
     "npamd_vq_gemv_coded": [_vp, _i64, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp,
                             _i64, _int, _int, _int, _int, _vp],  # fmt: skip

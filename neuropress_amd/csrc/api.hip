@@ -201,6 +201,12 @@ int plan_tile_mw(int M) {
 
 extern "C" int npamd_version(void) { return 3; }
 
+extern "C" int npamd_gemv_stages_activations(int M, int N, int K, int table_in_lds) {
+  if (M < 1 || M > NPAMD_GEMV_MAX_M || N < 1 || K < 64 || K % 64 || table_in_lds) return 0;
+  if (!npamd::gemv_stage_activations(M) || npamd::plan_gemv_parts(M, N, K / 64, 0) != 1) return 0;
+  return npamd::plan_gemv(N, K / 64, 4, M > 16 ? 8 : 16).R == 1 ? 1 : 0;
+}
+
 extern "C" void npamd_diag_reload_tuning(void) { npamd::tuning_table() = npamd::read_tuning(); }
 
 extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K) {

@@ -251,6 +251,13 @@ def vq_linear_perm_supported(m: int, n: int, k: int, num_centroids: int, vector_
                                                          int(vector_len), int(bits)))  # fmt: skip
 
 
+def gemv_stages_activations(m: int, n: int, k: int, table_in_lds: bool) -> bool:
+    """Whether a fused GEMV call of *m* tokens on an ``n x k`` layer runs the kernel that stages its
+    activations through LDS (``npamd_gemv_stages_activations``): then the GEMV stays ahead of the
+    tile GEMM up to its 32 tokens at any ``k``."""
+    return bool(_lib.load().npamd_gemv_stages_activations(int(m), int(n), int(k), int(bool(table_in_lds))))
+
+
 def vq_fused_supported(in_features: int, vector_len: int, bits: int) -> bool:
     """Whether the MFMA GEMV / tile GEMM take a VQ layer of this shape (``npamd_vq_fused_supported``).
     Other shapes run an element-wise kernel that decodes the weight once per 16 tokens."""

@@ -313,6 +313,14 @@ class NPLinear(nn.Module):
                 cap = 1 << 30  # the fused GEMM pays for the zero points per tile: GEMV at any K
             if m * self.in_features <= cap:
                 return _Q_FUSED_WIDE_MAX_TOKENS
+            # One row tile per workgroup: the GEMV stages its activations through LDS and stays
+            # ahead of the tile GEMM at any K (int4, GEMV vs tile GEMM at 17 / 24 / 32 tokens:
+            # 4096 x 14336 23.6 / 24.4 / 25.6 vs 29.5-29.9 us, 4096 x 8192 15.2 / 15.0 / 15.6 vs 21.8-22.5 us).
+            if self.nbits == 4:
+                from .. import kernels
+
+                if kernels.gemv_stages_activations(m, self.out_features, self.in_features, False):
+                    return _Q_FUSED_WIDE_MAX_TOKENS
         return _Q_FUSED_MAX_TOKENS
 
     def _forward_cuda(self, x: torch.Tensor) -> torch.Tensor:

@@ -757,7 +757,24 @@ class NPVQLinear(nn.Module):
         if limit == 16 and 16 < m <= min(_FUSED_WIDE_MAX_TOKENS, 32):
             if self.is_residual or m * self.in_features <= _FUSED_WIDE_MAX_ACTIVATIONS:
                 return 32
+            if self._gemv_stages_activations(m):
+                return 32
         return limit
+
+    def _gemv_stages_activations(self, m: int) -> bool:
+        """Layers of one row tile per workgroup whose lookups go to memory run the GEMV that stages
+        its activations through LDS, which stays ahead of the tile GEMM at any K (65536-row
+        codebook, GEMV vs tile GEMM at 17 / 24 / 32 tokens: 4096 x 14336 39.8 / 39.7 / 42.0 vs
+        48.7-49.6 us, 4096 x 8192 24.2 / 24.1 / 24.8 vs 33.8-34.8 us; with a 4096-row table, which
+        the GEMV looks up in LDS, it does not: 23.4 / 28.4 / 33.4 vs 24.6-25.8 us)."""
+        hit = self._derived.get("stages")
+        if hit is None or hit[0] != m:
+            from .. import kernels
+
+            table_bytes = self.proxy.num_centroids * self.vector_len * 2
+            hit = (m, kernels.gemv_stages_activations(m, self.out_features, self.in_features, table_bytes <= 65536))
+            self._derived["stages"] = hit
+        return hit[1]
 
     def _perm_fusable(self, x: torch.Tensor, m: int) -> bool:
         """Whether the fused GEMV gathers ``x[..., column_perm]`` itself for this call."""

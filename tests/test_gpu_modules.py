@@ -110,6 +110,39 @@ def test_residual_module_bands(gpu, monkeypatch):
         _close(layer(x.to(gpu)), x.float() @ w.T)
 
 
+def test_long_k_layers_of_one_row_tile_keep_the_gemv_to_32_tokens(gpu, monkeypatch):
+    """tokens x K above 2^18 normally ends the GEMV band at 16 tokens; a layer of one row tile per
+    workgroup whose lookups go to memory runs the GEMV that stages its activations and keeps it
+    to 32 tokens (65536-row codebook, int4), one with a 4096-row table (looked up in LDS) does
+    not.  Outputs against the dense product of the decoded weight."""
+    import neuropress_amd.nn.np_linear as qmod
+    from neuropress_amd import kernels
+
+    calls = []
+    for name in ("vq_linear", "vq_gemm_tile", "q_linear", "q_gemm_tile"):
+        real = getattr(kernels, name)
+        monkeypatch.setattr(kernels, name, lambda *a, _real=real, _name=name, **kw: (calls.append(_name), _real(*a, **kw))[1])
+    monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
+    monkeypatch.setattr(qmod, "_Q_TILE_MIN_GRID_FRACTION", 0.0)
+    n, k, m = 48, 16384, 24
+    x = torch.randn(m, k, generator=cases.gen(3)).half()
+    for nc, expect in ((65536, "vq_linear"), (4096, "vq_gemm_tile")):
+        L = cases.vq_layer(70 + nc, n, k, nc, bias=False, std=0.05)
+        layer = NPVQLinear(VQProxy(L["cb"]).to(gpu), L["packed"], L["bits"], n, k, 8, "cuda_wmma").to(gpu)
+        assert kernels.gemv_stages_activations(m, n, k, nc * 16 <= 65536) == (nc == 65536)
+        calls.clear()
+        y = layer(x.to(gpu))
+        assert calls == [expect], calls
+        _close(y, x.float() @ L["cb"][L["idx"]].reshape(n, k).float().T)
+    Q = cases.q4_layer(71, n, k)
+    qlayer = NPLinear(Q["blob"], Q["scale"], n, k, 32, 4, "sym", "cuda").to(gpu)
+    calls.clear()
+    y = qlayer(x.to(gpu))
+    assert calls == ["q_linear"], calls
+    w = ((Q["codes"].float() - 8).reshape(n, k // 32, 32) * Q["scale"].float().reshape(n, k // 32, 1)).reshape(n, k)
+    _close(y, x.float() @ w.half().float().T)
+
+
 def test_residual_layers_take_the_gemv_to_32_tokens_and_then_the_tile_band(gpu, monkeypatch):
     """A residual layer keeps the fused GEMV up to 32 tokens at any reduction length and takes the
     tile GEMM above, like a plain layer."""
