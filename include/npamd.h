@@ -105,7 +105,7 @@ int npamd_vq_fused_supported(int K, int vl, int bits);
 
 /* 1 when a fused GEMV call (npamd_vq_gemv, npamd_rvq_gemv, npamd_q_gemv) of M tokens on an N x K
  * layer runs the kernel that stages every step's activations through LDS (one 16-row tile per
- * workgroup, nine tokens or more, the operands not looked up in an LDS copy of the codebook:
+ * workgroup, three tokens or more, the operands not looked up in an LDS copy of the codebook:
  * table_in_lds = 0): such a call stays ahead of the tile GEMM up to the GEMV's 32 tokens whatever
  * K is, which is what the callers' band thresholds ask (the reference fixes its own thresholds per
  * backend, neuropress/nn/np_vq_linear.py:73-98).  Host-only arithmetic. */

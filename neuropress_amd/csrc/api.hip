@@ -89,13 +89,14 @@ static int device_cu_count() {
 bool gemv_lds_codebook_enabled() { return tuning().gemv_lds_cb != 0; }
 bool tile_lds_codebook_enabled() { return tuning().tile_lds_cb != 0; }
 bool gemv_lds_activations_forced() { return tuning().gemv_lds_x != 0; }
-// One token tile, one row tile, us, straight from memory / staged: int4 4096 x 4096 7.75 / 7.1 at 8
-// tokens, 9.2 / 7.8 at 16, 13.2 / 10.8 at 32; 4096 x 14336 27.5 / 19.7 at 16, 38.7 / 27.6 at 32;
-// 65536-row codebook 4096 x 14336 42.4 / 38.4 at 16, 52 / 42 at 32; but int4 1024 x 4096 5.8 / 6.2
-// at 8 tokens.  With more row tiles per block (14336 x 4096) or the table in LDS it does not pay.
+// One row tile per block, us, straight from memory / staged: int4 4096 x 4096 6.6 / 6.6 at 2 tokens,
+// 6.9 / 6.5 at 4, 7.9 / 6.6 at 8, 9.2 / 7.5 at 16, 13.2 / 9.0 at 32; 4096 x 14336 17.5 / 15.7 at 4,
+// 20.5 / 16.2 at 8, 27.5 / 18.9 at 16, 38.7 / 25.4 at 32; 65536-row codebook 4096 x 14336 35.8 / 34.6
+// at 4, 37.8 / 35.4 at 8, 42.4 / 37.6 at 16, 52 / 41 at 32.  With more row tiles per block
+// (14336 x 4096) or the table in LDS it does not pay.
 bool gemv_stage_activations(int M) {
   const int mode = tuning().gemv_xstage;
-  return mode >= 2 || (mode == 1 && M >= 9);
+  return mode >= 2 || (mode == 1 && M >= 3);
 }
 
 GemvPlan plan_gemv(int N, int chunks, int max_r, int max_waves_cap) {

@@ -62,7 +62,7 @@ constexpr int kGemvMaxWaves = (R >= 4 || MT >= 2) ? 8 : 16;
 // number, so D[m'][n'] is a wanted partial sum where m' and n' name the same part and is
 // ignored elsewhere.  A block then owns 16 / H rows: H times the blocks, each with 1 / H of the
 // lookups, for layers that would leave most compute units without a block.
-// XS (one row tile per block, from about nine tokens): a step's activations -- 16 * MT rows x 256
+// XS (one row tile per block, from three tokens): a step's activations -- 16 * MT rows x 256
 // k -- are loaded 512 contiguous bytes per row, two rows per instruction, parked in an LDS area
 // of the wave's own (rows 528 bytes apart: a 16-lane read of one k-slot then touches every
 // 16-byte bank group once) and read back in operand layout.  Straight from memory every x load
@@ -298,7 +298,7 @@ GemvPlan plan_gemv_rows(int N, int rows, int steps);
 constexpr int kGemvLdsCodebookMax = 64 * 1024;
 constexpr int kGemvLdsResidualMax = 16 * 1024;   // residual codebooks of up to 1024 rows
 constexpr int kGemvLdsPerBlockMax = 160 * 1024;
-// Whether a one-row-tile launch of M tokens stages its activations (XS kernels): from nine tokens
+// Whether a one-row-tile launch of M tokens stages its activations (XS kernels): from three tokens
 // (NPAMD_GEMV_XSTAGE: 0 never, 2 at every token count).
 bool gemv_stage_activations(int M);
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)

@@ -565,7 +565,7 @@ def gemv_tuning(monkeypatch):
 @pytest.mark.parametrize("kind", ["vq16", "vq16_bf16", "vq12_mem", "vq12_vl4_mem", "rvq", "q4", "q4_asym", "q8"])
 def test_gemv_staged_activations(gpu, oracle_lib, gemv_tuning, kind, n, k, m):
     """The fused GEMV with a step's activations staged through a per-wave LDS area (taken by itself
-    from nine tokens on layers of one row tile per block; forced here at every token count, whole
+    from three tokens on layers of one row tile per block; forced here at every token count, whole
     tiles): token counts on both sides of a token tile, rows past M, K whose chunks do not fill
     the last step, lookups from memory and (residual VQ) with a table in LDS next to the staging
     areas."""
