@@ -69,12 +69,22 @@ constexpr int kGemvMaxWaves = (R >= 4 || MT >= 2) ? 8 : 16;
 // instruction touches 64 cache lines at 16 tokens (a lane's 16 bytes lie in a line only the
 // lanes of its token and k-slot share), eight times per step, and with one row tile nothing
 // shares that cost.
-constexpr int kStageRowBytes = 528;
+// Staging layout of one wave: [token][chunk of the step][128 bytes], H parts: 4 * H chunks per
+// token.  Chunk and row strides are padded so that the 16 lanes of a read pass (one k-slot: 16 / H
+// tokens x H parts) fall into 16 different 16-byte bank groups: in units of 16 bytes the strides
+// are (chunk, row) = (8, 33) for whole tiles, (8, 65) for two parts, (9, 148) for four.
+template <int H>
+struct GemvStage {
+  static constexpr int kChunk = H == 4 ? 144 : 128;
+  static constexpr int kRow = 4 * H * kChunk + (H == 4 ? 64 : 16);
+  static constexpr int kRowData = 512 * H;      // bytes of one token's activations in a step
+  static constexpr int kBytes = (16 / H) * kRow;  // per token tile
+};
 template <int ACT, class Provider, int R, bool CB_LDS, bool X_LDS, int MT = 1, int H = 1, bool XS = false>
 __global__ void __launch_bounds__((kGemvMaxWaves<R, MT> * 64))
 fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
   static_assert(H == 1 || ((H == 2 || H == 4) && R == 1 && MT == 1), "k parts only with one row tile and one token tile");
-  static_assert(!XS || (R == 1 && H == 1 && !X_LDS), "staged activations: one row tile, whole tiles, x not already in LDS");
+  static_assert(!XS || (R == 1 && !X_LDS), "staged activations: one row tile, x not already in LDS");
   constexpr int RT = 16 / H;  // weight rows (and tokens) per MFMA tile
   extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][M][16*R] (+ codebook copy)
   Provider prov(pargs);
@@ -186,24 +196,34 @@ fused_gemv_kernel(const GemvShape s, const typename Provider::Args pargs) {
     if constexpr (XS) {
       // LDS operations of a wave complete in order, so the reads below see the stores above
       // them without a barrier; rows past M repeat row M - 1 and are zeroed after the read.
-      uint8_t* const mine = reinterpret_cast<uint8_t*>(red) + s.stage_offset + wave * (MT * 16 * kStageRowBytes);
-      const int piece = lane & 31;  // 16 bytes of the row's 512
-      const int kcp = min(step * 4 + (piece >> 3), s.chunks - 1);
+      using SL = GemvStage<H>;
+      uint8_t* const mine = reinterpret_cast<uint8_t*>(red) + s.stage_offset + wave * (MT * SL::kBytes);
       u32x4 tmp[8 * MT];
 #pragma unroll
-      for (int i = 0; i < 8 * MT; ++i) {
-        const int row = min(2 * i + (lane >> 5), s.M - 1);
-        tmp[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(s.x) + (int64_t)row * s.ldx +
-                                                 (int64_t)kcp * 64 + (piece & 7) * 8);
-      }
+      for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int i = 0; i < 8 * MT; ++i)
-        *reinterpret_cast<u32x4*>(mine + (2 * i + (lane >> 5)) * kStageRowBytes + piece * 16) = tmp[i];
+        for (int i = 0; i < 8; ++i) {  // 1 KiB per instruction of the tile's RT x kRowData bytes
+          const int flat = i * 1024 + lane * 16;
+          const int row = min(RT * t + flat / SL::kRowData, s.M - 1);
+          const int off = flat % SL::kRowData;
+          const int kcp = min(step * 4 * H + off / 128, s.chunks - 1);
+          tmp[t * 8 + i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(s.x) + (int64_t)row * s.ldx +
+                                                           (int64_t)kcp * 64 + (off % 128) / 2);
+        }
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int flat = i * 1024 + lane * 16;
+          const int off = flat % SL::kRowData;
+          *reinterpret_cast<u32x4*>(mine + (RT * t + flat / SL::kRowData) * SL::kRow + (off / 128) * SL::kChunk + off % 128) =
+              tmp[t * 8 + i];
+        }
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          xa[t][j] = *reinterpret_cast<const u32x4*>(mine + (16 * t + c) * kStageRowBytes + q * 128 + j * 16);
+          xa[t][j] = *reinterpret_cast<const u32x4*>(mine + (RT * t + cr) * SL::kRow + (q * H + part) * SL::kChunk + j * 16);
           xa[t][j] = (x_lane[t] && kvalid) ? xa[t][j] : zero4;
         }
     } else {
@@ -318,7 +338,7 @@ int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const
                             ((X_LDS && s.perm) ? (cb_lds_bytes > x_bytes ? cb_lds_bytes : x_bytes) : cb_lds_bytes);
   if constexpr (XS) {
     s.stage_offset = (lds + 15) & ~15;
-    lds = s.stage_offset + plan.waves * MT * 16 * kStageRowBytes;
+    lds = s.stage_offset + plan.waves * MT * GemvStage<H>::kBytes;
     if (lds > kGemvLdsPerBlockMax)  // no room for the staging areas: the same kernel without them
       return launch_fused_gemv_r<ACT, Provider, R, CB_LDS, X_LDS, MT, H, false>(s, pargs, plan, cb_bytes, st, what);
   }
@@ -367,12 +387,20 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
   if (h > 1 && !s.perm && !gemv_lds_activations_forced()) {
     s.steps = (s.chunks + 4 * h - 1) / (4 * h);
     const GemvPlan plan = plan_gemv_rows(s.N, 16 / h, s.steps);
+    // Staged activations as for whole tiles, except next to a whole codebook in LDS.
+    const bool staged = gemv_stage_activations(s.M) && !(lds_table && Provider::kLdsCodebook);
     if constexpr (Provider::kLdsResidual || Provider::kLdsCodebook) {
       if (lds_table) {
+        if constexpr (Provider::kLdsResidual) {
+          if (staged && h == 4) return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 4, true>(s, pargs, plan, cb_bytes, st, what);
+          if (staged) return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 2, true>(s, pargs, plan, cb_bytes, st, what);
+        }
         if (h == 4) return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 4>(s, pargs, plan, cb_bytes, st, what);
         return launch_fused_gemv_r<ACT, Provider, 1, true, false, 1, 2>(s, pargs, plan, cb_bytes, st, what);
       }
     }
+    if (staged && h == 4) return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 4, true>(s, pargs, plan, 0, st, what);
+    if (staged) return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 2, true>(s, pargs, plan, 0, st, what);
     if (h == 4) return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 4>(s, pargs, plan, 0, st, what);
     return launch_fused_gemv_r<ACT, Provider, 1, false, false, 1, 2>(s, pargs, plan, 0, st, what);
   }
