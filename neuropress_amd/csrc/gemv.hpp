@@ -62,10 +62,9 @@ constexpr int kGemvMaxWaves = (R >= 4 || MT >= 2) ? 8 : 16;
 // number, so D[m'][n'] is a wanted partial sum where m' and n' name the same part and is
 // ignored elsewhere.  A block then owns 16 / H rows: H times the blocks, each with 1 / H of the
 // lookups, for layers that would leave most compute units without a block.
-// XS (one row tile per block, from three tokens): a step's activations -- 16 * MT rows x 256
-// k -- are loaded 512 contiguous bytes per row, two rows per instruction, parked in an LDS area
-// of the wave's own (rows 528 bytes apart: a 16-lane read of one k-slot then touches every
-// 16-byte bank group once) and read back in operand layout.  Straight from memory every x load
+// XS (one row tile per block, from three tokens): a step's activations -- the tile's tokens x
+// 256 * H k -- are loaded 1 KiB of contiguous row bytes per instruction, parked in an LDS area of
+// the wave's own (GemvStage) and read back in operand layout.  Straight from memory every x load
 // instruction touches 64 cache lines at 16 tokens (a lane's 16 bytes lie in a line only the
 // lanes of its token and k-slot share), eight times per step, and with one row tile nothing
 // shares that cost.
