@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "../../include/npamd.h"
 
@@ -51,12 +52,14 @@ inline hipError_t enable_dynamic_lds(LdsLatch& latch, const void* kernel, int by
   if (hipGetDevice(&dev) != hipSuccess) dev = -1;
   std::atomic<int>* slot = (dev >= 0 && dev < kLdsLatchDevices) ? &latch.reserved[dev] : nullptr;
   if (slot && bytes <= slot->load(std::memory_order_acquire)) return hipSuccess;
+  // Raising the limit is serialised: two first callers with different sizes must not leave the
+  // kernel with the smaller one while the latch records the larger.
+  static std::mutex raise;
+  std::lock_guard<std::mutex> lock(raise);
+  if (slot && bytes <= slot->load(std::memory_order_acquire)) return hipSuccess;
   const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e != hipSuccess || !slot) return e;
-  int seen = slot->load(std::memory_order_relaxed);
-  while (seen < bytes && !slot->compare_exchange_weak(seen, bytes, std::memory_order_release)) {
-  }
-  return hipSuccess;
+  if (e == hipSuccess && slot) slot->store(bytes, std::memory_order_release);
+  return e;
 }
 
 #define NPAMD_REQUIRE(cond, ...)                                  \
