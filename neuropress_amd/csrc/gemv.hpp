@@ -409,7 +409,7 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
     // looks up in memory.
     if (cb_bytes > 0 && cb_bytes <= kGemvLdsResidualMax && gemv_lds_codebook_enabled()) {
       if (s.M > 16) {
-        const GemvPlan plan = plan_gemv(s.N, s.chunks, 2, 8);
+        const GemvPlan plan = plan_gemv(s.N, s.chunks, gemv_stage_activations(s.M) ? 1 : 2, 8);  // as for plain VQ below
         if (plan.R == 2) return launch_fused_gemv_r<ACT, Provider, 2, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
         if (gemv_stage_activations(s.M))
           return launch_fused_gemv_r<ACT, Provider, 1, true, false, 2, 1, true>(s, pargs, plan, cb_bytes, st, what);
@@ -429,7 +429,13 @@ int launch_fused_gemv(GemvShape s, const typename Provider::Args& pargs, hipStre
     // 17..32 tokens: two token tiles per weight operand, eight waves.  Every block reads all of
     // x, twice as much as at 16 tokens, so four row tiles per block (half the blocks) pay more
     // than anywhere else: 14336 x 4096, 4096-row codebook, 17 tokens: 20.0 us at R = 2, 12.9 at 4.
-    const GemvPlan plan = plan_gemv(s.N, s.chunks, (Provider::kGathers && !cb_in_lds) ? 2 : 4, 8);
+    // Lookups in memory: one staged row tile per block instead of two plain ones (65536-row
+    // codebook, 24 / 32 tokens, us: 6144 x 4096 22.45 / 24.3 -> 22.2 / 22.8, 11008 x 4096 41.5 /
+    // 44.8 -> 34.9 / 35.75, 14336 x 4096 46.7 / 49.7 -> 44.8 / 45.8, 28672 x 4096 83.3 / 89.75 ->
+    // 74.8 / 77.7, 8192 x 8192 47.0 / 50.3 -> 45.3 / 46.8); at 16 tokens and below it depends on
+    // the layer (6144 x 4096 20.5 -> 21.45 at 16), so there the plan stands.
+    const bool memory_lookups = Provider::kGathers && !cb_in_lds;
+    const GemvPlan plan = plan_gemv(s.N, s.chunks, memory_lookups ? (gemv_stage_activations(s.M) ? 1 : 2) : 4, 8);
     if constexpr (Provider::kLdsCodebook) {
       if (cb_in_lds) {
         if (plan.R == 4) return launch_fused_gemv_r<ACT, Provider, 4, true, false, 2>(s, pargs, plan, cb_bytes, st, what);
