@@ -49,7 +49,8 @@ def _compile(src: Path, force: bool) -> Path:
     newest = max(src.stat().st_mtime, _headers_mtime())
     if not force and obj.exists() and obj.stat().st_mtime >= newest:
         return obj
-    cmd = [_hipcc(), *CXXFLAGS, *DEVICE_FLAGS, "-c", os.fspath(src), "-o", os.fspath(obj)]
+    extra = os.environ.get("NPAMD_HIPCC_FLAGS", "").split()  # e.g. -DNPAMD_TILE2_ABLATIONS for a tuning build
+    cmd = [_hipcc(), *CXXFLAGS, *DEVICE_FLAGS, *extra, "-c", os.fspath(src), "-o", os.fspath(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stderr}")

@@ -4,7 +4,7 @@
 
 #include <stdlib.h>
 
-#include "gemm_tile.hpp"
+#include "gemm_tile2.hpp"
 #include "gemv.hpp"
 
 namespace npamd {
@@ -53,6 +53,7 @@ static Tuning read_tuning() {
   t.gemv_xstage = env_int("NPAMD_GEMV_XSTAGE", 1);
   t.tile_splits = env_int("NPAMD_TILE_SPLITS", 0);
   t.tile_mw = env_int("NPAMD_TILE_MW", 0);
+  t.tile_wide = env_int("NPAMD_TILE_WIDE", 1);
   t.q4_rows = env_int("NPAMD_Q4_ROWS", 0);
   t.q4_rowwise = env_int("NPAMD_Q4_ROWWISE", 1);
   t.q4_rowwise_bf16 = env_int("NPAMD_Q4_ROWWISE_BF16", 0);
@@ -189,6 +190,21 @@ int plan_tile_splits(int M, int N, int chunks, int mw) {
   return splits < 1 ? 1 : splits;
 }
 
+int tile2_mode() { return tuning().tile_wide; }
+
+int plan_tile2_splits(int M, int N, int chunks, int mw) {
+  const int env = tuning().tile_splits;
+  const int cus = device_cu_count();
+  const int blocks = ((N + kT2Cols - 1) / kT2Cols) * ((M + 128 * mw - 1) / (128 * mw));
+  int splits = 1;
+  if (env > 0) splits = env;
+  else if (blocks * 10 < cus * 7) splits = cus / blocks;
+  const int max_by_k = chunks / 8 > 1 ? chunks / 8 : 1;
+  if (splits > max_by_k) splits = max_by_k;
+  if (splits > 16) splits = 16;
+  return splits < 1 ? 1 : splits;
+}
+
 extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K);
 
 int plan_tile_mw(int M) {
@@ -212,8 +228,11 @@ extern "C" void npamd_diag_reload_tuning(void) { npamd::tuning_table() = npamd::
 
 extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K < 64) return 0;
-  const int splits = npamd::plan_tile_splits(M, N, K / 64, npamd::plan_tile_mw(M));
-  return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
+  const int mw = npamd::plan_tile_mw(M);
+  const int splits = npamd::plan_tile_splits(M, N, K / 64, mw);
+  const int64_t narrow = splits > 1 ? (int64_t)splits * M * N * 4 : 0;
+  const int64_t wide = npamd::tile2_mode() ? npamd::tile2_workspace_bytes(M, N, K / 64, mw) : 0;
+  return narrow > wide ? narrow : wide;
 }
 
 extern "C" const char* npamd_last_error(void) { return npamd::error_text(); }

@@ -34,7 +34,7 @@ int check_launch(const char* what);
 
 // Values of the NPAMD_* tuning environment variables, read once per process.
 struct Tuning {
-  int gemv_lds_cb, tile_lds_cb, gemv_lds_x, gemv_r, gemv_spw, gemv_parts, gemv_xstage, tile_splits, tile_mw;
+  int gemv_lds_cb, tile_lds_cb, gemv_lds_x, gemv_r, gemv_spw, gemv_parts, gemv_xstage, tile_splits, tile_mw, tile_wide;
   int q4_rows, q4_rowwise, q4_rowwise_bf16, q4_stream;
 };
 const Tuning& tuning();

@@ -110,6 +110,71 @@ constexpr int kTileLdsCodebookMax = 64 * 1024;
 constexpr int kTileLdsResidualMax = 16 * 1024;
 constexpr int kLdsPerBlockMax = 160 * 1024;
 
+// Output of one wave's MFMA 32x32 tiles: 32 MW rows x 32 NT columns of f32 sums (+ bias) -> 16-bit y.
+// A lane holds one column of a tile, so storing from the registers is one 2-byte store per value
+// (the vector memory path takes such an instruction lane by lane: 4 waves x 96..192 of them were
+// 8 us of a 90 us launch).  Instead neighbouring lanes swap every second value, so that each
+// holds two adjacent columns of one row, the pairs are parked in an LDS area of the wave's own
+// (row-major, 16-byte pieces swizzled by row against bank conflicts), and the wave stores whole
+// 16-byte pieces, 4 (NT = 4) or 8 (NT = 2) complete rows per instruction.
+// `ep`: 32 MW x 64 NT bytes of LDS nobody else touches; y needs 16-byte aligned rows (else, and
+// for the columns of a ragged last piece, element stores).
+template <int NT>
+__device__ __forceinline__ int ep_swizzle(int row, int piece) {
+  const int g = NT == 4 ? ((row & 1) | (((row >> 2) & 1) << 1)) : ((row >> 2) & 1);
+  return piece ^ (g << 2);
+}
+template <int ACT, int MW, int NT>
+__device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[MW][NT], uint8_t* ep, int lane, void* y, int64_t ldy,
+                                                int row0, int col0, int M, int N, const float* bias) {
+  static_assert(NT == 2 || NT == 4, "two or four column tiles per wave");
+  constexpr int kRowBytes = 64 * NT;
+  const int c = lane & 31, h = lane >> 5;
+  const bool odd = c & 1;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int n = col0 + t * 32 + c;
+    const float bv = (bias && n < N) ? bias[n] : 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MW; ++mt) {
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float v0 = acc[mt][t][i] + bv, v1 = acc[mt][t][i + 1] + bv;
+        // even lane keeps row i and gets the neighbour's (column c + 1); odd lane keeps row i + 1
+        const float got = __shfl_xor(odd ? v0 : v1, 1, 64);
+        const float lo = odd ? got : v0, hi = odd ? v1 : got;
+        uint32_t packed;
+        if constexpr (ACT == NPAMD_BF16) packed = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+        else packed = f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+        const int row = mt * 32 + 8 * (i / 4) + 4 * h + (i % 4) + (odd ? 1 : 0);
+        const int dw = t * 16 + (c >> 1);  // dword of the row: columns 2 dw, 2 dw + 1
+        *reinterpret_cast<uint32_t*>(ep + row * kRowBytes + ep_swizzle<NT>(row, dw >> 2) * 16 + (dw & 3) * 4) = packed;
+      }
+    }
+  }
+  // The wave reads back what its own lanes wrote: LDS operations of a wave complete in order.
+  constexpr int kPiecesPerRow = 4 * NT;            // 16-byte pieces
+  constexpr int kRowsPerInst = 64 / kPiecesPerRow;  // 4 or 8
+  const bool vec_ok = (ldy % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+  const int piece = lane % kPiecesPerRow;
+  uint16_t* const yo = reinterpret_cast<uint16_t*>(y);
+#pragma unroll
+  for (int it = 0; it < 32 * MW / kRowsPerInst; ++it) {
+    const int row = it * kRowsPerInst + lane / kPiecesPerRow;
+    const int m = row0 + row, n = col0 + piece * 8;
+    if (m >= M || n >= N) continue;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * kRowBytes + ep_swizzle<NT>(row, piece) * 16);
+    if (vec_ok && n + 8 <= N) {
+      *reinterpret_cast<u32x4*>(yo + (int64_t)m * ldy + n) = v;
+    } else {
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (n + e < N) yo[(int64_t)m * ldy + n + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    }
+  }
+}
+
 template <int ACT, class Provider, int MW, bool CB_LDS = false>
 __global__ void __launch_bounds__(512)
 tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
@@ -392,11 +457,15 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: D[m = 8*(i/4) + 4h + i%4][n = c] --------------------------
+  if (s.splits <= 1) {
+    // The rows this wave staged its x tile in (first buffer) are its own: 32 MW x 128 bytes.
+    store_wave_tile<ACT, MW, 2>(acc, xs + wrow0 * XS::kXRowBytes, lane, s.y, s.ldy, m0 + wrow0, n0, s.M, s.N, s.bias);
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int n = n0 + t * 32 + c;
     if (n >= s.N) continue;
-    const float bv = s.bias ? s.bias[n] : 0.f;
     float* part = s.partials + (size_t)blockIdx.z * s.M * s.N;
 #pragma unroll
     for (int mt = 0; mt < MW; ++mt) {
@@ -404,8 +473,7 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
       for (int i = 0; i < 16; ++i) {
         const int m = m0 + wrow0 + mt * 32 + 8 * (i / 4) + 4 * h + (i % 4);
         if (m >= s.M) continue;
-        if (s.splits > 1) part[(size_t)m * s.N + n] = acc[mt][t][i];
-        else store_from_f32<ACT>(s.y, (int64_t)m * s.ldy + n, acc[mt][t][i] + bv);
+        part[(size_t)m * s.N + n] = acc[mt][t][i];
       }
     }
   }

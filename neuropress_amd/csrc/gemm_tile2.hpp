@@ -1,0 +1,82 @@
+// Tile-decode GEMM, 128-column blocks: y = x @ W^T (+ bias) for VQ weights with 16-bit indices into a
+// codebook too large for LDS (more than 4096 rows), wave64 + MFMA 32x32x16, f32 accumulate.
+//
+// Why a second block shape.  A block's x tile (BM rows x 64 k) passes the compute unit's vector
+// memory path once per 64-k step whatever the block's width, and that path moves 64 bytes per
+// cycle: with 64 columns it is busy with x as long as the matrix pipe is busy with the MFMAs, on
+// top of the codebook lookups that go the same way.  128 columns halve the x bytes per MFMA.
+//
+// Block = 4 waves, one per SIMD, each with the whole register file of its SIMD (512 registers:
+// 192 accumulators for a 96 x 128 tile and two operand sets).  There are no producer waves:
+// every weight operand is one codebook row, so the decode is a gather, and the gather is issued
+// as a load that writes LDS directly (global_load_lds_dwordx4, one row per lane, 64 rows = one KiB
+// per instruction) -- no register, no LDS store instruction, no arithmetic.  The codebook the
+// caller passes is already in the activation dtype.
+//
+// Roles of wave w in every 64-k step t:
+//   MFMA:    rows [32 MW w, 32 MW (w + 1)) of the block tile x all 128 columns.
+//   x tile:  its own rows of step t + 2, loaded straight into LDS (swizzled 128-byte rows) into
+//            the buffer of step t as soon as the last operands of step t are in registers; no
+//            other wave reads those rows, so the x tile needs no barrier.
+//   W tile:  columns [32 w, 32 w + 32) of step t + 2: lane (c = l % 32, h = l / 32) reads the four
+//            indices 4h .. 4h+3 of its column's chunk from an LDS staging area of the wave (the
+//            16 bytes of a chunk were loaded there, also directly, in step t - 2) and issues four
+//            gathers; gather j lands in position l of KiB (w, j) of W slot (t + 2) % 3, which is
+//            exactly where lane l looks for B operand j of column tile w: MFMA j of a step
+//            contracts k = 64 t + 32 h + 8 j .. + 7, x and W alike.
+// All loads of a wave complete in order, and everything it requests in step t is due at the end
+// of step t + 1 (the W slot and the x buffer of step t + 2, the indices for the gathers of step
+// t + 3): one `s_waitcnt vmcnt(loads of one step)` in front of the step's only barrier.
+//
+// K is split in two (blockIdx.z) when the column blocks alone leave compute units idle:
+// 14336 columns are 112 blocks of 128, so 224 workgroups each contract half of K.  The halves
+// meet without a second kernel and without spinning: whichever workgroup of a pair finishes
+// first stores its f32 tile to the workspace and counts itself in; the other adds that tile to
+// its registers, adds the bias and stores y.  Two addends commute, so the result does not
+// depend on which half was first.  More than two splits (layers of few columns) store partial
+// tiles for splitk_reduce_kernel as the 64-column kernel does.
+#pragma once
+
+#include "gemm_tile.hpp"
+
+namespace npamd {
+
+constexpr int kT2Cols = 128;
+constexpr int kT2WSlotBytes = kT2Cols * kStepK * 2;  // 16 KiB: [column tile 4][operand j 4][lane 64][16 B]
+constexpr int kT2WRing = 3;
+constexpr int kT2IdxBytes = 4 * 2 * 1024;  // per wave two staged chunks of 64 lanes x 16 bytes
+
+struct T2Args {
+  const uint8_t* packed;  // 16-bit indices, [N][K / 8]
+  const void* cb;         // [nc][8] in the activation dtype
+  uint32_t nc_minus_1;
+  int chunks;             // K / 64
+  uint32_t* counters;     // splits == 2: one arrival counter per block tile, zero on entry
+  float* pair_tiles;      // splits == 2: [2][tiles][BM * 128] f32 in register order
+};
+
+template <int MW>
+struct T2Lds {
+  static constexpr int kXBufBytes = 128 * MW * kStepK * 2;
+  static constexpr int kBytes = 2 * kXBufBytes + kT2WRing * kT2WSlotBytes + kT2IdxBytes;
+};
+
+// Splits of K for the 128-column kernel: 1 while the block tiles cover most compute units, else as
+// many as fill them, each at least 8 steps long.
+int plan_tile2_splits(int M, int N, int chunks, int mw);
+// 0: never take the 128-column kernel, 1: where it is the faster one (default), 2: wherever it applies.
+int tile2_mode();
+
+inline int64_t tile2_workspace_bytes(int M, int N, int chunks, int mw) {
+  const int splits = plan_tile2_splits(M, N, chunks, mw);
+  if (splits <= 1) return 0;
+  if (splits > 2) return (int64_t)splits * M * N * 4;
+  const int64_t tiles = (int64_t)((N + kT2Cols - 1) / kT2Cols) * ((M + 128 * mw - 1) / (128 * mw));
+  return ((tiles * 4 + 255) & ~(int64_t)255) + 2 * tiles * (128 * mw) * kT2Cols * 4;
+}
+
+// Takes the call when the workspace allows the planned split; returns 1 when it did not take it.
+// act: NPAMD_F16 or NPAMD_BF16 (activations, codebook and output).
+int launch_tile2(int act, GemmShape s, T2Args a, hipStream_t st, const char* what, void* workspace, int64_t workspace_bytes);
+
+}  // namespace npamd

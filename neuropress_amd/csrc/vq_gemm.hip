@@ -1,5 +1,5 @@
 // C-ABI entry points of the tile-decode MFMA GEMM (plain and residual VQ).
-#include "gemm_tile.hpp"
+#include "gemm_tile2.hpp"
 #include "vq_call.hpp"
 
 using namespace npamd;
@@ -13,6 +13,20 @@ int run_vq(const VqCall& c, const GemmShape& s) {
       using P = VqProvider<ACT, BITS, true, VL>;
       typename P::Args a{c.packed, (const u32x4*)c.cb, (uint32_t)c.nc - 1u, s.chunks};
       return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes, (VL == 8 ? c.nc * 16 : (c.nc % 2 == 0 ? c.nc * 8 : 0)));
+    }
+  }
+  if constexpr (BITS == 16 && VL == 8) {
+    // Codebooks LDS does not hold, in the activation dtype: the 128-column kernel, whose gathers write LDS directly.
+    const int mode = tile2_mode();
+    const bool big = (int64_t)c.nc * 16 > kTileLdsCodebookMax;
+    // Measured against the 64-column kernel on 65536-row codebooks at 17 .. 384 tokens: ahead on 14336 x 4096
+    // (74.6 against 83.1 us at 384 tokens), 28672 x 4096 (117 against 159) and 4096 x 14336 (78 against 88), behind
+    // by 3 to 19 % on 4096 x 4096 and 1024 x 4096, where more than two splits of K meet in a second kernel.
+    const bool wins = big && (c.N >= 8192 || c.K >= 8192);
+    if (c.cb_dtype == c.act && c.n_bytes < ((int64_t)1 << 32) && (mode >= 2 || (mode == 1 && wins))) {
+      T2Args t2{c.packed, c.cb, (uint32_t)c.nc - 1u, s.chunks, nullptr, nullptr};
+      const int rc = launch_tile2(ACT, s, t2, c.st, c.what, c.ws, c.ws_bytes);
+      if (rc != 1) return rc;
     }
   }
   using P = VqProvider<ACT, BITS, false, VL>;

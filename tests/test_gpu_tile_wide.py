@@ -1,0 +1,106 @@
+"""The 128-column tile-decode GEMM (csrc/gemm_tile2.hip) through the C ABI, against the oracle.
+
+The library takes this kernel by itself only for large layers with codebooks LDS does not hold; the
+tests force it (NPAMD_TILE_WIDE=2) on small ragged shapes the oracle finishes in milliseconds, and
+compare with the oracle's decode + double-accumulated product, with the one-pass decode through
+one-hot activations (bit for bit), and with itself from run to run.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def tile_wide(monkeypatch):
+    """force(mode, splits): NPAMD_TILE_WIDE / NPAMD_TILE_SPLITS for one test (the library reads its
+    tuning variables once, so they are re-read on the way in and out)."""
+    from neuropress_amd import _lib
+
+    def force(mode: int, splits: int = 0):
+        monkeypatch.setenv("NPAMD_TILE_WIDE", str(mode))
+        monkeypatch.setenv("NPAMD_TILE_SPLITS", str(splits))
+        _lib.load().npamd_diag_reload_tuning()
+
+    yield force
+    monkeypatch.delenv("NPAMD_TILE_WIDE", raising=False)
+    monkeypatch.delenv("NPAMD_TILE_SPLITS", raising=False)
+    _lib.load().npamd_diag_reload_tuning()
+
+
+def _ref(oracle_lib, L, act):
+    code = orc.torch_dtype_code(act)
+    w = oracle_lib.vq_decode(L["packed"].numpy(), L["bits"], orc.to_bits(L["cb"]), L["n"], L["k"], code)
+    bias = None if L["bias"] is None else orc.to_bits(L["bias"])
+    return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
+
+
+def _check(y, ref):
+    ok, max_abs, excess = cases.within_tol(y.float().cpu().numpy(), ref)
+    assert ok, f"max abs err {max_abs:.3e}, {excess:.2f}x the 1e-2 bound"
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 17, 96, 130, 257, 300, 384, 400])
+@pytest.mark.parametrize("n,k,splits", [(300, 448, 1), (300, 448, 2), (130, 1024, 2), (264, 1088, 3), (1004, 512, 0)])
+def test_wide_tile_gemm_against_the_oracle(gpu, oracle_lib, tile_wide, act, m, n, k, splits):
+    """Ragged N (two to eight 128-column blocks, N % 8 != 0 once: element stores), K of 7 to 17 steps, every row
+    tile count (one to three per wave, two row blocks at 400 tokens), K whole, in two halves that meet
+    in the kernel, and in three parts that meet in the reduction kernel."""
+    from neuropress_amd import kernels
+
+    tile_wide(2, splits)
+    L = cases.vq_layer(700 + m + n, n, k, 65536, bits=16, act=act, m=m, bias=True, std=0.05)
+    cb = L["cb"].to(act).to(gpu)  # the kernel takes the codebook in the activation dtype
+    y = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), cb, 16, n, L["bias"].to(gpu))
+    _check(y, _ref(oracle_lib, L, act))
+    y2 = kernels.vq_gemm_tile(L["x"].to(gpu), L["packed"].to(gpu), cb, 16, n, L["bias"].to(gpu))
+    assert torch.equal(y, y2), "the result depends on which half of K finished first"
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("splits", [1, 2, 4])
+def test_wide_tile_gemm_decodes_bit_exactly(gpu, tile_wide, act, splits):
+    """One-hot activations: y[m, n] is the single product 1 * W[n, k_m], so the kernel must return the
+    one-pass decode (itself bit-exact against the oracle) exactly, whichever way K is split."""
+    from neuropress_amd import kernels
+
+    n, k = 200, 1024
+    L = cases.vq_layer(77, n, k, 65536, bits=16, act=act, m=1, std=0.05)
+    pk, cb = L["packed"].to(gpu), L["cb"].to(gpu)
+    wt = kernels.vq_dequant(pk, cb, 16, n, k, act).t().contiguous()
+    tile_wide(2, splits)
+    eye = torch.eye(k, dtype=act, device=gpu)
+    cba = cb.to(act)
+    assert torch.equal(kernels.vq_gemm_tile(eye, pk, cba, 16, n, None), wt), "1024 tokens"
+    assert torch.equal(kernels.vq_gemm_tile(eye[100:330], pk, cba, 16, n, None), wt[100:330]), "230 tokens"
+    assert torch.equal(kernels.vq_gemm_tile(eye[5:26], pk, cba, 16, n, None), wt[5:26]), "21 tokens"
+
+
+def test_wide_and_narrow_tile_gemm_agree_on_a_large_layer(gpu, tile_wide):
+    """A layer of the size the library takes the 128-column kernel for by itself (8192 columns), K in two
+    halves: against the 64-column kernel and the dense product of the decoded weight."""
+    from neuropress_amd import _lib, kernels
+
+    n, k, m = 8192, 1024, 384
+    g = cases.gen(5)
+    cb = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.float16)
+    pk = torch.randint(0, 65536, (n * k // 8,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8).to(gpu)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(gpu)
+    cba = cb.to(torch.bfloat16).to(gpu)
+    assert _lib.load().npamd_gemm_tile_workspace_bytes(m, n, k) > 0
+    tile_wide(1)
+    y_auto = kernels.vq_gemm_tile(x, pk, cba, 16, n, None)
+    tile_wide(0)
+    y_narrow = kernels.vq_gemm_tile(x, pk, cba, 16, n, None)
+    ref = x.float() @ kernels.vq_dequant(pk, cb.to(gpu), 16, n, k, torch.bfloat16).float().t()
+    for y in (y_auto, y_narrow):
+        err = (y.float() - ref).abs()
+        assert bool((err <= 1e-2 + 1e-2 * ref.abs()).all()), float(err.max())
+    # same products, f32 sums in a different order: they differ by output roundings at most
+    assert float((y_auto.float() - y_narrow.float()).abs().max()) <= 2.0 ** -6
