@@ -231,7 +231,12 @@ extern "C" int64_t npamd_gemm_tile_workspace_bytes(int M, int N, int K) {
   const int mw = npamd::plan_tile_mw(M);
   const int splits = npamd::plan_tile_splits(M, N, K / 64, mw);
   const int64_t narrow = splits > 1 ? (int64_t)splits * M * N * 4 : 0;
-  const int64_t wide = npamd::tile2_mode() ? npamd::tile2_workspace_bytes(M, N, K / 64, mw) : 0;
+  int64_t wide = 0;
+  if (npamd::tile2_mode()) {
+    wide = npamd::tile2_workspace_bytes(M, N, K / 64, mw);
+    const int64_t wide_q = npamd::tile2_workspace_bytes(M, N, K / 64, npamd::plan_tile2_q_mw(M));
+    if (wide_q > wide) wide = wide_q;
+  }
   return narrow > wide ? narrow : wide;
 }
 

@@ -141,7 +141,9 @@ __device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[MW][NT], uin
       for (int i = 0; i < 16; i += 2) {
         const float v0 = acc[mt][t][i] + bv, v1 = acc[mt][t][i + 1] + bv;
         // even lane keeps row i and gets the neighbour's (column c + 1); odd lane keeps row i + 1
-        const float got = __shfl_xor(odd ? v0 : v1, 1, 64);
+        // neighbour in the lane pair, as a DPP move (quad_perm [1, 0, 3, 2]): one VALU instruction
+        const float got = __builtin_bit_cast(
+            float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, odd ? v0 : v1), 0xB1, 0xF, 0xF, true));
         const float lo = odd ? got : v0, hi = odd ? v1 : got;
         uint32_t packed;
         if constexpr (ACT == NPAMD_BF16) packed = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);

@@ -1,6 +1,9 @@
-// The 128-column tile-decode GEMM (see gemm_tile2.hpp): kernel and launcher.
+// The 128-column tile-decode GEMM (see gemm_tile2.hpp): kernel, weight-tile producers and launchers.
 #include "gemm_tile2.hpp"
+
 #include <stdlib.h>
+
+#include <type_traits>
 
 namespace npamd {
 
@@ -9,12 +12,10 @@ __global__ void __launch_bounds__(256) tile2_zero_counters_kernel(uint32_t* coun
   if (i < n) counters[i] = 0u;
 }
 
-// ABL (builds with -DNPAMD_TILE2_ABLATIONS only; 0 in the library): parts of the step compiled out, to time the
-// others -- 1 no gathers, 2 no x loads, 4 no MFMAs, 8 no operand reads, 16 no index loads, 32 element-wise epilogue.
-// Sixteen 16-byte loads / stores of agent scope (sc1: coherent between the L2 caches of the GPU's
-// dies without a cache invalidate or write-back), issued together and waited for once.  The
-// compiler waits for every atomic load on its own; a tile handed over in 192 round trips costs
-// 45 us.  `p`: the lane's address; consecutive vectors are 1 KiB apart.
+// Sixteen 16-byte loads / four 16-byte stores of agent scope (sc1: coherent between the L2 caches of
+// the GPU's dies without a cache invalidate or write-back), issued together and waited for once.
+// The compiler waits for every atomic load on its own; a tile handed over in 192 round trips
+// costs 45 us.  `p`: the lane's address; consecutive vectors are 1 KiB apart.
 __device__ __forceinline__ void load16_sc1(const float* p, f32x4 (&v)[16]) {
   asm volatile(
       "global_load_dwordx4 %0, %16, off sc1\n\tglobal_load_dwordx4 %1, %16, off offset:1024 sc1\n\t"
@@ -39,23 +40,220 @@ __device__ __forceinline__ void store4_sc1(float* p, const f32x4& v0, const f32x
       : "memory");
 }
 
+// Loads that write LDS directly: lane l's 16 (4) bytes land at dst + 16 l (4 l); dst is uniform
+// over the wave.  The statements write m0, which the compiler does not let an asm statement declare
+// as clobbered; that is sound as long as the compiler keeps nothing of its own in m0 in these kernels.
+__device__ __forceinline__ void lds_load16(uint32_t dst, uint32_t voff, const void* base) {
+  dst = __builtin_amdgcn_readfirstlane(dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_load4(uint32_t dst, uint32_t voff, const void* base) {
+  dst = __builtin_amdgcn_readfirstlane(dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(voff), "s"(base) : "memory");
+}
+
+// The block's walk over K: step t contracts chunk (t + rot) mod steps of the block's range (column
+// blocks start at different chunks, which spreads the traffic over the L2 channels); steps past the
+// end repeat the last one (their loads land where nobody looks).
+struct KWalk {
+  int chunk0, steps, rot;
+  __device__ __forceinline__ int chunk_of(int step) const {
+    const int kc = min(step, steps - 1) + rot;
+    return chunk0 + (kc >= steps ? kc - steps : kc);
+  }
+};
+
+// What a producer needs to know about its wave: it decodes columns [32 wave, 32 wave + 32) of the
+// block's W tile, lane (c = lane % 32, h = lane / 32) the operands 4h .. 4h + 3 (k = 32 h .. 32 h + 31
+// of the step) of column c, and operand j of a step goes to byte (wave * 4 + j) * 1024 + 16 * lane
+// of the step's W slot.
+struct WaveCtx {
+  int wave, lane, c, h;
+  int ncol;            // the lane's weight row, clamped to N - 1
+  uint8_t* ws;         // W slots, kWRing x 16 KiB
+  uint32_t ws_lds;     // the same as an LDS address
+  uint8_t* stage;      // the block's staging area
+  uint32_t stage_lds;
+};
+
+// ---------------------------------------------------------------------------------------------
+// Producer: VQ, 16-bit indices, vector length 8, codebook in the activation dtype, looked up in
+// memory.  A weight operand is one codebook row: the gather writes the W slot directly.  In step t
+// the wave gathers for step t + 2 (W ring of three) from the indices it staged in step t - 2.
+// ---------------------------------------------------------------------------------------------
+template <int ACT>
+struct T2ProdVq16 {
+  using Args = T2Args;
+  static constexpr int kWRing = 3;
+  static constexpr int kLoads = 5;                 // per step: four gathers, one index load
+  static constexpr int kStageBytes = 4 * 2 * 1024;  // per wave two staged chunks of 64 lanes x 16 bytes
+  const Args& a;
+  const KWalk& kw;
+  const WaveCtx& w;
+  uint32_t idx_row_off;
+  __device__ T2ProdVq16(const Args& args, const KWalk& walk, const WaveCtx& ctx)
+      : a(args), kw(walk), w(ctx), idx_row_off((uint32_t)ctx.ncol * (uint32_t)args.chunks * 16u) {}
+  __device__ __forceinline__ void load_idx(int step, int par) const {
+    lds_load16(w.stage_lds + (uint32_t)((w.wave * 2 + par) * 1024), idx_row_off + (uint32_t)kw.chunk_of(step) * 16u, a.packed);
+  }
+  __device__ __forceinline__ void gathers(int par, int slot) const {
+    const u32x2 v = *reinterpret_cast<const u32x2*>(w.stage + (w.wave * 2 + par) * 1024 + w.lane * 16 + w.h * 8);
+    const uint32_t off[4] = {(uint32_t)(min(v.x & 0xFFFFu, a.nc_minus_1) << 4), (uint32_t)(min(v.x >> 16, a.nc_minus_1) << 4),
+                             (uint32_t)(min(v.y & 0xFFFFu, a.nc_minus_1) << 4), (uint32_t)(min(v.y >> 16, a.nc_minus_1) << 4)};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      lds_load16(w.ws_lds + (uint32_t)(slot * kT2WSlotBytes + (w.wave * 4 + j) * 1024), off[j], a.cb);
+  }
+  // Before the loop: W tiles of steps 0 and 1 requested, indices of steps 2 and 3 requested.
+  __device__ __forceinline__ void prologue_issue() const {
+    load_idx(0, 0);
+    load_idx(1, 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    gathers(0, 0);
+    gathers(1, 1);
+    load_idx(2, 0);
+    load_idx(3, 1);
+  }
+  __device__ __forceinline__ void prologue_finish() const {}
+  // Work behind the MFMAs of k group J, column tile T of step `step` (W slot wslot = step % 3).
+  template <int J, int T>
+  __device__ __forceinline__ void work(int step, int wslot) const {
+    if (J == 0 && T == 0) gathers(step & 1, wslot == 0 ? 2 : wslot - 1);
+    if (J == 0 && T == 1) load_idx(step + 4, step & 1);
+  }
+  __device__ __forceinline__ void work_all(int step, int wslot) const {
+    work<0, 0>(step, wslot);
+    work<0, 1>(step, wslot);
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Producers: int4 / int8 group-affine codes.  Packed bytes and scales go to an LDS staging ring
+// (directly, like everything else the kernel loads, so that one in-order counter tracks all of a
+// wave's loads); in step t the wave requests the bytes of step t + 3, and turns the bytes of step
+// t + 1, which arrived during step t - 1, into four operands that it writes to the other W slot
+// (ring of two): 16 (int4, f16) to 40 VALU instructions per operand, issued between the MFMAs.
+// The arithmetic is the providers' (providers.hpp): bit for bit the one-pass decode.
+// ---------------------------------------------------------------------------------------------
+template <int ACT, int NBITS, bool ASYM>
+struct T2ProdQ {
+  using P = typename std::conditional<NBITS == 4, Q4Provider<ACT, ASYM>, Q8Provider<ACT, ASYM>>::type;
+  using Args = typename P::Args;
+  static constexpr int kWRing = 2;
+  static constexpr int kCodeLoads = NBITS == 4 ? 1 : 2;         // 16 bytes of nibbles, 32 of bytes per lane and step
+  static constexpr int kLoads = kCodeLoads + 1 + (ASYM ? 1 : 0);  // + the dword that holds the scale (+ zero point)
+  static constexpr int kSlot = kCodeLoads * 1024 + 256 + (ASYM ? 256 : 0);
+  static constexpr int kStageWave = 3 * kSlot;
+  static constexpr int kStageBytes = 4 * kStageWave;
+  const Args& a;
+  const KWalk& kw;
+  const WaveCtx& w;
+  const P prov;
+  uint32_t code_off;   // byte offset of the lane's share of chunk 0 of its row
+  uint32_t scale_row;  // index of the row's first scale
+  int req_slot = 0;    // staging slot of the next request (the bytes of step s live in slot s % 3)
+  int fetch_slot = 0;  // staging slot of the next step to decode
+  u32x4 raw0, raw1;    // the step being decoded
+  uint32_t s2, z;
+  __device__ T2ProdQ(const Args& args, const KWalk& walk, const WaveCtx& ctx)
+      : a(args), kw(walk), w(ctx), prov(args),
+        code_off((uint32_t)ctx.ncol * (uint32_t)args.chunks * (NBITS == 4 ? 32u : 64u) + (uint32_t)ctx.h * (NBITS == 4 ? 16u : 32u)),
+        scale_row((uint32_t)ctx.ncol * (uint32_t)args.groups_per_row) {}
+  __device__ __forceinline__ uint32_t scale_index(int step) const {
+    return scale_row + (uint32_t)((2 * kw.chunk_of(step) + w.h) >> a.gs_shift_chunks);
+  }
+  __device__ __forceinline__ void request(int step) {
+    const uint32_t dst = w.stage_lds + (uint32_t)(w.wave * kStageWave + req_slot * kSlot);
+    const uint32_t off = code_off + (uint32_t)kw.chunk_of(step) * (NBITS == 4 ? 32u : 64u);
+    lds_load16(dst, off, a.w_pack);
+    if (NBITS == 8) lds_load16(dst + 1024, off + 16u, a.w_pack);
+    const uint32_t sb = (scale_index(step) * 2u) & ~3u;
+    lds_load4(dst + kCodeLoads * 1024, sb, a.scale);
+    if (ASYM) lds_load4(dst + kCodeLoads * 1024 + 256, sb, a.zp);
+    req_slot = req_slot == 2 ? 0 : req_slot + 1;
+  }
+  // Reads the staged bytes of `step`; steps are requested and fetched in order.
+  __device__ __forceinline__ void fetch(int step) {
+    const uint8_t* src = w.stage + w.wave * kStageWave + fetch_slot * kSlot;
+    fetch_slot = fetch_slot == 2 ? 0 : fetch_slot + 1;
+    raw0 = *reinterpret_cast<const u32x4*>(src + w.lane * 16);
+    if (NBITS == 8) raw1 = *reinterpret_cast<const u32x4*>(src + 1024 + w.lane * 16);
+    const uint32_t sh = (scale_index(step) & 1u) * 16u;
+    const uint32_t sd = *reinterpret_cast<const uint32_t*>(src + kCodeLoads * 1024 + w.lane * 4);
+    s2 = ((sd >> sh) & 0xFFFFu) * 0x10001u;
+    z = 0;
+    if (ASYM) z = (*reinterpret_cast<const uint32_t*>(src + kCodeLoads * 1024 + 256 + w.lane * 4) >> sh) & 0xFFFFu;
+  }
+  template <int O>
+  __device__ __forceinline__ void decode(int wslot) const {
+    u32x4 op;
+    if constexpr (NBITS == 4) {
+      op = prov.dequant8(O == 0 ? raw0.x : O == 1 ? raw0.y : O == 2 ? raw0.z : raw0.w, s2, z);
+    } else {
+      const u32x4& r = O < 2 ? raw0 : raw1;
+      op = prov.dequant8((O & 1) ? r.z : r.x, (O & 1) ? r.w : r.y, s2, z);
+    }
+    *reinterpret_cast<u32x4*>(w.ws + wslot * kT2WSlotBytes + (w.wave * 4 + O) * 1024 + w.lane * 16) = op;
+  }
+  __device__ __forceinline__ void prologue_issue() {
+    request(0);
+    request(1);
+    request(2);
+  }
+  // Everything requested has arrived: the W tile of step 0.
+  __device__ __forceinline__ void prologue_finish() {
+    fetch(0);
+    decode<0>(0);
+    decode<1>(0);
+    decode<2>(0);
+    decode<3>(0);
+  }
+  template <int J, int T>
+  __device__ __forceinline__ void work(int step, int wslot) {
+    if (J == 0 && T == 0) request(step + 3);
+    if (J == 0 && T == 1) fetch(step + 1);
+    if (J == 0 && T == 2) decode<0>(wslot ^ 1);
+    if (J == 0 && T == 3) decode<1>(wslot ^ 1);
+    if (J == 1 && T == 0) decode<2>(wslot ^ 1);
+    if (J == 1 && T == 1) decode<3>(wslot ^ 1);
+  }
+  __device__ __forceinline__ void work_all(int step, int wslot) {
+    request(step + 3);
+    fetch(step + 1);
+    decode<0>(wslot ^ 1);
+    decode<1>(wslot ^ 1);
+    decode<2>(wslot ^ 1);
+    decode<3>(wslot ^ 1);
+  }
+};
+
+template <int MW, class Prod>
+struct T2Lds {
+  static constexpr int kXBufBytes = 128 * MW * kStepK * 2;
+  static constexpr int kBytes = 2 * kXBufBytes + Prod::kWRing * kT2WSlotBytes + Prod::kStageBytes;
+  static_assert(kBytes <= kLdsPerBlockMax, "the block's tiles do not fit LDS");
+};
+
+// ABL (builds with -DNPAMD_TILE2_ABLATIONS only; 0 in the library): parts of the step compiled out, to time the
+// others -- 1 no weight tile (the producer's work), 2 no x loads, 4 no MFMAs, 8 no operand reads, 32 element-wise epilogue.
 #ifdef NPAMD_TILE2_ABLATIONS
 __device__ unsigned long long* g_t2_debug = nullptr;
 #endif
-template <int ACT, int MW, int ABL = 0>
+template <int ACT, int MW, class Prod, int ABL = 0>
 __global__ void __launch_bounds__(256)
-tile2_gemm_kernel(const GemmShape s, const T2Args a) {
+tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pair pair) {
 #ifdef NPAMD_TILE2_ABLATIONS
   const unsigned long long t_start = __builtin_amdgcn_s_memrealtime();
 #endif
-  constexpr int kNG = (ABL & 1) ? 0 : 4, kNI = (ABL & 16) ? 0 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = 128 * MW;
-  constexpr int kXBufBytes = T2Lds<MW>::kXBufBytes;
+  constexpr int kXBufBytes = T2Lds<MW, Prod>::kXBufBytes;
   constexpr int kPieces = 4 * MW;  // x-tile load instructions per wave and step (8 rows each)
-  uint8_t* const xs = lds;                                   // [2][BM][128]
-  uint8_t* const ws = lds + 2 * kXBufBytes;                  // [3][16 KiB]
-  uint8_t* const is = ws + kT2WRing * kT2WSlotBytes;         // [4 waves][2][1 KiB]
+  constexpr int kWRing = Prod::kWRing;
+  constexpr int kProdLoads = (ABL & 1) ? 0 : Prod::kLoads;
+  uint8_t* const xs = lds;                              // [2][BM][128]
+  uint8_t* const ws = lds + 2 * kXBufBytes;             // [kWRing][16 KiB]
+  uint8_t* const stage = ws + kWRing * kT2WSlotBytes;   // the producer's staging area
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -64,43 +262,24 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
   const int h = lane >> 5;
   const int m0 = blockIdx.y * BM;
   const int n0 = blockIdx.x * kT2Cols;
-  const int chunk0 = blockIdx.z * s.split_chunks;
-  const int steps = min(s.split_chunks, s.chunks - chunk0);
-  const int rot = (int)((blockIdx.x * 7u) % (unsigned)steps);
-  auto chunk_of = [&](int step) {
-    const int kc = min(step, steps - 1) + rot;
-    return chunk0 + (kc >= steps ? kc - steps : kc);
-  };
+  KWalk kw;
+  kw.chunk0 = blockIdx.z * s.split_chunks;
+  kw.steps = min(s.split_chunks, s.chunks - kw.chunk0);
+  kw.rot = (int)((blockIdx.x * 7u) % (unsigned)kw.steps);
+  const int steps = kw.steps;
 
   const uint32_t xs_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)xs;
-  const uint32_t ws_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)ws;
-  const uint32_t is_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)is;
-
-  // ---- W tile: indices and gathers -----------------------------------------------------------
-  const int ncol = min(n0 + 32 * wave + c, s.N - 1);  // columns past N decode a valid row nobody stores
-  const uint32_t idx_row_off = (uint32_t)ncol * (uint32_t)s.chunks * 16u;  // byte offset of the column's first chunk
-  auto load_idx = [&](int step, int par) {
-    if (ABL & 16) return;
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(is_lds + (uint32_t)((wave * 2 + par) * 1024));
-    const uint32_t off = idx_row_off + (uint32_t)chunk_of(step) * 16u;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(a.packed)
-                 : "memory");
-  };
-  auto row_off16 = [&](uint32_t i) { return (uint32_t)(min(i, a.nc_minus_1) << 4); };
-  auto gather_rows = [&](const u32x2 v, int slot) {
-    if (ABL & 1) return;
-    const uint32_t off[4] = {row_off16(v.x & 0xFFFFu), row_off16(v.x >> 16), row_off16(v.y & 0xFFFFu), row_off16(v.y >> 16)};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t dst =
-          __builtin_amdgcn_readfirstlane(ws_lds + (uint32_t)(slot * kT2WSlotBytes + (wave * 4 + j) * 1024));
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off[j]), "s"(a.cb)
-                   : "memory");
-    }
-  };
-  auto gathers = [&](int par, int slot) {
-    gather_rows(*reinterpret_cast<const u32x2*>(is + (wave * 2 + par) * 1024 + lane * 16 + h * 8), slot);
-  };
+  WaveCtx wc;
+  wc.wave = wave;
+  wc.lane = lane;
+  wc.c = c;
+  wc.h = h;
+  wc.ncol = min(n0 + 32 * wave + c, s.N - 1);  // columns past N decode a valid row nobody stores
+  wc.ws = ws;
+  wc.ws_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)ws;
+  wc.stage = stage;
+  wc.stage_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)stage;
+  Prod prod(pargs, kw, wc);
 
   // ---- x tile ----------------------------------------------------------------------------------
   const int wrow0 = wave * (32 * MW);
@@ -117,20 +296,12 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
   const uint32_t wave_x_lds = xs_lds + (uint32_t)(wrow0 * 128);
   auto fetch_piece = [&](int i, int buf, const uint8_t* src) {
     if (ABL & 2) return;
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(wave_x_lds + (uint32_t)(buf * kXBufBytes + i * 1024));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff[i]), "s"(src)
-                 : "memory");
+    lds_load16(wave_x_lds + (uint32_t)(buf * kXBufBytes + i * 1024), voff[i], src);
   };
-  auto tile_src = [&](int step) { return xbase + (int64_t)chunk_of(step) * (kStepK * 2); };
+  auto tile_src = [&](int step) { return xbase + (int64_t)kw.chunk_of(step) * (kStepK * 2); };
 
-  // ---- prologue: indices of steps 0..3, W tiles and x tiles of steps 0 and 1 -------------------
-  load_idx(0, 0);
-  load_idx(1, 1);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  gathers(0, 0);
-  gathers(1, 1);
-  load_idx(2, 0);
-  load_idx(3, 1);
+  // ---- prologue ----------------------------------------------------------------------------------
+  if (!(ABL & 1)) prod.prologue_issue();
   if (wave_active) {
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -140,6 +311,7 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (!(ABL & 1)) prod.prologue_finish();
   block_sync_lds();
 
   f32x16 acc[MW][4];
@@ -166,14 +338,12 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
       for (int mt = 0; mt < MW; ++mt) ao[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * 128);
     };
     // One step; buf = step % 2 is a compile-time constant through the unrolled loops below.
-    // The step's loads are issued behind MFMAs: the gathers of step + 2 and the next indices in k
-    // group 0, the x tile of step + 2 in k group 3, whose operands are the last this step reads
-    // from the buffer the tile goes into (the wait in front of the first piece makes sure they
-    // have arrived, wherever the scheduler puts that piece among the group's MFMAs).
+    // The step's loads are issued behind MFMAs: the producer's in k groups 0 and 1, the x tile of
+    // step + 2 in k group 3, whose operands are the last this step reads from the buffer the tile
+    // goes into (the wait in front of the first piece makes sure they have arrived, wherever the
+    // scheduler puts that piece among the group's MFMAs).
     auto one_step = [&](int buf, int step, int wslot) {
-      const int gslot = wslot == 0 ? 2 : wslot - 1;  // (step + 2) % 3
       read_ops(0, buf, wslot, 0);
-      const u32x2 iv = *reinterpret_cast<const u32x2*>(is + (wave * 2 + buf) * 1024 + lane * 16 + h * 8);
       const uint8_t* src = tile_src(step + 2);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -184,8 +354,14 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
 #pragma unroll
           for (int mt = 0; mt < MW; ++mt)
             if (!(ABL & 4)) acc[mt][t] = mfma32<ACT>(ao[j & 1][mt], bo[j & 1][t], acc[mt][t]);
-          if (j == 0 && t == 0) gather_rows(iv, gslot);
-          if (j == 0 && t == 1) load_idx(step + 4, buf);
+          if (!(ABL & 1)) {
+            if (j == 0 && t == 0) prod.template work<0, 0>(step, wslot);
+            if (j == 0 && t == 1) prod.template work<0, 1>(step, wslot);
+            if (j == 0 && t == 2) prod.template work<0, 2>(step, wslot);
+            if (j == 0 && t == 3) prod.template work<0, 3>(step, wslot);
+            if (j == 1 && t == 0) prod.template work<1, 0>(step, wslot);
+            if (j == 1 && t == 1) prod.template work<1, 1>(step, wslot);
+          }
           if (j == 3 && t < 3) {
             if (t == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -194,7 +370,7 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kNG + kNI + ((ABL & 2) ? 0 : kPieces)) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kProdLoads + ((ABL & 2) ? 0 : kPieces)) : "memory");
       block_sync_lds();
     };
     int wslot = 0;
@@ -203,7 +379,7 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
 #pragma unroll
       for (int d = 0; d < 2; ++d) {
         one_step(d, t0 + d, wslot);
-        wslot = wslot == kT2WRing - 1 ? 0 : wslot + 1;
+        wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
       }
     }
     if (whole < steps) one_step(0, whole, wslot);
@@ -211,12 +387,10 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
     // No rows of this wave lie inside M: it still decodes its 32 columns for the others.
     int wslot = 0;
     for (int t = 0; t < steps; ++t) {
-      const int gslot = wslot == 0 ? 2 : wslot - 1;
-      gathers(t & 1, gslot);
-      load_idx(t + 4, t & 1);
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kNG + kNI) : "memory");
+      if (!(ABL & 1)) prod.work_all(t, wslot);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kProdLoads) : "memory");
       block_sync_lds();
-      wslot = wslot == kT2WRing - 1 ? 0 : wslot + 1;
+      wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
     }
   }
   // Nothing may still be on its way into LDS when the wave ends.
@@ -234,20 +408,23 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
   // ---- epilogue: D[m = 8 (i / 4) + 4 h + i % 4][n = c] of each 32 x 32 tile ---------------------
   bool finish = true;
   if (s.splits == 2) {
-    // Registers as they are, 256 bytes per store instruction: [tile][wave][register 0 .. 64 MW)[lane] floats.
-    // Stores and loads of the tile and the counter are relaxed atomics of agent scope, i.e. they
-    // bypass the caches that are not shared by the whole GPU: no cache is written back or
-    // invalidated to hand the tile over (an agent-scope fence does both for a whole L2, under
-    // the other workgroups still running their loops).
+    // Whichever workgroup of the pair arrives first stores its f32 tile and counts itself in; the
+    // other adds that tile to its registers.  Stores and loads of the tile and the counter are of
+    // agent scope (sc1): they bypass the caches that are not shared by the whole GPU (every die has
+    // an L2 of its own), so no cache is written back or invalidated to hand the tile over (an
+    // agent-scope fence does both for a whole L2, under the workgroups still running their loops).
+    // Measured and dropped: ordinary stores and loads when both halves run on the same die (each
+    // said so at its start): the tiles then sit dirty in that die's L2, 2.7 of its 4 MiB at 384
+    // tokens, and the last workgroups finish 6 us later than with the trip through memory.
     const int tile_id = blockIdx.y * gridDim.x + blockIdx.x;
     const int tiles = gridDim.x * gridDim.y;
     constexpr int kTileFloats = BM * kT2Cols;
     // [tile][wave][row tile mt][column tile t][quarter q][lane] float4: 1 KiB per instruction
-    float* const mine = a.pair_tiles + ((size_t)blockIdx.z * tiles + tile_id) * kTileFloats + wave * (MW * 64 * 64) + lane * 4;
+    float* const mine = pair.tiles + ((size_t)blockIdx.z * tiles + tile_id) * kTileFloats + wave * (MW * 64 * 64) + lane * 4;
     const float* const theirs =
-        a.pair_tiles + ((size_t)(blockIdx.z ^ 1) * tiles + tile_id) * kTileFloats + wave * (MW * 64 * 64) + lane * 4;
-    uint32_t* const flag = reinterpret_cast<uint32_t*>(is);  // outside the waves' output areas
-    uint32_t* const cnt = a.counters + tile_id;
+        pair.tiles + ((size_t)(blockIdx.z ^ 1) * tiles + tile_id) * kTileFloats + wave * (MW * 64 * 64) + lane * 4;
+    uint32_t* const flag = reinterpret_cast<uint32_t*>(ws);  // outside the waves' output areas
+    uint32_t* const cnt = pair.counters + tile_id;
     __syncthreads();  // every wave is past its last LDS read
     if (tid == 0) flag[0] = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
@@ -274,14 +451,14 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
       if (tid == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next call
       if (wave_active) {
 #pragma unroll
-        for (int mt = 0; mt < MW; ++mt) {
-          f32x4 v[16];
-          load16_sc1(theirs + mt * 4096, v);
+          for (int mt = 0; mt < MW; ++mt) {
+            f32x4 v[16];
+            load16_sc1(theirs + mt * 4096, v);
 #pragma unroll
-          for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[mt][t][i] += v[t * 4 + i / 4][i % 4];
-        }
+              for (int i = 0; i < 16; ++i) acc[mt][t][i] += v[t * 4 + i / 4][i % 4];
+          }
       }
     }
   }
@@ -321,20 +498,20 @@ tile2_gemm_kernel(const GemmShape s, const T2Args a) {
   }
 }
 
-template <int ACT, int MW, int ABL = 0>
-int launch_tile2_mw(GemmShape s, T2Args a, hipStream_t st, const char* what) {
+template <int ACT, int MW, class Prod, int ABL = 0>
+int launch_tile2_mw(const GemmShape& s, const typename Prod::Args& a, const T2Pair& pair, hipStream_t st, const char* what) {
   constexpr int BM = 128 * MW;
   const dim3 grid((s.N + kT2Cols - 1) / kT2Cols, (s.M + BM - 1) / BM, s.splits);
-  constexpr int lds = T2Lds<MW>::kBytes;
+  constexpr int lds = T2Lds<MW, Prod>::kBytes;
   static LdsLatch latch;
-  const hipError_t e = enable_dynamic_lds(latch, reinterpret_cast<const void*>(&tile2_gemm_kernel<ACT, MW, ABL>), lds);
+  const hipError_t e = enable_dynamic_lds(latch, reinterpret_cast<const void*>(&tile2_gemm_kernel<ACT, MW, Prod, ABL>), lds);
   if (e != hipSuccess)
     return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
   if (s.splits == 2) {
     const int tiles = (int)(grid.x * grid.y);
-    tile2_zero_counters_kernel<<<(tiles + 255) / 256, 256, 0, st>>>(a.counters, tiles);
+    tile2_zero_counters_kernel<<<(tiles + 255) / 256, 256, 0, st>>>(pair.counters, tiles);
   }
-  tile2_gemm_kernel<ACT, MW, ABL><<<grid, 256, lds, st>>>(s, a);
+  tile2_gemm_kernel<ACT, MW, Prod, ABL><<<grid, 256, lds, st>>>(s, a, pair);
   if (s.splits > 2) {
     const int64_t quads = (int64_t)s.M * ((s.N + 3) / 4);
     splitk_reduce_kernel<ACT><<<(unsigned)((quads + 255) / 256), 256, 0, st>>>(s.partials, s.splits, s.M, s.N,
@@ -343,72 +520,90 @@ int launch_tile2_mw(GemmShape s, T2Args a, hipStream_t st, const char* what) {
   return check_launch(what);
 }
 
-template <int ACT>
-int launch_tile2_act(GemmShape s, T2Args a, hipStream_t st, const char* what, void* workspace, int64_t workspace_bytes) {
-  const int mw = plan_tile_mw(s.M);
-  int splits = plan_tile2_splits(s.M, s.N, s.chunks, mw);
+// Plans the split, carves the workspace and picks the row-tile count; returns 1 when the
+// workspace does not allow the planned split (the caller then takes the 64-column kernel).
+template <int ACT, class Prod>
+int launch_tile2_prod(GemmShape s, const typename Prod::Args& a, hipStream_t st, const char* what, void* workspace,
+                      int64_t workspace_bytes, int mw) {
+  const int splits = plan_tile2_splits(s.M, s.N, s.chunks, mw);
   if (splits > 1 && (!workspace || tile2_workspace_bytes(s.M, s.N, s.chunks, mw) > workspace_bytes)) return 1;
   s.steps = s.chunks;
   s.split_chunks = (s.chunks + splits - 1) / splits;
   s.splits = (s.chunks + s.split_chunks - 1) / s.split_chunks;
   s.partials = (float*)workspace;
+  T2Pair pair{nullptr, nullptr};
   if (s.splits == 2) {
     const int64_t tiles = (int64_t)((s.N + kT2Cols - 1) / kT2Cols) * ((s.M + 128 * mw - 1) / (128 * mw));
-    a.counters = (uint32_t*)workspace;
-    a.pair_tiles = (float*)((uint8_t*)workspace + ((tiles * 4 + 255) & ~(int64_t)255));
+    pair.counters = (uint32_t*)workspace;
+    pair.tiles = (float*)((uint8_t*)workspace + ((tiles * 4 + 255) & ~(int64_t)255));
   }
-#ifdef NPAMD_TILE2_ABLATIONS
-  if constexpr (ACT == NPAMD_BF16) {
-    const char* e = getenv("NPAMD_T2_ABL");
-    const int abl = e ? atoi(e) : 0;
-    if (abl && mw == 3) {
-      switch (abl) {
-        case 32: return launch_tile2_mw<ACT, 3, 32>(s, a, st, what);
-        case 27: return launch_tile2_mw<ACT, 3, 27>(s, a, st, what);
-        case 23: return launch_tile2_mw<ACT, 3, 23>(s, a, st, what);
-        case 51: return launch_tile2_mw<ACT, 3, 51>(s, a, st, what);
-        case 1: return launch_tile2_mw<ACT, 3, 1>(s, a, st, what);
-        case 2: return launch_tile2_mw<ACT, 3, 2>(s, a, st, what);
-        case 4: return launch_tile2_mw<ACT, 3, 4>(s, a, st, what);
-        case 8: return launch_tile2_mw<ACT, 3, 8>(s, a, st, what);
-        case 16: return launch_tile2_mw<ACT, 3, 16>(s, a, st, what);
-        case 17: return launch_tile2_mw<ACT, 3, 17>(s, a, st, what);
-        case 14: return launch_tile2_mw<ACT, 3, 14>(s, a, st, what);
-        case 12: return launch_tile2_mw<ACT, 3, 12>(s, a, st, what);
-        case 19: return launch_tile2_mw<ACT, 3, 19>(s, a, st, what);
-        case 31: return launch_tile2_mw<ACT, 3, 31>(s, a, st, what);
-        case 3: return launch_tile2_mw<ACT, 3, 3>(s, a, st, what);
-      }
-    }
-    if (abl && mw == 1) {
-      switch (abl) {
-        case 1: return launch_tile2_mw<ACT, 1, 1>(s, a, st, what);
-        case 2: return launch_tile2_mw<ACT, 1, 2>(s, a, st, what);
-        case 16: return launch_tile2_mw<ACT, 1, 16>(s, a, st, what);
-        case 14: return launch_tile2_mw<ACT, 1, 14>(s, a, st, what);
-        case 30: return launch_tile2_mw<ACT, 1, 30>(s, a, st, what);
-        case 31: return launch_tile2_mw<ACT, 1, 31>(s, a, st, what);
-      }
-    }
-  }
-#endif
-  switch (mw) {
-    case 1: return launch_tile2_mw<ACT, 1>(s, a, st, what);
-    case 2: return launch_tile2_mw<ACT, 2>(s, a, st, what);
-    default: return launch_tile2_mw<ACT, 3>(s, a, st, what);
-  }
-}
-
-
-int launch_tile2(int act, GemmShape s, T2Args a, hipStream_t st, const char* what, void* workspace, int64_t workspace_bytes) {
 #ifdef NPAMD_TILE2_ABLATIONS
   if (const char* e = getenv("NPAMD_T2_DEBUG_PTR")) {
     unsigned long long* p = (unsigned long long*)strtoull(e, nullptr, 10);
     (void)hipMemcpyToSymbol(HIP_SYMBOL(g_t2_debug), &p, sizeof(p));
   }
+  if constexpr (ACT == NPAMD_BF16 || std::is_same<Prod, T2ProdQ<NPAMD_F16, 4, false>>::value) {
+    const char* e = getenv("NPAMD_T2_ABL");
+    const int abl = e ? atoi(e) : 0;
+    if (abl && mw == 3) {
+      switch (abl) {
+        case 1: return launch_tile2_mw<ACT, 3, Prod, 1>(s, a, pair, st, what);
+        case 2: return launch_tile2_mw<ACT, 3, Prod, 2>(s, a, pair, st, what);
+        case 4: return launch_tile2_mw<ACT, 3, Prod, 4>(s, a, pair, st, what);
+        case 3: return launch_tile2_mw<ACT, 3, Prod, 3>(s, a, pair, st, what);
+        case 6: return launch_tile2_mw<ACT, 3, Prod, 6>(s, a, pair, st, what);
+        case 11: return launch_tile2_mw<ACT, 3, Prod, 11>(s, a, pair, st, what);
+        case 15: return launch_tile2_mw<ACT, 3, Prod, 15>(s, a, pair, st, what);
+      }
+    }
+    if (abl && mw == 2) {
+      switch (abl) {
+        case 1: return launch_tile2_mw<ACT, 2, Prod, 1>(s, a, pair, st, what);
+        case 2: return launch_tile2_mw<ACT, 2, Prod, 2>(s, a, pair, st, what);
+        case 4: return launch_tile2_mw<ACT, 2, Prod, 4>(s, a, pair, st, what);
+        case 3: return launch_tile2_mw<ACT, 2, Prod, 3>(s, a, pair, st, what);
+        case 6: return launch_tile2_mw<ACT, 2, Prod, 6>(s, a, pair, st, what);
+        case 11: return launch_tile2_mw<ACT, 2, Prod, 11>(s, a, pair, st, what);
+        case 15: return launch_tile2_mw<ACT, 2, Prod, 15>(s, a, pair, st, what);
+      }
+    }
+  }
 #endif
-  return act == NPAMD_BF16 ? launch_tile2_act<NPAMD_BF16>(s, a, st, what, workspace, workspace_bytes)
-                           : launch_tile2_act<NPAMD_F16>(s, a, st, what, workspace, workspace_bytes);
+  switch (mw) {
+    case 1: return launch_tile2_mw<ACT, 1, Prod>(s, a, pair, st, what);
+    case 2: return launch_tile2_mw<ACT, 2, Prod>(s, a, pair, st, what);
+    default: return launch_tile2_mw<ACT, 3, Prod>(s, a, pair, st, what);
+  }
+}
+
+int launch_tile2(int act, const GemmShape& s, const T2Args& a, hipStream_t st, const char* what, void* workspace,
+                 int64_t workspace_bytes) {
+  const int mw = plan_tile_mw(s.M);
+  return act == NPAMD_BF16 ? launch_tile2_prod<NPAMD_BF16, T2ProdVq16<NPAMD_BF16>>(s, a, st, what, workspace, workspace_bytes, mw)
+                           : launch_tile2_prod<NPAMD_F16, T2ProdVq16<NPAMD_F16>>(s, a, st, what, workspace, workspace_bytes, mw);
+}
+
+template <int ACT, int NBITS>
+static int launch_tile2_q_bits(bool asym, const GemmShape& s, const T2QArgs& q, hipStream_t st, const char* what,
+                               void* workspace, int64_t workspace_bytes) {
+  if (asym) {
+    using Prod = T2ProdQ<ACT, NBITS, true>;
+    const typename Prod::Args a{q.w_pack, q.scale, q.chunks, q.groups_per_row, q.gs_shift_chunks, q.zp};
+    return launch_tile2_prod<ACT, Prod>(s, a, st, what, workspace, workspace_bytes, plan_tile2_q_mw(s.M));
+  }
+  using Prod = T2ProdQ<ACT, NBITS, false>;
+  const typename Prod::Args a{q.w_pack, q.scale, q.chunks, q.groups_per_row, q.gs_shift_chunks, q.zp};
+  return launch_tile2_prod<ACT, Prod>(s, a, st, what, workspace, workspace_bytes, plan_tile2_q_mw(s.M));
+}
+
+int launch_tile2_q(int act, int nbits, const GemmShape& s, const T2QArgs& q, hipStream_t st, const char* what,
+                   void* workspace, int64_t workspace_bytes) {
+  const bool asym = q.zp != nullptr;
+  if (act == NPAMD_BF16)
+    return nbits == 4 ? launch_tile2_q_bits<NPAMD_BF16, 4>(asym, s, q, st, what, workspace, workspace_bytes)
+                      : launch_tile2_q_bits<NPAMD_BF16, 8>(asym, s, q, st, what, workspace, workspace_bytes);
+  return nbits == 4 ? launch_tile2_q_bits<NPAMD_F16, 4>(asym, s, q, st, what, workspace, workspace_bytes)
+                    : launch_tile2_q_bits<NPAMD_F16, 8>(asym, s, q, st, what, workspace, workspace_bytes);
 }
 
 }  // namespace npamd

@@ -44,21 +44,28 @@ namespace npamd {
 constexpr int kT2Cols = 128;
 constexpr int kT2WSlotBytes = kT2Cols * kStepK * 2;  // 16 KiB: [column tile 4][operand j 4][lane 64][16 B]
 constexpr int kT2WRing = 3;
-constexpr int kT2IdxBytes = 4 * 2 * 1024;  // per wave two staged chunks of 64 lanes x 16 bytes
 
 struct T2Args {
   const uint8_t* packed;  // 16-bit indices, [N][K / 8]
   const void* cb;         // [nc][8] in the activation dtype
   uint32_t nc_minus_1;
   int chunks;             // K / 64
-  uint32_t* counters;     // splits == 2: one arrival counter per block tile, zero on entry
-  float* pair_tiles;      // splits == 2: [2][tiles][BM * 128] f32 in register order
 };
 
-template <int MW>
-struct T2Lds {
-  static constexpr int kXBufBytes = 128 * MW * kStepK * 2;
-  static constexpr int kBytes = 2 * kXBufBytes + kT2WRing * kT2WSlotBytes + kT2IdxBytes;
+// int4 / int8 group-affine codes (group size a multiple of 32): what the providers of the 64-column kernel take.
+struct T2QArgs {
+  const uint8_t* w_pack;
+  const uint16_t* scale;  // 4-byte aligned
+  int chunks, groups_per_row, gs_shift_chunks;
+  const uint16_t* zp;     // null: symmetric
+};
+
+// K in two halves: one arrival counter per block tile (zeroed by a fill kernel in front of the GEMM,
+// zero again on exit) and the f32 tile of whichever half finished first, [2][tiles][BM * 128] in
+// register order.
+struct T2Pair {
+  uint32_t* counters;
+  float* tiles;
 };
 
 // Splits of K for the 128-column kernel: 1 while the block tiles cover most compute units, else as
@@ -66,6 +73,13 @@ struct T2Lds {
 int plan_tile2_splits(int M, int N, int chunks, int mw);
 // 0: never take the 128-column kernel, 1: where it is the faster one (default), 2: wherever it applies.
 int tile2_mode();
+
+// Row tiles per wave for the group-affine producers, whose decode is cheap enough to repeat per row block: past
+// 384 tokens two (256-row blocks: int4 14336 x 4096 at 512 / 1024 tokens 77 / 155 us against 97 / 173 with three).
+inline int plan_tile2_q_mw(int M) {
+  const int mw = plan_tile_mw(M);
+  return M > 384 && mw == 3 ? 2 : mw;
+}
 
 inline int64_t tile2_workspace_bytes(int M, int N, int chunks, int mw) {
   const int splits = plan_tile2_splits(M, N, chunks, mw);
@@ -75,8 +89,11 @@ inline int64_t tile2_workspace_bytes(int M, int N, int chunks, int mw) {
   return ((tiles * 4 + 255) & ~(int64_t)255) + 2 * tiles * (128 * mw) * kT2Cols * 4;
 }
 
-// Takes the call when the workspace allows the planned split; returns 1 when it did not take it.
+// Take the call when the workspace allows the planned split; return 1 when they did not take it.
 // act: NPAMD_F16 or NPAMD_BF16 (activations, codebook and output).
-int launch_tile2(int act, GemmShape s, T2Args a, hipStream_t st, const char* what, void* workspace, int64_t workspace_bytes);
+int launch_tile2(int act, const GemmShape& s, const T2Args& a, hipStream_t st, const char* what, void* workspace,
+                 int64_t workspace_bytes);
+int launch_tile2_q(int act, int nbits, const GemmShape& s, const T2QArgs& q, hipStream_t st, const char* what,
+                   void* workspace, int64_t workspace_bytes);
 
 }  // namespace npamd

@@ -7,7 +7,7 @@
 // combination (1/2 bits, odd group sizes, odd K) runs the element-wise fallback.
 #include <stdlib.h>
 
-#include "gemm_tile.hpp"
+#include "gemm_tile2.hpp"
 #include "gemv.hpp"
 
 namespace npamd {
@@ -645,9 +645,27 @@ static int q8_fused(const QCall& c, bool gemv) {
   return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
+// The 128-column tile GEMM (gemm_tile2.hpp) for int4 / int8: 0 when it took the call.
+static int q_tile_wide(const QCall& c) {
+  const int mode = tile2_mode();
+  // Measured against the 64-column kernel, int4, us: 14336 x 4096 at 128 / 256 / 384 / 512 / 1024 tokens 36.7 / 53.5 /
+  // 67.7 / 77.2 / 155 against 37.0 / 52.5 / 75.2 / 113 / 193; 4096 x 14336 38.6 / 55.1 / 72.8 / 83.8 / 143 against
+  // 40.7 / 59.9 / 79.7 / 118 / 200; 4096 x 4096 behind at every count (more than two splits of K).
+  const bool wins = (c.K >= 8192 && c.M >= 128) || (c.N >= 8192 && c.M > 256);
+  if (!(mode >= 2 || (mode == 1 && wins))) return 1;
+  if (!ptr_aligned(c.scale, 4) || (c.zp && !ptr_aligned(c.zp, 4)) || (int64_t)c.N * c.K >= ((int64_t)1 << 32)) return 1;
+  const GemmShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, c.K / 64, 0};
+  const T2QArgs q{c.w_pack, (const uint16_t*)c.scale, c.K / 64, c.K / c.gs, log2i(c.gs / 32), (const uint16_t*)c.zp};
+  return launch_tile2_q(c.act, c.nbits, s, q, c.st, c.what, c.ws, c.ws_bytes);
+}
+
 template <int ACT>
 static int q_dispatch(const QCall& c, bool gemv) {
   if (q_fast_ok(c)) {
+    if (!gemv) {
+      const int rc = q_tile_wide(c);
+      if (rc != 1) return rc;
+    }
     if (c.nbits == 8) return c.zp ? q8_fused<ACT, true>(c, gemv) : q8_fused<ACT, false>(c, gemv);
     if (gemv && q4_rowwise_ok(c)) {
       Q4StreamGeom geo;

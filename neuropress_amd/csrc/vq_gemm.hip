@@ -24,7 +24,7 @@ int run_vq(const VqCall& c, const GemmShape& s) {
     // by 3 to 19 % on 4096 x 4096 and 1024 x 4096, where more than two splits of K meet in a second kernel.
     const bool wins = big && (c.N >= 8192 || c.K >= 8192);
     if (c.cb_dtype == c.act && c.n_bytes < ((int64_t)1 << 32) && (mode >= 2 || (mode == 1 && wins))) {
-      T2Args t2{c.packed, c.cb, (uint32_t)c.nc - 1u, s.chunks, nullptr, nullptr};
+      const T2Args t2{c.packed, c.cb, (uint32_t)c.nc - 1u, s.chunks};
       const int rc = launch_tile2(ACT, s, t2, c.st, c.what, c.ws, c.ws_bytes);
       if (rc != 1) return rc;
     }

@@ -104,3 +104,48 @@ def test_wide_and_narrow_tile_gemm_agree_on_a_large_layer(gpu, tile_wide):
         assert bool((err <= 1e-2 + 1e-2 * ref.abs()).all()), float(err.max())
     # same products, f32 sums in a different order: they differ by output roundings at most
     assert float((y_auto.float() - y_narrow.float()).abs().max()) <= 2.0 ** -6
+
+
+def _q_ref(oracle_lib, L, act):
+    code = orc.torch_dtype_code(act)
+    zp = None if L["zp"] is None else orc.to_bits(L["zp"])
+    w = oracle_lib.q_decode(L["blob"].numpy(), orc.to_bits(L["scale"]), zp, L["nbits"], L["gs"], code)
+    bias = None if L["bias"] is None else orc.to_bits(L["bias"])
+    return oracle_lib.linear_f64(orc.to_bits(L["x"]), code, w, code, bias, code)
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("nbits,asym,gs", [(4, False, 32), (4, True, 32), (4, False, 128), (8, False, 32), (8, True, 64)])
+@pytest.mark.parametrize("m", [1, 17, 130, 257, 384, 400, 520])
+@pytest.mark.parametrize("n,k,splits", [(300, 512, 1), (300, 512, 2), (264, 1024, 3)])
+def test_wide_tile_gemm_group_affine_against_the_oracle(gpu, oracle_lib, tile_wide, act, nbits, asym, gs, m, n, k, splits):
+    """int4 / int8 codes through the 128-column kernel (packed bytes staged in LDS, decoded between the MFMAs):
+    symmetric and with zero points, group sizes of 32 to 128, one to three row tiles per wave and the 256-row
+    blocks taken past 384 tokens, K whole, in two halves and in three parts."""
+    from neuropress_amd import kernels
+
+    tile_wide(2, splits)
+    Q = cases.q4_layer(800 + m + nbits, n, k, nbits=nbits, gs=gs, act=act, m=m, asym=asym, bias=True)
+    zp = None if Q["zp"] is None else Q["zp"].to(gpu)
+    args = (Q["x"].to(gpu), Q["blob"].to(gpu), Q["scale"].to(gpu), nbits, gs, zp, Q["bias"].to(gpu))
+    y = kernels.q_gemm_tile(*args)
+    _check(y, _q_ref(oracle_lib, Q, act))
+    assert torch.equal(y, kernels.q_gemm_tile(*args)), "the result depends on which half of K finished first"
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("nbits,asym,gs", [(4, False, 32), (4, True, 128), (8, False, 32), (8, True, 32)])
+def test_wide_tile_gemm_group_affine_decodes_bit_exactly(gpu, tile_wide, act, nbits, asym, gs):
+    """One-hot activations through the 128-column kernel return the one-pass decode exactly."""
+    from neuropress_amd import kernels
+
+    n, k = 200, 1024
+    Q = cases.q4_layer(63, n, k, nbits=nbits, gs=gs, act=act, m=1, asym=asym)
+    blob, sc = Q["blob"].to(gpu), Q["scale"].to(gpu)
+    zp = None if Q["zp"] is None else Q["zp"].to(gpu)
+    wt = kernels.q_dequant(blob, sc, nbits, gs, zp, act).t().contiguous()
+    eye = torch.eye(k, dtype=act, device=gpu)
+    for splits in (1, 2, 4):
+        tile_wide(2, splits)
+        assert torch.equal(kernels.q_gemm_tile(eye, blob, sc, nbits, gs, zp), wt), f"1024 tokens, {splits} splits"
+        assert torch.equal(kernels.q_gemm_tile(eye[100:330], blob, sc, nbits, gs, zp), wt[100:330]), f"230 tokens, {splits} splits"
