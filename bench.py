@@ -102,6 +102,28 @@ def time_graph(fn, n_rot, steps, warmup, dev, replays=5, flush=None):
     return sorted(times)[len(times) // 2]
 
 
+def host_cpu_description():
+    """Model string of the host CPU with what /proc/cpuinfo adds to it (family / model / stepping, logical CPUs,
+    sockets): the name alone can be as short as "AMD EPYC" on virtualised hosts."""
+    fields, logical, sockets = {}, 0, set()
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for ln in fh:
+                key, _, val = ln.partition(":")
+                key, val = key.strip(), val.strip()
+                if key == "processor":
+                    logical += 1
+                elif key == "physical id":
+                    sockets.add(val)
+                elif key in ("model name", "cpu family", "model", "stepping", "vendor_id") and key not in fields:
+                    fields[key] = val
+    except OSError:
+        return ""
+    name = fields.get("model name", fields.get("vendor_id", "unknown"))
+    return (f"{name} (family {fields.get('cpu family', '?')} model {fields.get('model', '?')} stepping "
+            f"{fields.get('stepping', '?')}; {logical} logical CPUs visible, {max(len(sockets), 1)} socket(s))")
+
+
 def rot_for(bytes_per_buffer, cap=512):
     """Buffers in a rotating pool: enough for POOL_BYTES, at most `cap` (small layers)."""
     return max(2, min(cap, -(-POOL_BYTES // max(int(bytes_per_buffer), 1))))
@@ -361,6 +383,15 @@ def main():
     del layer
     torch.cuda.empty_cache()
 
+    # The most any kernel could show on this shape, measured in this run: a plain read (one 16-byte load per
+    # lane, nothing else) of as many bytes as the reference's format holds, launch included.
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    read16 = alg // 16 * 16
+    assert read16 <= sl0.total_bytes
+    floor_us = time_graph(lambda i: _lib.call("npamd_diag_stream_read", spool[i].blob.data_ptr(), read16, sink.data_ptr(),
+                                              torch.cuda.current_stream(dev).cuda_stream),
+                          s_rot, s_rot, 3, dev, flush=flush)
+
     result = {
         "metric": METRIC,
         "value": round(gbs, 2),
@@ -388,20 +419,22 @@ def main():
         "eager_us_per_call": {"kernels.vq_linear_sliced": {"host_issue": round(host_us, 2), "wall": round(wall_us, 2)},
                               "NPVQLinear.forward": {"host_issue": round(host_us_module, 2), "wall": round(wall_us_module, 2)},
                               "graph_replay": round(us, 3), "module_has_slice_lists": has_lists},
-        "roofline": {
-            "bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": TRAFFIC["sliced_m1"]["bytes"], "traffic_source": TRAFFIC["sliced_m1"]["source"],
-            "kernel": "sliced_gemv_kernel<bf16, M=1>", "algorithmic_bytes_per_launch": alg,
-            "avg_launch_us": round(us, 3),
-            "streamed_bytes_per_launch": int(sl0.total_bytes + sl0.n_workgroups * sl0.slice_rows * 16 + k * 2 + n * 2),
-            "note": "one launch per call: achieved = bytes of the reference's format (16-bit index stream + codebook "
-                    "+ x + y) / launch duration; streamed_bytes_per_launch is what this kernel's own format moves "
-                    "(slice lists + one codebook slice per workgroup, the latter from L2)",
-        },
         "footprint": footprint,
-        "checks": {"decode_bit_exact": decode_exact, "output_within_1e-2": ok, "max_abs_err": max_abs},
     }
+    # `roofline`, `roofline_m384`, `cpu_baseline` and `checks` are appended last, behind the long `sweep` and
+    # `cpu_baselines` lists, so that a reader who keeps only the end of the line still has them.
+    roofline = {
+        "bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(gbs / HBM_PEAK_GBS, 4),
+        "traffic": TRAFFIC["sliced_m1"]["bytes"], "traffic_source": TRAFFIC["sliced_m1"]["source"],
+        "kernel": "sliced_gemv_kernel<bf16, M=1>", "algorithmic_bytes_per_launch": alg,
+        "avg_launch_us": round(us, 3),
+        # plain read of the same bytes in this run (launch included): what a kernel that only read them would take
+        "floor_us": round(floor_us, 3), "frac_at_floor": round(alg / floor_us / 1e3 / HBM_PEAK_GBS, 4),
+        "streamed_bytes_per_launch": int(sl0.total_bytes + sl0.n_workgroups * sl0.slice_rows * 16 + k * 2 + n * 2),
+        "note": "achieved = bytes of the reference's format (index stream + codebook + x + y) / launch duration",
+    }
+    checks = {"decode_bit_exact": decode_exact, "output_within_1e-2": ok, "max_abs_err": max_abs}
 
     # The second half of the metric: the tile-decode GEMM at M = 384 on the same layer, priced against the
     # dense bf16 MFMA peak.  Timed here so that the line carries it with --no-sweep too.
@@ -411,14 +444,22 @@ def main():
     flops2 = 2.0 * m2 * n * k
     y2 = kernels.vq_gemm_tile(xm2[0], c3["pool"][0], c3["d_cb_act"], 16, n, None)
     ok2, max_abs2 = check_against_cpu(y2, (xm2[0].float() @ w_gpu.float().T).cpu())
-    result["roofline_m384"] = {
+    # The matrix pipes alone, in this run: the same number of MFMA 32x32x16 spread over every compute unit,
+    # random finite operands, nothing else in the kernel.
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    per_wave = -(-int(flops2 / (2 * 32 * 32 * 16)) // (cus * 4))
+    ops = torch.randn(7 * 64 * 8, generator=gen(9)).to(torch.bfloat16).to(dev)
+    us_mfma = time_graph(lambda i: _lib.call("npamd_diag_mfma", ops.data_ptr(), cus, per_wave, _lib.BF16, sink.data_ptr(),
+                                             torch.cuda.current_stream(dev).cuda_stream), 1, 20, 3, dev)
+    roofline_m384 = {
         "bound": "mfma", "achieved": round(flops2 / us_tile / 1e6, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(flops2 / us_tile / 1e6 / MFMA_PEAK_TFLOPS, 4),
         "traffic": TRAFFIC["tile_m384"]["bytes"], "traffic_source": TRAFFIC["tile_m384"]["source"],
-        "kernel": "tile_gemm_kernel<bf16, VqProvider<bf16,16>, MW=3>", "flops_per_launch": flops2,
+        "kernel": "tile2_gemm_kernel<bf16, MW=3, VQ 16-bit> (128 columns, K in two halves)", "flops_per_launch": flops2,
         "avg_launch_us": round(us_tile, 3), "M": m2, "output_within_1e-2": ok2, "max_abs_err": max_abs2,
-        "note": "same layer and codebook as `roofline`, 384 tokens, one launch decodes every weight once and "
-                "contracts it with MFMA 32x32x16; HIP-graph replay over the rotating index pool",
+        # the same flops as MFMAs only, on all compute units, in this run
+        "floor_us": round(us_mfma, 3), "frac_at_floor": round(flops2 / us_mfma / 1e6 / MFMA_PEAK_TFLOPS, 4),
+        "note": "same layer as `roofline`, 384 tokens; one call (a counter fill + the GEMM) decodes every weight once",
     }
     x384_cpu = xm2[0].cpu()
     del xm2, y2
@@ -589,12 +630,16 @@ def main():
             blobs = [blob.to(dev)]
             blobs += [blobs[0].clone() for _ in range(rot - 1)]
             w32 = kernels.q_dequant(blobs[0], sc, 4, 32, None, torch.float16).float()
-            for m in (1, 16, 32, 256):
+            for m in (1, 16, 32, 256) + ((384, 512) if nn_ == 14336 else ()):
                 xm = xpair(m, kk, 90 + m, torch.float16)
                 algq = nn_ * kk // 2 + nn_ * kk // 32 * 2 + m * kk * 2 + m * nn_ * 2
                 run(f"cfg5 int4 {nn_}x{kk} f16", "a:gemv" if m <= 32 else "b:tile-gemm", m,
                     lambda i: kernels.q_linear(xm[i % 2], blobs[i], sc, 4, 32), rot, algq, 2.0 * m * nn_ * kk,
                     ref=lambda: xm[0].float() @ w32.T)
+                if m >= 256:
+                    run(f"cfg5 int4 {nn_}x{kk} f16", "c:decode+gemm", m, lambda i: torch.nn.functional.linear(
+                        xm[i % 2], kernels.q_dequant(blobs[i], sc, 4, 32, None, torch.float16)), rot, algq,
+                        2.0 * m * nn_ * kk, ref=lambda: xm[0].float() @ w32.T)
             if nn_ == 14336:
                 q5 = {"blob": blob, "scale": sc.cpu(), "x": xpair(1, kk, 91, torch.float16)[0].cpu(), "n": nn_, "k": kk,
                       "y": kernels.q_linear(xpair(1, kk, 91, torch.float16)[0], blobs[0], sc, 4, 32).cpu()}
@@ -629,15 +674,7 @@ def main():
 
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
         torch.set_num_threads(cores)
-        cpu_model = ""
-        try:
-            with open("/proc/cpuinfo") as fh:
-                for ln in fh:
-                    if ln.startswith("model name"):
-                        cpu_model = ln.split(":", 1)[1].strip()
-                        break
-        except OSError:
-            pass
+        cpu_model = host_cpu_description()
 
         def median_ms(fn):
             """(median seconds, last result): 1-2 warm-up calls, then 5 timed (fewer when one call is slow)."""
@@ -682,15 +719,18 @@ def main():
                     lambda: torch_path.q_decode_cpu(q5["blob"], q5["scale"], 4, 32, torch.float16),
                     q5["x"], q5["n"] * q5["k"] // 2 + q5["n"] * q5["k"] // 32 * 2 + q5["k"] * 2 + q5["n"] * 2, q5["y"]))
         head = cpu_rows[0]
+        result["cpu_baselines"] = cpu_rows
         result["cpu_baseline"] = {
             "value": head["value"], "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "the full config-3 up/gate layer at M=1: median of 5 timed calls each of the decode "
-                      "(vectorised 16-bit view + codebook gather + cast to bf16) and of torch F.linear in bf16",
+            "sample": "the full config-3 up/gate layer at M=1: median of 5 calls each of the decode (16-bit view + "
+                      "codebook gather + cast to bf16) and of torch F.linear in bf16",
             "ms_per_call": head["ms_per_call"], "decode_ms": head["decode_ms"], "matmul_ms": head["matmul_ms"],
             "cpu": cpu_model,
             "gpu_matches_cpu_within_1e-2": head["gpu_matches_cpu_within_1e-2"], "max_abs_diff": head["max_abs_diff"],
         }
-        result["cpu_baselines"] = cpu_rows
+    result["roofline"] = roofline
+    result["roofline_m384"] = roofline_m384
+    result["checks"] = checks
     print(json.dumps(result))
 
 

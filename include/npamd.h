@@ -382,27 +382,6 @@ int npamd_q_embedding(const int64_t* ids, int64_t n_ids, const uint8_t* w_pack,
                       int64_t vocab, int dim, int64_t padding_idx, float embed_scale,
                       void* out, int out_dtype, void* stream);
 
-/* ------------------------------------------------------ diagnostics ---- */
-/*
- * Memory-system ceilings for the access patterns of the kernels above (no
- * counterpart in the reference; used by the benchmark to state what bounds the
- * decode kernels).  Results are discarded; `sink16` is a 16-byte device buffer.
- *
- * npamd_diag_stream_read: read `n_bytes` (multiple of 16) once.
- * npamd_diag_gather: stream `n_indices` uint16 indices (multiple of 8) and fetch
- *   one 16-byte row of `table16` per index (index masked to `table_entries`, a
- *   power of two), from global memory or, with from_lds != 0, from an LDS copy
- *   of the table (at most 8192 rows).
- *
- * npamd_diag_reload_tuning: the NPAMD_* tuning environment variables are read once, at the first
- *   launch; this reads them again.  For tests and tuning runs only: it must not run while
- *   another thread launches.
- */
-void npamd_diag_reload_tuning(void);
-int npamd_diag_stream_read(const void* src, int64_t n_bytes, void* sink16, void* stream);
-int npamd_diag_gather(const void* idx_u16, int64_t n_indices, const void* table16,
-                      int table_entries, int from_lds, void* sink16, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -61,6 +61,7 @@ SIGNATURES: dict[str, list] = {
     "npamd_diag_reload_tuning": [],
     "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
     "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],
+    "npamd_diag_mfma": [_vp, _int, _int, _int, _vp, _vp],
 }
 
 _RESTYPES = {"npamd_vq_sliced_workspace_bytes": _i64, "npamd_gemm_tile_workspace_bytes": _i64,

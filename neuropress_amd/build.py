@@ -40,7 +40,7 @@ def sources() -> list[Path]:
 
 
 def _headers_mtime() -> float:
-    hdrs = list(CSRC.glob("*.hpp")) + [PKG_DIR.parent / "include" / "npamd.h"]
+    hdrs = list(CSRC.glob("*.hpp")) + list((PKG_DIR.parent / "include").glob("*.h"))
     return max(h.stat().st_mtime for h in hdrs)
 
 

@@ -4,6 +4,7 @@
 
 #include <stdlib.h>
 
+#include "../../include/npamd_diag.h"
 #include "gemm_tile2.hpp"
 #include "gemv.hpp"
 

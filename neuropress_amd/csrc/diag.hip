@@ -6,6 +6,7 @@
 //                   table row per index from global memory or from an LDS copy
 //                   of the table; results are xor-folded and never stored
 #include "common.hpp"
+#include "../../include/npamd_diag.h"
 
 namespace npamd {
 
@@ -59,9 +60,47 @@ diag_gather_lds_kernel(const u32x4* __restrict__ idx, const u32x4* __restrict__ 
   if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) sink[0] = acc;
 }
 
+// The matrix pipes alone: twelve independent accumulator tiles per wave, one wave per SIMD.
+template <int ACT>
+__global__ void __launch_bounds__(256)
+diag_mfma_kernel(const u32x4* __restrict__ operands, float* __restrict__ sink, int rounds) {
+  u32x4 a[3], b[4];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) a[i] = operands[(threadIdx.x & 63) + 64 * i];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b[i] = operands[(threadIdx.x & 63) + 64 * (3 + i)];
+  f32x16 acc[12];
+#pragma unroll
+  for (int i = 0; i < 12; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+  for (int r = 0; r < rounds; ++r) {
+#pragma unroll
+    for (int i = 0; i < 12; ++i) acc[i] = mfma32<ACT>(a[i % 3], b[i / 3], acc[i]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 12; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  if (s == 12345.678f) sink[0] = s;  // never true in practice
+}
+
 }  // namespace npamd
 
 using namespace npamd;
+
+extern "C" int npamd_diag_mfma(const void* operands, int blocks, int mfmas_per_wave, int act_dtype, void* sink16,
+                               void* stream) {
+  NPAMD_REQUIRE(operands && sink16 && blocks >= 1 && mfmas_per_wave >= 1, "npamd_diag_mfma: bad arguments");
+  NPAMD_REQUIRE(act_dtype == NPAMD_F16 || act_dtype == NPAMD_BF16, "npamd_diag_mfma: f16 or bf16");
+  const int rounds = (mfmas_per_wave + 11) / 12;
+  if (act_dtype == NPAMD_BF16)
+    diag_mfma_kernel<NPAMD_BF16><<<blocks, 256, 0, (hipStream_t)stream>>>((const u32x4*)operands, (float*)sink16, rounds);
+  else
+    diag_mfma_kernel<NPAMD_F16><<<blocks, 256, 0, (hipStream_t)stream>>>((const u32x4*)operands, (float*)sink16, rounds);
+  return check_launch("npamd_diag_mfma");
+}
 
 extern "C" int npamd_diag_stream_read(const void* src, int64_t n_bytes, void* sink16, void* stream) {
   NPAMD_REQUIRE(src && sink16 && n_bytes >= 16 && n_bytes % 16 == 0,

@@ -111,6 +111,13 @@ _TILE_MAX_TOKENS: int = _env_int(
     ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 256
 )
 
+# Layers whose codebook LDS does not hold (more than 4096 rows of eight) and that have at least
+# _TILE_WIDE_MIN_FEATURES output or input features run the 128-column tile GEMM, which stays ahead
+# of decode + GEMM up to its 384-row block: 14336 x 4096 75-77 us at 384 tokens against 102 us,
+# 4096 x 14336 78-82 us against 117 us (the 64-column kernel: 84-97 us).
+_TILE_WIDE_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_TILE_WIDE_MAX_TOKENS",), 384)
+_TILE_WIDE_MIN_FEATURES: int = 8192
+
 # The tile GEMM gives each workgroup 64 output columns (and up to 384 rows).  When
 # that grid covers less than this fraction of the compute units the kernel splits
 # the reduction over up to 16 workgroups per tile (at least 512 input features
@@ -604,7 +611,7 @@ class NPVQLinear(nn.Module):
             if m > self._gemv_max_tokens(m):
                 if (
                     self.backend != VQBackend.CUDA_LUT
-                    and m <= _TILE_MAX_TOKENS
+                    and m <= self._tile_max_tokens()
                     and self._tile_band_ok(x, m)
                 ):
                     return self._forward_tile_gemm(x)
@@ -822,6 +829,18 @@ class NPVQLinear(nn.Module):
             ok = kernels.vq_fused_supported(self.in_features, self.vector_len, bits)
             self._derived["mfma_layer"] = ok
         return ok
+
+    def _tile_max_tokens(self) -> int:
+        """Upper end of the tile-decode GEMM band for this layer."""
+        if (
+            _TILE_MAX_TOKENS > 0
+            and not self.is_residual
+            and self.vector_len == 8
+            and self.proxy.num_centroids * self.vector_len * 2 > 65536
+            and max(self.in_features, self.out_features) >= _TILE_WIDE_MIN_FEATURES
+        ):
+            return max(_TILE_MAX_TOKENS, _TILE_WIDE_MAX_TOKENS)
+        return _TILE_MAX_TOKENS
 
     def _tile_band_ok(self, x: torch.Tensor, m: int) -> bool:
         """True when the tile GEMM's grid (64 columns x up to 384 rows per workgroup,

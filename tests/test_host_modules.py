@@ -339,13 +339,18 @@ def test_warn_kernel_fallback_once_per_kernel(caplog):
 
 
 def test_library_exports_every_declared_symbol():
-    """Every function include/npamd.h declares is exported by the built library and
-    bound by the ctypes layer (no compute calls: there is no GPU here)."""
+    """Every function include/npamd.h (the drop-in contract) and include/npamd_diag.h (measurement
+    aids) declare is exported by the built library and bound by the ctypes layer (no compute calls:
+    there is no GPU here)."""
     from neuropress_amd import _lib
 
     header = (ROOT / "include" / "npamd.h").read_text()
     declared = set(re.findall(r"\b(npamd_[a-z0-9_]+)\s*\(", header))
     assert {"npamd_vq_gemv", "npamd_vq_gemm_tile", "npamd_vq_dequant", "npamd_q_gemv"} <= declared
+    assert not any(name.startswith("npamd_diag_") for name in declared), "measurement aids belong in npamd_diag.h"
+    diag = set(re.findall(r"\b(npamd_diag_[a-z0-9_]+)\s*\(", (ROOT / "include" / "npamd_diag.h").read_text()))
+    assert {"npamd_diag_reload_tuning", "npamd_diag_stream_read", "npamd_diag_mfma"} <= diag
+    declared |= diag
     lib = ctypes.CDLL(str(_lib.LIB_PATH))
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in npamd.h but not exported"
