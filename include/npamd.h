@@ -103,13 +103,13 @@ int npamd_vq_gemv_perm_supported(int M, int N, int K, int nc, int vl, int bits);
  * Host-only arithmetic. */
 int npamd_vq_fused_supported(int K, int vl, int bits);
 
-/* 1 when a fused GEMV call (npamd_vq_gemv, npamd_rvq_gemv, npamd_q_gemv) of M tokens on an N x K
- * layer runs the kernel that stages every step's activations through LDS (one 16-row tile per
- * workgroup, three tokens or more, the operands not looked up in an LDS copy of the codebook:
- * table_in_lds = 0): such a call stays ahead of the tile GEMM up to the GEMV's 32 tokens whatever
- * K is, which is what the callers' band thresholds ask (the reference fixes its own thresholds per
- * backend, neuropress/nn/np_vq_linear.py:73-98).  Host-only arithmetic. */
-int npamd_gemv_stages_activations(int M, int N, int K, int table_in_lds);
+/* 1 when a fused GEMV call of M tokens on an N x K layer runs the kernel that stages every step's
+ * activations through LDS: npamd_vq_gemv on a layer with a codebook of `nc` rows of eight (nc > 0),
+ * or npamd_q_gemv (nc = 0).  Such a call stays ahead of the tile GEMM up to the GEMV's 32 tokens
+ * whatever K is, which is what the callers' band thresholds ask (the reference fixes its own
+ * thresholds per backend, neuropress/nn/np_vq_linear.py:73-98).  The answer is the launcher's own:
+ * it is run up to the point of the launch.  Host-only arithmetic. */
+int npamd_gemv_stages_activations(int M, int N, int K, int nc);
 
 /*
  * Tile-decode MFMA GEMM, any M >= 1: same contraction, weight tiles decoded
@@ -217,8 +217,12 @@ int64_t npamd_vq_sliced_workspace_bytes(const npamd_sliced_header* header_host, 
  * 2^16 rows) every lane adds its partial sum, as a fixed-point number in units of
  * 2^-24, to a 64-bit word of the workspace with one atomic; the lane that completes
  * a row's count adds the bias, rounds once and stores y -- one kernel, and the sum
- * does not depend on the order of arrival (partial sums of magnitude 2^15 or more go
- * through a float accumulator).  Otherwise the partial sums are written out and a
+ * does not depend on the order of arrival.  The rounding of the partial sums adds an absolute
+ * error of at most n_partials * 2^-25 (n_partials from the header: 4.8e-7 at 16) to the float32
+ * sum, whatever the magnitude of y: outputs far below 1e-4 lose relative precision against a
+ * float32 accumulation.  Partial sums of magnitude 2^15 or more, NaN and infinities go through a
+ * float accumulator with a float atomic: a row with two or more of those may differ in its last
+ * bits from run to run.  Otherwise the partial sums are written out and a
  * second kernel adds them in a fixed order.
  * `column_perm`: NULL, or K int32 column numbers (16-byte aligned, each < ldx):
  * the kernel then reads x[m, column_perm[k]] wherever it would read x[m, k],

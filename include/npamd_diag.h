@@ -28,11 +28,16 @@ extern "C" {
  *   on operands read from `operands` (7 KiB of device memory, any finite values) and nothing
  *   else: the time the matrix pipes alone need for that many flops.
  *
+ * npamd_diag_last_gemv_staged: 1 / 0 when the calling thread's last fused GEMV launch (npamd_vq_gemv,
+ *   npamd_q_gemv and their variants) was / was not of a kernel that stages activations in LDS, -1
+ *   before the first; npamd_gemv_stages_activations (npamd.h) must predict it.
+ *
  * npamd_diag_reload_tuning: the NPAMD_* tuning environment variables are read once, at the first
  *   launch; this reads them again.  For tests and tuning runs only: it must not run while
  *   another thread launches.
  */
 void npamd_diag_reload_tuning(void);
+int npamd_diag_last_gemv_staged(void);
 int npamd_diag_stream_read(const void* src, int64_t n_bytes, void* sink16, void* stream);
 int npamd_diag_gather(const void* idx_u16, int64_t n_indices, const void* table16,
                       int table_entries, int from_lds, void* sink16, void* stream);

@@ -59,6 +59,7 @@ SIGNATURES: dict[str, list] = {
     "npamd_q_embedding": [_vp, _i64, _vp, _vp, _vp, _int, _int, _i64, _int, _i64, ctypes.c_float, _vp, _int, _vp],
     "npamd_q_gemm_tile": _Q_LINEAR[:-1] + _WS + [_vp],
     "npamd_diag_reload_tuning": [],
+    "npamd_diag_last_gemv_staged": [],
     "npamd_diag_stream_read": [_vp, _i64, _vp, _vp],
     "npamd_diag_gather": [_vp, _i64, _vp, _int, _int, _vp, _vp],
     "npamd_diag_mfma": [_vp, _int, _int, _int, _vp, _vp],

@@ -96,6 +96,11 @@ bool gemv_lds_activations_forced() { return tuning().gemv_lds_x != 0; }
 // 20.5 / 16.2 at 8, 27.5 / 18.9 at 16, 38.7 / 25.4 at 32; 65536-row codebook 4096 x 14336 35.8 / 34.6
 // at 4, 37.8 / 35.4 at 8, 42.4 / 37.6 at 16, 52 / 41 at 32.  With more row tiles per block
 // (14336 x 4096) or the table in LDS it does not pay.
+int& last_gemv_staged() {
+  static thread_local int staged = -1;
+  return staged;
+}
+
 bool gemv_stage_activations(int M) {
   const int mode = tuning().gemv_xstage;
   return mode >= 2 || (mode == 1 && M >= 3);
@@ -219,11 +224,12 @@ int plan_tile_mw(int M) {
 
 extern "C" int npamd_version(void) { return 3; }
 
-extern "C" int npamd_gemv_stages_activations(int M, int N, int K, int table_in_lds) {
-  if (M < 1 || M > NPAMD_GEMV_MAX_M || N < 1 || K < 64 || K % 64 || table_in_lds) return 0;
-  if (!npamd::gemv_stage_activations(M) || npamd::plan_gemv_parts(M, N, K / 64, 0) != 1) return 0;
-  return npamd::plan_gemv(N, K / 64, 4, M > 16 ? 8 : 16).R == 1 ? 1 : 0;
+extern "C" int npamd_gemv_stages_activations(int M, int N, int K, int nc) {
+  if (M < 1 || M > NPAMD_GEMV_MAX_M || N < 1 || K < 64 || K % 64 || nc < 0) return 0;
+  return nc ? npamd::vq_gemv_plan_stages(M, N, K, nc) : npamd::q_gemv_plan_stages(M, N, K);
 }
+
+extern "C" int npamd_diag_last_gemv_staged(void) { return npamd::last_gemv_staged(); }
 
 extern "C" void npamd_diag_reload_tuning(void) { npamd::tuning_table() = npamd::read_tuning(); }
 

@@ -37,6 +37,9 @@ struct GemvShape {
   // Only with the X_LDS variant (every block first copies the permuted rows of x into LDS).
   const int32_t* perm = nullptr;
   int stage_offset = 0;  // XS kernels: byte offset of the waves' activation staging areas in LDS
+  // Planning only: when set, the launcher writes here whether the kernel it chose stages its
+  // activations (1 / 0) and launches nothing.
+  int* plan_only = nullptr;
 };
 
 // Largest M * K (elements) whose activations the GEMV stages in LDS (32 KiB; the unpermuted
@@ -320,6 +323,13 @@ constexpr int kGemvLdsPerBlockMax = 160 * 1024;
 // Whether a one-row-tile launch of M tokens stages its activations (XS kernels): from three tokens
 // (NPAMD_GEMV_XSTAGE: 0 never, 2 at every token count).
 bool gemv_stage_activations(int M);
+// Whether this thread's last fused GEMV launch was of a kernel that stages its activations (-1:
+// none yet).  Tests compare it with what npamd_gemv_stages_activations answers for the same shape.
+int& last_gemv_staged();
+// The launcher's own answer, without a launch, for a plain VQ layer with a codebook of `nc` rows of
+// eight (vq_gemv.hip) and for a group-quantized layer (q4.hip).
+int vq_gemv_plan_stages(int M, int N, int K, int nc);
+int q_gemv_plan_stages(int M, int N, int K);
 bool gemv_lds_codebook_enabled();  // NPAMD_GEMV_LDS_CB=0 switches the LDS copy off (tuning aid)
 bool gemv_lds_activations_forced();  // NPAMD_GEMV_LDS_X=1: stage x in LDS also without a permutation (tuning aid)
 
@@ -341,6 +351,10 @@ int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const
     if (lds > kGemvLdsPerBlockMax)  // no room for the staging areas: the same kernel without them
       return launch_fused_gemv_r<ACT, Provider, R, CB_LDS, X_LDS, MT, H, false>(s, pargs, plan, cb_bytes, st, what);
   }
+  if (s.plan_only) {
+    *s.plan_only = XS ? 1 : 0;
+    return 0;
+  }
   if (lds > 64 * 1024) {
     static LdsLatch latch;  // per instantiation
     const hipError_t e = enable_dynamic_lds(
@@ -348,6 +362,7 @@ int launch_fused_gemv_r(GemvShape s, const typename Provider::Args& pargs, const
     if (e != hipSuccess)
       return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
   }
+  last_gemv_staged() = XS ? 1 : 0;
   fused_gemv_kernel<ACT, Provider, R, CB_LDS, X_LDS, MT, H, XS><<<blocks, plan.waves * 64, lds, st>>>(s, pargs);
   return check_launch(what);
 }

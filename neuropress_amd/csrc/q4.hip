@@ -633,6 +633,16 @@ static int q4_fused(const QCall& c, bool gemv) {
   return launch_tile_gemm<ACT, P>(s, a, c.st, c.what, c.ws, c.ws_bytes);
 }
 
+int npamd::q_gemv_plan_stages(int M, int N, int K) {
+  int staged = 0;
+  GemvShape s{nullptr, K, nullptr, nullptr, N, M, N, K / 64, 0, 0};
+  s.plan_only = &staged;
+  using P = Q4Provider<NPAMD_F16, false>;  // int4 / int8, with or without zero points: one plan
+  typename P::Args a{};
+  launch_fused_gemv<NPAMD_F16, P>(s, a, nullptr, "plan");
+  return staged;
+}
+
 template <int ACT, bool ASYM>
 static int q8_fused(const QCall& c, bool gemv) {
   using P = Q8Provider<ACT, ASYM>;

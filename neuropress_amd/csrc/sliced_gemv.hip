@@ -5,10 +5,20 @@
 // and a zero row in LDS.  Every lane owns one output row and
 // walks the entries filed under (slice, group range, row): two 16-byte LDS reads
 // (codebook row, activation vector) and four packed dot products per entry, the
-// sum kept in registers.  Each lane then writes one float into the partial-sum
-// vector of its (slice, group range); a second kernel adds the partial vectors
-// of a row in a fixed order, adds the bias and rounds once.  No atomics: the
-// result does not depend on timing.
+// sum kept in registers.
+//
+// Finish.  A row's result is spread over the workgroups that hold the slices its indices
+// point into (n_partials of them).  With fewer than 256 per row -- every codebook of up to
+// 2^16 rows -- each lane rounds its partial sum to a multiple of 2^-24 and adds it, with one
+// 64-bit integer atomic, to the row's word of the workspace, which also counts the arrivals;
+// the lane that completes the count converts the total, adds the bias, rounds once to the
+// activation dtype, stores y and zeroes the word.  Integer addition commutes, so the result
+// does not depend on the order of arrival; it differs from the exact sum by at most
+// n_partials * 2^-25 plus the final roundings, whatever the magnitude of y.  Partial sums of
+// magnitude 2^15 or more (and NaN / infinity) do not fit the word: they are added to a float
+// accumulator with a float atomic instead, and only then -- two or more such partial sums in
+// one row -- can the last bits depend on the order of arrival.  With 256 partial vectors or
+// more every lane writes its partial sum out and a second kernel adds them in a fixed order.
 #include <stdlib.h>
 
 #include <mutex>
@@ -86,10 +96,13 @@ constexpr bool straight_tokens(int m) { return m <= 2 || m >= 6; }
 constexpr int kMaxTokens = 7;  // tokens per pass over the entries (an eighth token's activations would not fit in LDS)
 constexpr int kLdsX = 0;       // [token][group] vectors: a token's 512 vectors are contiguous, so the
                                // lanes of a read spread over all sixteen 16-byte bank groups
-constexpr int kLdsSlice = kSlicedMaxGroups * 16 * kMaxTokens;
-constexpr int kLdsStage = kLdsSlice + (kSlicedMaxSliceRows + 1) * 16;  // [token][row of the block] sums, fused finish
-constexpr int kLdsBytes = kLdsStage + kMaxTokens * kSlicedTasks * 4;
-static_assert(kLdsBytes <= kSlicedLdsBytes && kLdsSlice < 65536, "LDS map");
+// The map is sized by the launch's token count M (76 KiB at one token).  Two workgroups per compute
+// unit -- 512 workgroups of 448 rows, 64 registers per lane -- were measured at one token and lose:
+// 12.8 against 11.4 us (more slice copies, waves without a strip, and 10.9 us with 71 registers).
+constexpr int lds_slice(int m) { return kSlicedMaxGroups * 16 * m; }
+constexpr int lds_stage(int m) { return lds_slice(m) + (kSlicedMaxSliceRows + 1) * 16; }  // [token][row of the block] sums, fused finish
+constexpr int lds_bytes(int m) { return lds_stage(m) + m * kSlicedTasks * 4; }
+static_assert(lds_bytes(kMaxTokens) <= kSlicedLdsBytes && lds_slice(kMaxTokens) < 65536, "LDS map");
 // The first eight waves copy the slice into LDS.
 constexpr int kLoaderThreads = kSlicedTasks / 2;
 constexpr int kSliceLoads = kSlicedMaxSliceRows / kLoaderThreads;
@@ -133,7 +146,7 @@ __device__ __forceinline__ void run_quad(const QuadAddr& ad, const uint8_t* lds,
     u32x4 c[kBatch], xv[kBatch][M];
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {
-      c[j] = *reinterpret_cast<const u32x4*>(lds + kLdsSlice + ad.row[j0 + j]);
+      c[j] = *reinterpret_cast<const u32x4*>(lds + lds_slice(M) + ad.row[j0 + j]);
       const uint8_t* xg = lds + kLdsX + ad.grp[j0 + j];
 #pragma unroll
       for (int m = 0; m < M; ++m) xv[j][m] = *reinterpret_cast<const u32x4*>(xg + m * (kSlicedMaxGroups * 16));
@@ -199,7 +212,7 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int D = kDepth;
   u32x4* xl = reinterpret_cast<u32x4*>(lds + kLdsX);
-  u32x4* cb = reinterpret_cast<u32x4*>(lds + kLdsSlice);
+  u32x4* cb = reinterpret_cast<u32x4*>(lds + lds_slice(M));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -333,7 +346,7 @@ __global__ void __launch_bounds__(kSlicedTasks, 1) sliced_gemv_kernel(SlicedArgs
     // The lanes of a wave work for rows scattered over the workgroup's block (strips are sorted
     // by length); the sums change hands through LDS so that thread t finishes row row_begin + t
     // and a wave's atomics, bias reads and stores fall on consecutive addresses.
-    float* stage = reinterpret_cast<float*>(lds + kLdsStage);
+    float* stage = reinterpret_cast<float*>(lds + lds_stage(M));
     if (row != kSlicedNoRow) {
 #pragma unroll
       for (int m = 0; m < M; ++m) stage[m * kSlicedTasks + (row - row_begin)] = acc[m][0] + acc[m][1];
@@ -384,6 +397,7 @@ __global__ void __launch_bounds__(256) sliced_reduce_kernel(float* __restrict__ 
 template <int ACT, int M, bool PERM>
 int launch_sliced_tokens_p(const SlicedArgs& a, int n_workgroups, hipStream_t st, const char* what) {
   static LdsLatch latch;  // per instantiation
+  constexpr int kLdsBytes = lds_bytes(M);
   const hipError_t e = enable_dynamic_lds(latch, reinterpret_cast<const void*>(&sliced_gemv_kernel<ACT, M, PERM>), kLdsBytes);
   if (e != hipSuccess)
     return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, kLdsBytes, hipGetErrorString(e));

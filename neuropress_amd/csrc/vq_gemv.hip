@@ -19,6 +19,20 @@ int run_vq(const VqCall& c, const GemvShape& s) {
   return launch_fused_gemv<ACT, P>(s, a, c.st, c.what, (VL == 8 ? c.nc * 16 : (c.nc % 2 == 0 ? c.nc * 8 : 0)));
 }
 
+}  // namespace
+
+int npamd::vq_gemv_plan_stages(int M, int N, int K, int nc) {
+  int staged = 0;
+  GemvShape s{nullptr, K, nullptr, nullptr, N, M, N, K / 64, 0, 0};
+  s.plan_only = &staged;
+  using P = VqProvider<NPAMD_F16, 16, false, 8>;  // the choice depends on the table's size, not on the index width
+  typename P::Args a{};
+  launch_fused_gemv<NPAMD_F16, P>(s, a, nullptr, "plan", nc * 16);
+  return staged;
+}
+
+namespace {
+
 template <int ACT, int VL>
 int run_vq_bits_vl(const VqCall& c, const GemvShape& s) {
   switch (c.bits) {

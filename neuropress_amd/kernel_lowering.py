@@ -252,9 +252,11 @@ def prepare_decode(model: nn.Module) -> int:
     lists exist afterwards.
 
     ``forward`` never does this work: a layer that was not prepared runs its slower decode
-    kernel (and says so once).  ``AutoKernelLowering.apply`` calls this function when the model
-    is already on a GPU; call it yourself after moving a lowered model there, after
-    ``load_state_dict``, and before capturing a HIP graph.  No counterpart in the reference.
+    kernel (and says so once).  A lowered module does it by itself when ``.to()`` / ``.cuda()`` /
+    ``load_state_dict()`` leave it on a GPU (``NEUROPRESS_VQ_PREPARE_ON_MOVE=0`` switches that
+    off), and ``AutoKernelLowering.apply`` calls this function when the model is already there;
+    it remains the explicit form -- for buffers replaced by hand, and in front of a HIP-graph
+    capture.  No counterpart in the reference.
     """
     from .nn.np_linear import NPLinear
     from .nn.np_vq_linear import NPVQLinear

@@ -251,11 +251,12 @@ def vq_linear_perm_supported(m: int, n: int, k: int, num_centroids: int, vector_
                                                          int(vector_len), int(bits)))  # fmt: skip
 
 
-def gemv_stages_activations(m: int, n: int, k: int, table_in_lds: bool) -> bool:
+def gemv_stages_activations(m: int, n: int, k: int, num_centroids: int) -> bool:
     """Whether a fused GEMV call of *m* tokens on an ``n x k`` layer runs the kernel that stages its
     activations through LDS (``npamd_gemv_stages_activations``): then the GEMV stays ahead of the
-    tile GEMM up to its 32 tokens at any ``k``."""
-    return bool(_lib.load().npamd_gemv_stages_activations(int(m), int(n), int(k), int(bool(table_in_lds))))
+    tile GEMM up to its 32 tokens at any ``k``.  *num_centroids*: rows of the layer's codebook of
+    eight-element vectors, 0 for a group-quantized layer."""
+    return bool(_lib.load().npamd_gemv_stages_activations(int(m), int(n), int(k), int(num_centroids)))
 
 
 def vq_fused_supported(in_features: int, vector_len: int, bits: int) -> bool:
@@ -371,8 +372,18 @@ def sliced_workspace(device: torch.device, nbytes: int, stream: int | None = Non
     ws = _SLICED_WORKSPACES.get(key)
     if ws is None or ws.numel() * 4 < nbytes:
         ws = torch.zeros(max(nbytes, 1 << 20) // 4 + 4, device=device, dtype=torch.float32)
-        _SLICED_WORKSPACES[key] = ws
+        # A buffer made inside a graph capture lives in the graph's private pool and is zero-filled
+        # only when the graph is replayed: it serves this capture and is not kept (an eager call, or
+        # another capture on the same stream, before the first replay would start from garbage).
+        if not torch.cuda.is_current_stream_capturing():
+            _SLICED_WORKSPACES[key] = ws
     return ws
+
+
+def drop_sliced_workspace(device: torch.device, stream: int) -> None:
+    """Forget the cached workspace of (*device*, *stream*): after a failed call it may not be
+    zero-filled any more, and the kernels count on that."""
+    _SLICED_WORKSPACES.pop((device.index, stream), None)
 
 
 def vq_linear_sliced(
@@ -419,15 +430,21 @@ def vq_linear_sliced_checked(x, sliced, cb, bias_f32, column_perm, workspace=Non
     on ``x``'s device.  The library still validates sizes and pointers."""
     m = x.shape[0]
     stream = _stream(x)
-    if workspace is None:
+    own = workspace is None
+    if own:
         workspace = sliced_workspace(x.device, sliced.workspace_bytes(max(m, 1)), stream)
     y = torch.empty((m, sliced.n), device=x.device, dtype=x.dtype)
     dt = _DT[x.dtype]
-    _lib.call(
-        "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), _ptr(column_perm), sliced.header_ptr, sliced.blob.data_ptr(),
-        cb.data_ptr(), dt, _ptr(bias_f32), y.data_ptr(), sliced.n, m, dt,
-        workspace.data_ptr(), workspace.numel() * 4, stream,
-    )  # fmt: skip
+    try:
+        _lib.call(
+            "npamd_vq_gemv_sliced", x.data_ptr(), x.stride(0), _ptr(column_perm), sliced.header_ptr, sliced.blob.data_ptr(),
+            cb.data_ptr(), dt, _ptr(bias_f32), y.data_ptr(), sliced.n, m, dt,
+            workspace.data_ptr(), workspace.numel() * 4, stream,
+        )  # fmt: skip
+    except RuntimeError:
+        if own:  # a launch of a multi-pass call may have run: the shared buffer is not known to be zero
+            drop_sliced_workspace(x.device, stream)
+        raise
     return y
 
 

@@ -125,6 +125,18 @@ class Backend(_StrEnum):
     AUTO = "auto"
 
 
+def tensor_version(t) -> int:
+    """``t._version`` for cache keys, or -1 for tensors that keep no version counter.
+
+    Tensors created or moved under ``torch.inference_mode()`` raise on ``_version``; they
+    cannot be written in place outside inference mode either, so device and address identify them.
+    """
+    try:
+        return t._version
+    except RuntimeError:
+        return -1
+
+
 def tile_band_ok(
     m: int, n: int, k: int, cus: int, min_fraction: float, split_max_tokens: int, long_k: int
 ) -> bool:

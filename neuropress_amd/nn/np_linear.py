@@ -29,7 +29,7 @@ import torch.nn.functional as F
 
 from ..qweights import ScalarQScheme, ScalarQWeight, is_scalar_qweight
 from ..t2n.packing import BitPacking
-from .backends import Backend, LinearBackend, is_hip_backend_available, tile_band_ok
+from .backends import Backend, LinearBackend, is_hip_backend_available, tensor_version, tile_band_ok
 
 log = logging.getLogger(__name__)
 
@@ -265,7 +265,7 @@ class NPLinear(nn.Module):
         # copy_ into `bias` makes a new fp32 copy.  Not stored inside a graph capture (a tensor made
         # there holds data only after a replay).
         src = self.bias
-        key = (src.device, src.data_ptr(), src._version)
+        key = (src.device, src.data_ptr(), tensor_version(src))
         hit = self._derived.get("bias_f32")
         if hit is not None and hit[0] == key:
             return hit[1]
@@ -324,7 +324,7 @@ class NPLinear(nn.Module):
             if self.nbits == 4:
                 from .. import kernels
 
-                if kernels.gemv_stages_activations(m, self.out_features, self.in_features, False):
+                if kernels.gemv_stages_activations(m, self.out_features, self.in_features, 0):
                     return _Q_FUSED_WIDE_MAX_TOKENS
         return _Q_FUSED_MAX_TOKENS
 

@@ -31,6 +31,7 @@ from __future__ import annotations
 
 import logging
 import os
+import weakref
 
 import torch
 import torch.nn as nn
@@ -44,7 +45,7 @@ from ..transforms.vq_packing import (
     TieredIndexPacking,
     ZeroEscapePacking,
 )
-from .backends import Backend, VQBackend, is_hip_backend_available, tile_band_ok
+from .backends import Backend, VQBackend, is_hip_backend_available, tensor_version, tile_band_ok
 
 log = logging.getLogger(__name__)
 
@@ -98,6 +99,9 @@ _GEMV_KERNEL_MAX_TOKENS: int = 32  # what the GEMV entry points accept (NPAMD_GE
 _SLICED_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_SLICED_MAX_TOKENS",), 7)
 _SLICED_MIN_CENTROIDS: int = 4097
 _SLICED_MIN_INDICES: int = _env_int(("NEUROPRESS_VQ_SLICED_MIN_INDICES",), 1 << 20)
+# Whether a module that reaches a GPU through .to() / .cuda() / load_state_dict() builds the tensors
+# its kernels derive from the buffers there and then (slice lists: a host round trip per layer).
+_PREPARE_ON_MOVE: bool = _env_int(("NEUROPRESS_VQ_PREPARE_ON_MOVE",), 1) != 0
 
 # cuda_lut layers: 0 = always decode + GEMM, the reference's default routing.
 _LUT_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_LUT_MAX_TOKENS",), 0)
@@ -249,6 +253,38 @@ class VQProxy(nn.Module):
         super().__init__()
         self.register_buffer("centroids", centroids.to(torch.float16))
         self._cast_cache: dict = {}
+        # Layers that read this codebook (weakly held, not copied or pickled with the proxy): told
+        # when the codebook moves or is reloaded, because a parent's .to() may move a layer first.
+        self._users: weakref.WeakSet = weakref.WeakSet()
+        self.register_load_state_dict_post_hook(VQProxy._after_load_state_dict)
+
+    def _bind(self, user: nn.Module) -> None:
+        self._users.add(user)
+
+    def _notify_users(self) -> None:
+        for user in list(self._users):
+            if user.proxy is self or user.residual_proxy is self:
+                user._prepare_after_move()
+
+    def _apply(self, fn, recurse: bool = True):
+        result = super()._apply(fn, recurse)
+        self._cast_cache = {}
+        self._notify_users()
+        return result
+
+    @staticmethod
+    def _after_load_state_dict(module, incompatible_keys) -> None:
+        module._cast_cache = {}
+        module._notify_users()
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state.pop("_users", None)
+        return state
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        self._users = weakref.WeakSet()
 
     @property
     def num_centroids(self) -> int:
@@ -268,7 +304,7 @@ class VQProxy(nn.Module):
         c = self.centroids
         if dtype == c.dtype:
             return c
-        key = (dtype, c.device, c.data_ptr(), c._version)
+        key = (dtype, c.device, c.data_ptr(), tensor_version(c))
         hit = self._cast_cache.get("entry")
         if hit is None or hit[0] != key:
             hit = (key, c.to(dtype).contiguous())
@@ -377,6 +413,7 @@ class NPVQLinear(nn.Module):
         # once per layer in state_dict (reference: np_vq_linear.py:588-590).
         object.__setattr__(self, "proxy", proxy)
         object.__setattr__(self, "residual_proxy", residual_proxy)
+        self._bind_proxies()
 
         self.register_buffer("packed_indices", packed_indices.contiguous())
         self._register_optional("bias", bias)
@@ -395,6 +432,8 @@ class NPVQLinear(nn.Module):
         self._register_optional("row_bias", None if row_bias is None else row_bias.to(torch.float16))
         # Derived, rebuilt on demand: f32 bias for the kernels, widened index stream.
         self._derived: dict = {}
+        # load_state_dict() copies into the buffers in place: what was derived from them is stale.
+        self.register_load_state_dict_post_hook(NPVQLinear._after_load_state_dict)
 
     def _expand_prefix_coded(self, coded: torch.Tensor, num_centroids: int) -> tuple[torch.Tensor, int]:
         """Prefix-coded buffer -> ``(fixed-width stream, its bit width)``.
@@ -437,10 +476,52 @@ class NPVQLinear(nn.Module):
         else:
             setattr(self, name, None)
 
+    def _bind_proxies(self) -> None:
+        for proxy in (self.proxy, self.residual_proxy):
+            if proxy is not None:
+                proxy._bind(self)
+
+    def _buffer_places(self) -> tuple:
+        return tuple((b.device, b.data_ptr(), b.dtype) for b in self._buffers.values() if b is not None)
+
     def _apply(self, fn, recurse: bool = True):
+        """``.to()`` / ``.cuda()`` / ``.half()``: the derived tensors belong to the old buffers.  A move
+        is already a heavy host operation, so when the module arrives on a GPU the tensors its
+        kernels derive from the buffers -- the slice lists included -- are made here (or, when the
+        shared codebook arrives after the layer, by the codebook's own move): ``lower on the CPU ->
+        model.to("cuda") -> forward`` reaches the fast decode kernel with no further call, as a
+        caller of the reference expects (neuropress/t2n/model_io.py:590-596).
+        ``NEUROPRESS_VQ_PREPARE_ON_MOVE=0`` leaves that to :func:`neuropress_amd.prepare_decode`."""
+        before = self._buffer_places()
         result = super()._apply(fn, recurse)
-        self._derived = {}
+        if self._buffer_places() != before:
+            self._derived = {}
+        self._bind_proxies()  # a copied or unpickled proxy starts with no users
+        self._prepare_after_move()
         return result
+
+    def _prepare_after_move(self) -> None:
+        if not _PREPARE_ON_MOVE or not self.packed_indices.is_cuda or self.backend not in _FUSED_BACKENDS:
+            return
+        if torch.cuda.is_current_stream_capturing():
+            return
+        # The shared codebooks are sub-modules of the model root, not of this layer, and may still be
+        # on their way: they call back when they arrive.
+        for proxy in (self.proxy, self.residual_proxy):
+            if proxy is not None and proxy.centroids.device != self.packed_indices.device:
+                return
+        try:
+            if not self.prepare_sliced():
+                self.prepare()
+        except RuntimeError as exc:  # no kernel library on this machine: forward will say so
+            if not _ALLOW_FALLBACK:
+                raise
+            self._fallback("prepare", "unprepared kernels", exc)
+
+    @staticmethod
+    def _after_load_state_dict(module, incompatible_keys) -> None:
+        module._derived = {}
+        module._prepare_after_move()
 
     # ------------------------------------------------------------------
     # Factory / inverse
@@ -539,7 +620,7 @@ class NPVQLinear(nn.Module):
         Inside a graph capture nothing is stored: a tensor made there lives in the graph's
         private pool and holds data only after a replay, so a later eager call must make its own.
         """
-        key = (source.device, source.data_ptr(), source._version)
+        key = (source.device, source.data_ptr(), tensor_version(source))
         hit = self._derived.get(name)
         if hit is not None and hit[0] == key:
             return hit[1]
@@ -551,7 +632,7 @@ class NPVQLinear(nn.Module):
     def _derived_hit(self, name: str, source: torch.Tensor):
         """The cached value of :meth:`_derive`, or None when it is missing or stale."""
         hit = self._derived.get(name)
-        if hit is not None and hit[0] == (source.device, source.data_ptr(), source._version):
+        if hit is not None and hit[0] == (source.device, source.data_ptr(), tensor_version(source)):
             return hit[1]
         return None
 
@@ -778,8 +859,8 @@ class NPVQLinear(nn.Module):
         if hit is None or hit[0] != m:
             from .. import kernels
 
-            table_bytes = self.proxy.num_centroids * self.vector_len * 2
-            hit = (m, kernels.gemv_stages_activations(m, self.out_features, self.in_features, table_bytes <= 65536))
+            rows = max(1, self.proxy.num_centroids * self.vector_len // 8)  # table size in rows of eight
+            hit = (m, kernels.gemv_stages_activations(m, self.out_features, self.in_features, rows))
             self._derived["stages"] = hit
         return hit[1]
 

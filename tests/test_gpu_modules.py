@@ -129,7 +129,7 @@ def test_long_k_layers_of_one_row_tile_keep_the_gemv_to_32_tokens(gpu, monkeypat
     for nc, expect in ((65536, "vq_linear"), (4096, "vq_gemm_tile")):
         L = cases.vq_layer(70 + nc, n, k, nc, bias=False, std=0.05)
         layer = NPVQLinear(VQProxy(L["cb"]).to(gpu), L["packed"], L["bits"], n, k, 8, "cuda_wmma").to(gpu)
-        assert kernels.gemv_stages_activations(m, n, k, nc * 16 <= 65536) == (nc == 65536)
+        assert kernels.gemv_stages_activations(m, n, k, nc) == (nc == 65536)
         calls.clear()
         y = layer(x.to(gpu))
         assert calls == [expect], calls

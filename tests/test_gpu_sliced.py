@@ -214,6 +214,7 @@ def test_forward_never_builds_slice_lists(gpu, monkeypatch, caplog):
 
     monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
     monkeypatch.setattr(mod, "_unprepared_warned", False)
+    monkeypatch.setattr(mod, "_PREPARE_ON_MOVE", False)  # as for a layer built from tensors already on the GPU
     L = cases.vq_layer(42, 128, 256, 20000, bits=15, act=torch.float16, m=1, bias=True, std=0.05)  # 15 bits: widened stream
     proxy = mod.VQProxy(L["cb"]).to(gpu)
     layer = mod.NPVQLinear(proxy, L["packed"], L["bits"], 128, 256, 8, "cuda_wmma", bias=L["bias"].float()).to(gpu)
@@ -258,6 +259,7 @@ def test_reloaded_buffers_invalidate_everything_derived_from_them(gpu, oracle_li
     from neuropress_amd.nn import np_vq_linear as mod
 
     monkeypatch.setattr(mod, "_SLICED_MIN_INDICES", 1)
+    monkeypatch.setattr(mod, "_PREPARE_ON_MOVE", False)  # the reload leaves the layer unprepared: fused paths first
     act = torch.float16
     n, k, nc = 192, 512, 20000
     A = cases.vq_layer(71, n, k, nc, bits=15, act=act, m=m, bias=True, std=0.05)

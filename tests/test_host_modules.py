@@ -484,3 +484,31 @@ def test_prefix_coded_backends_resolve_like_the_reference(monkeypatch):
     assert res("auto", use_tiered=True).value == "cuda_tiered"
     assert res("auto").value == "cuda_wmma"
     assert res("cuda_tiered").value == "cuda_tiered"
+
+
+def test_modules_built_under_inference_mode_keep_their_caches_working():
+    """Inference tensors raise on ``_version``; the caches of derived tensors (fp32 bias, codebook
+    casts) key on device and address for them (the reference quantises under inference mode,
+    neuropress/methods/gptq.py:253)."""
+    from neuropress_amd.nn import NPLinear, NPVQLinear, VQProxy
+    from neuropress_amd.nn.backends import tensor_version
+    from tests import cases
+
+    L = cases.vq_layer(5, 32, 64, 256, bits=8, act=torch.float32, m=3, bias=True)
+    Q = cases.q4_layer(6, 32, 64, act=torch.float32, m=3, bias=True)
+    with torch.inference_mode():
+        t = torch.zeros(4)
+        assert tensor_version(t) == -1
+        vq = NPVQLinear(VQProxy(L["cb"].clone()), L["packed"].clone(), 8, 32, 64, 8, "default", bias=L["bias"].clone())
+        ql = NPLinear(Q["blob"].clone(), Q["scale"].clone(), 32, 64, 32, 4, "sym", "default", bias=Q["bias"].clone())
+        assert vq._bias_f32().dtype == torch.float32 and vq._bias_f32() is vq._bias_f32()  # cached
+        assert ql._bias_f32() is ql._bias_f32()
+        assert vq.proxy.centroids_as(torch.bfloat16) is vq.proxy.centroids_as(torch.bfloat16)
+        vq.prepare()
+        y = vq(L["x"])
+        yq = ql(Q["x"])
+    w = L["cb"][L["idx"]].reshape(32, 64).float()
+    assert torch.allclose(y, L["x"] @ w.T + L["bias"], atol=1e-4)
+    wq = ((Q["codes"].float() - 8).reshape(32, 2, 32) * Q["scale"].float().reshape(32, 2, 1)).reshape(32, 64)
+    assert torch.allclose(yq, Q["x"] @ wq.T + Q["bias"], atol=1e-3)
+    assert tensor_version(torch.zeros(2)) == 0
