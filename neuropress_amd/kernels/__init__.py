@@ -448,6 +448,66 @@ def vq_linear_sliced_checked(x, sliced, cb, bias_f32, column_perm, workspace=Non
     return y
 
 
+class SlicedCallPlan:
+    """One layer's :func:`vq_linear_sliced_checked` call with everything that does not change from
+    call to call worked out once: the entry point, the addresses of the codebook, bias, permutation,
+    header and blob, the workspace need per token count.  ``run`` does per call only what depends on
+    the call (x's shape and address, the output tensor, the current stream and its workspace) and
+    returns None whenever anything is not as planned -- the caller then takes the ordinary route,
+    which checks and reports.  The host time to issue a one-token decode call is Python's, not the
+    kernel's: 14 us through the ordinary route against an 11 us kernel."""
+
+    __slots__ = ("fn", "sliced", "cb", "bias_f32", "perm", "device", "index", "dtype", "dt", "n", "k", "limit",
+                 "cb_ptr", "bias_ptr", "perm_ptr", "header_ptr", "blob_ptr", "need", "ws", "ws_ptr", "ws_bytes")
+
+    def __init__(self, sliced: SlicedIndices, cb: torch.Tensor, bias_f32, perm, dtype: torch.dtype, limit: int):
+        self.fn = getattr(_lib.load(), "npamd_vq_gemv_sliced")
+        self.sliced, self.cb, self.bias_f32, self.perm = sliced, cb, bias_f32, perm  # kept alive
+        self.device = sliced.blob.device
+        self.index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self.dtype, self.dt = dtype, _DT[dtype]
+        self.n, self.k = sliced.n, sliced.k
+        self.limit = min(int(limit), _lib.GEMV_MAX_M)
+        self.cb_ptr, self.bias_ptr, self.perm_ptr = cb.data_ptr(), _ptr(bias_f32), _ptr(perm)
+        self.header_ptr, self.blob_ptr = sliced.header_ptr, sliced.blob.data_ptr()
+        self.need = [0] + [sliced.workspace_bytes(m) for m in range(1, self.limit + 1)]
+        self.ws, self.ws_ptr, self.ws_bytes = None, 0, 0
+
+    def run(self, x: torch.Tensor):
+        if x.dtype != self.dtype or x.device != self.device:
+            return None
+        shape = x.shape
+        k, n = self.k, self.n
+        if len(shape) == 2:
+            m, ldx = shape[0], x.stride(0)
+            if shape[1] != k or x.stride(1) != 1:
+                return None
+            out_shape = (m, n)
+        else:
+            if not shape or shape[-1] != k or not x.is_contiguous():
+                return None
+            m, ldx = x.numel() // k, k
+            out_shape = (*shape[:-1], n)
+        if not 1 <= m <= self.limit or _raw_stream is None:
+            return None
+        stream = _raw_stream(self.index)
+        ws = _SLICED_WORKSPACES.get((self.index, stream))
+        if ws is not self.ws:
+            if ws is None:
+                return None
+            self.ws, self.ws_ptr, self.ws_bytes = ws, ws.data_ptr(), ws.numel() * 4
+        if self.ws_bytes < self.need[m]:
+            return None
+        y = torch.empty(out_shape, dtype=self.dtype, device=self.device)
+        rc = self.fn(x.data_ptr(), ldx, self.perm_ptr, self.header_ptr, self.blob_ptr, self.cb_ptr, self.dt,
+                     self.bias_ptr, y.data_ptr(), n, m, self.dt, self.ws_ptr, self.ws_bytes, stream)  # fmt: skip
+        if rc != 0:
+            drop_sliced_workspace(self.device, stream)  # it may not be zero-filled any more
+            self.ws = None
+            return None
+        return y
+
+
 def _vq_linear_coded(what, x, flat, class_streams, payload_streams, payload_bits, payload_base, row_offsets,
                      centroids, vector_len, bias):
     """Shared body of the three prefix-coded GEMV wrappers (``npamd_vq_gemv_coded``)."""

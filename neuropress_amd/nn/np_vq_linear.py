@@ -239,6 +239,15 @@ def _vq_dequant_linear(
 # ---------------------------------------------------------------------------
 
 
+def _versions_of(packed, bias, perm, cent) -> tuple:
+    return (
+        packed._version,
+        cent._version,
+        -1 if bias is None else bias._version,
+        -1 if perm is None else perm._version,
+    )
+
+
 class VQProxy(nn.Module):
     """Shared VQ codebook holder (reference: neuropress/nn/np_vq_linear.py:399-455).
 
@@ -432,6 +441,8 @@ class NPVQLinear(nn.Module):
         self._register_optional("row_bias", None if row_bias is None else row_bias.to(torch.float16))
         # Derived, rebuilt on demand: f32 bias for the kernels, widened index stream.
         self._derived: dict = {}
+        # Per activation dtype: the decode call with its constant arguments worked out once (see forward).
+        self._plans: dict = {}
         # load_state_dict() copies into the buffers in place: what was derived from them is stale.
         self.register_load_state_dict_post_hook(NPVQLinear._after_load_state_dict)
 
@@ -496,6 +507,7 @@ class NPVQLinear(nn.Module):
         result = super()._apply(fn, recurse)
         if self._buffer_places() != before:
             self._derived = {}
+        self._plans = {}
         self._bind_proxies()  # a copied or unpickled proxy starts with no users
         self._prepare_after_move()
         return result
@@ -521,6 +533,7 @@ class NPVQLinear(nn.Module):
     @staticmethod
     def _after_load_state_dict(module, incompatible_keys) -> None:
         module._derived = {}
+        module._plans = {}
         module._prepare_after_move()
 
     # ------------------------------------------------------------------
@@ -670,6 +683,24 @@ class NPVQLinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """Band dispatch by token count (reference: neuropress/nn/np_vq_linear.py:1014-1058)."""
+        entry = self._plans.get(x.dtype)
+        if entry is not None:
+            # A decode call this layer has made before: same buffers, not written to since?  Then the
+            # call is issued with its constant arguments as they were worked out then.
+            plan, packed, bias, perm, cent, versions = entry
+            buffers = self._buffers
+            if (
+                buffers["packed_indices"] is packed
+                and buffers.get("bias") is bias
+                and buffers.get("column_perm") is perm
+                and self.proxy._buffers["centroids"] is cent
+                and (versions is None or versions == _versions_of(packed, bias, perm, cent))
+            ):
+                y = plan.run(x)
+                if y is not None:
+                    return y
+            else:
+                self._plans = {}
         if self.backend in _FUSED_BACKENDS and x.dtype in (torch.float16, torch.bfloat16):
             m = x.numel() // self.in_features
             if m <= min(_SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)) and x.is_cuda:
@@ -898,7 +929,26 @@ class NPVQLinear(nn.Module):
             if self.column_perm is not None:
                 x = x[..., self.column_perm]
             return self._forward_dequant_gemm(x)
+        if x.dtype not in self._plans and not torch.cuda.is_current_stream_capturing():
+            self._plan_sliced_calls(x.dtype, sliced, perm)
         return y.reshape(*leading, self.out_features)
+
+    def _plan_sliced_calls(self, dtype: torch.dtype, sliced, perm) -> None:
+        """Remember how the slice-list call for *dtype* activations was made, with the buffers it was
+        made from: forward() reuses it while those are the module's buffers and unwritten."""
+        from .. import kernels
+
+        hit = self._derived_hit("sliced", self.packed_indices)
+        if hit is None or hit[0] is not sliced:
+            return
+        packed, bias, column_perm, cent = self.packed_indices, self.bias, self.column_perm, self.proxy.centroids
+        plan = kernels.SlicedCallPlan(sliced, self.proxy.centroids_as(dtype), self._bias_f32(), perm, dtype,
+                                      min(hit[1], _SLICED_MAX_TOKENS, _fused_max_tokens(self.backend)))  # fmt: skip
+        try:
+            versions = _versions_of(packed, bias, column_perm, cent)
+        except RuntimeError:  # inference tensors count no versions: writes into them go unseen, as for every cache here
+            versions = None
+        self._plans[dtype] = (plan, packed, bias, column_perm, cent, versions)
 
     def _mfma_layer(self) -> bool:
         """Whether the MFMA kernels take this layer's shape (vector length 8, K a multiple of 64)."""

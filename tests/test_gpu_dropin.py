@@ -260,3 +260,58 @@ def test_the_staging_predicate_names_the_kernel_the_launcher_takes(gpu):
         said, launched = lib.npamd_gemv_stages_activations(m, 6144, 4096, 0), lib.npamd_diag_last_gemv_staged()
         assert said == launched, (m, said, launched)
     assert seen == {0, 1}
+
+
+def test_planned_decode_calls_follow_the_buffers(gpu, oracle_lib, monkeypatch):
+    """A layer's second decode call reuses the arguments of its first.  Writing into a buffer,
+    replacing one, or calling with another dtype, shape or stride must not reuse what no longer holds."""
+    from neuropress_amd import kernels
+
+    monkeypatch.setattr(vqmod, "_SLICED_MIN_INDICES", 1)
+    act = torch.bfloat16
+    n, k = 256, 512
+    A = cases.vq_layer(41, n, k, 20000, bits=15, act=act, m=3, bias=True, std=0.05)
+    B = cases.vq_layer(42, n, k, 20000, bits=15, act=act, m=3, bias=True, std=0.05)
+    proxy = VQProxy(A["cb"]).to(gpu)
+    layer = NPVQLinear(proxy, A["packed"], 15, n, k, 8, "cuda_wmma", bias=A["bias"].float()).to(gpu)
+    planned = []
+    real_run = kernels.SlicedCallPlan.run
+    monkeypatch.setattr(kernels.SlicedCallPlan, "run",
+                        lambda p, xx: (lambda yy: (planned.append(yy is not None), yy)[1])(real_run(p, xx)))
+    x = A["x"].to(gpu)
+    ref = _vq_ref(oracle_lib, A, act)
+    _check(layer(x), ref)
+    assert planned == []  # the first call makes the plan
+    _check(layer(x), ref)
+    _check(layer(x[:1]), ref[:1])
+    _check(layer(x.reshape(1, 3, k)).reshape(3, n), ref)  # leading dimensions are kept
+    wide = torch.zeros(3, 2 * k, dtype=act, device=gpu)
+    wide[:, :k] = x
+    _check(layer(wide[:, :k]), ref)  # a row stride that is not K
+    assert planned == [True] * 4
+    A16 = dict(A, x=A["x"].half(), bias=A["bias"].half())  # bf16 values are fp16 values at these magnitudes
+    _check(layer(x.half()), _vq_ref(oracle_lib, A16, torch.float16))  # another dtype: its own first call
+    planned.clear()
+    # written in place: bias first, then the indices (the lists are stale: fused GEMV until they are rebuilt)
+    layer.bias.copy_(B["bias"].float())
+    _check(layer(x), _vq_ref(oracle_lib, dict(A, bias=B["bias"]), act))
+    assert planned == []
+    layer.packed_indices.copy_(B["packed"])
+    Bx = dict(B, x=A["x"], cb=A["cb"])
+    _check(layer(x), _vq_ref(oracle_lib, Bx, act))
+    layer.prepare_sliced()
+    _check(layer(x), _vq_ref(oracle_lib, Bx, act))
+    _check(layer(x), _vq_ref(oracle_lib, Bx, act))
+    assert planned == [True]
+    # the codebook written in place, then replaced by moving the proxy
+    proxy.centroids.copy_(B["cb"])
+    Bb = dict(B, x=A["x"])
+    _check(layer(x), _vq_ref(oracle_lib, Bb, act))
+    _check(layer(x), _vq_ref(oracle_lib, Bb, act))
+    proxy.to("cpu")
+    proxy.centroids.copy_(A["cb"])
+    proxy.to(gpu)
+    _check(layer(x), _vq_ref(oracle_lib, Bx, act))
+    # eight tokens are past the lists' band: the plan declines, the fused GEMV answers
+    x8 = torch.randn(8, k, generator=cases.gen(8)).to(act)
+    _check(layer(x8.to(gpu)), _vq_ref(oracle_lib, Bx, act, x=x8))
