@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="headline kernel only")
-    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "gemv_cfg2_gateup_m1", "gemv_cfg2_down_m1", "tile_m256", "tile_m384", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_gemv_m16", "q4_gemv_4096_m16", "q4_gemv_28672_m1", "q4_tile_m128", "q4_tile_m256", "rvq_gemv_m1", "rvq_tile_m128",
+    ap.add_argument("--case", default="", choices=["", "sliced_m1", "gemv_m1", "gemv_nc4096_m1", "gemv_cfg2_gateup_m1", "gemv_cfg2_down_m1", "tile_m256", "tile_m384", "tile_nc4096_m128", "dequant", "q4_gemv_m1", "q4_gemv_m16", "q4_gemv_4096_m16", "q4_gemv_28672_m1", "q4_tile_m128", "q4_tile_m256", "q4_tile_m512", "rvq_gemv_m1", "rvq_tile_m128",
                                                     "rms_norm_m4096", "vq_embedding_m4096", "q4_embedding_m4096"],
                     help="profiling aid: launch only this kernel `--steps` times (eagerly, one kernel per launch) "
                          "on the config-3 / config-5 shape (rvq_*: the config-4 4096x4096 projection) and print a one-line JSON with its HIP-event time")
@@ -248,7 +248,7 @@ def main():
             blob = BitPacking4.compress(torch.randint(0, 16, (n, k), generator=g, dtype=torch.int64).to(torch.uint8))
             sc = (torch.rand(n * k // 32, generator=g) * 0.019 + 0.001).to(torch.float16).to(dev)
             pool = [blob.to(dev).clone() for _ in range(n_rot)]
-            m = {"q4_gemv_m1": 1, "q4_gemv_28672_m1": 1, "q4_gemv_m16": 16, "q4_gemv_4096_m16": 16, "q4_tile_m256": 256}.get(args.case, 128)
+            m = {"q4_gemv_m1": 1, "q4_gemv_28672_m1": 1, "q4_gemv_m16": 16, "q4_gemv_4096_m16": 16, "q4_tile_m256": 256, "q4_tile_m512": 512}.get(args.case, 128)
             x = torch.randn(m, k, generator=g).to(torch.float16).to(dev)
             fn = lambda i: kernels.q_linear(x, pool[i], sc, 4, 32)
             alg, flops = n * k // 2 + n * k // 32 * 2 + m * k * 2 + m * n * 2, 2.0 * m * n * k

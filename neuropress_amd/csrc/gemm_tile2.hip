@@ -3,13 +3,29 @@
 
 #include <stdlib.h>
 
+#include <atomic>
+#include <chrono>
+#include <random>
+
 #include <type_traits>
 
 namespace npamd {
 
-__global__ void __launch_bounds__(256) tile2_zero_counters_kernel(uint32_t* counters, int n) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) counters[i] = 0u;
+// A number for one call of the kernel whose two K halves meet through the workspace: the tile words
+// there need no clearing, because a word only counts while it holds the number of the call that
+// reads it, and 64 pseudo-random bits are never what memory happens to hold (the finishing
+// workgroup stores zero over it, so a graph that replays one call, number included, starts clean).
+static unsigned long long next_call_number() {
+  static std::atomic<unsigned long long> counter{[] {
+    std::random_device rd;
+    return ((unsigned long long)rd() << 32) ^ (unsigned long long)rd() ^
+           (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count();
+  }()};
+  unsigned long long z = counter.fetch_add(0x9E3779B97F4A7C15ull) + 0x9E3779B97F4A7C15ull;  // splitmix64
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return z ? z : 1ull;  // zero is what a finished tile holds
 }
 
 // Sixteen 16-byte loads / four 16-byte stores of agent scope (sc1: coherent between the L2 caches of
@@ -86,6 +102,7 @@ struct T2ProdVq16 {
   using Args = T2Args;
   static constexpr int kWRing = 3;
   static constexpr int kLoads = 5;                 // per step: four gathers, one index load
+  static constexpr bool kLoadsLast = true;         // ... issued behind the step's x pieces, in k group 3
   static constexpr int kStageBytes = 4 * 2 * 1024;  // per wave two staged chunks of 64 lanes x 16 bytes
   const Args& a;
   const KWalk& kw;
@@ -142,6 +159,7 @@ struct T2ProdQ {
   static constexpr int kWRing = 2;
   static constexpr int kCodeLoads = NBITS == 4 ? 1 : 2;         // 16 bytes of nibbles, 32 of bytes per lane and step
   static constexpr int kLoads = kCodeLoads + 1 + (ASYM ? 1 : 0);  // + the dword that holds the scale (+ zero point)
+  static constexpr bool kLoadsLast = false;        // requested in k group 0, in front of the step's x pieces
   static constexpr int kSlot = kCodeLoads * 1024 + 256 + (ASYM ? 256 : 0);
   static constexpr int kStageWave = 3 * kSlot;
   static constexpr int kStageBytes = 4 * kStageWave;
@@ -303,12 +321,9 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
   // ---- prologue ----------------------------------------------------------------------------------
   if (!(ABL & 1)) prod.prologue_issue();
   if (wave_active) {
+    const uint8_t* src = tile_src(0);
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      const uint8_t* src = tile_src(p);
-#pragma unroll
-      for (int i = 0; i < kPieces; ++i) fetch_piece(i, p, src);
-    }
+    for (int i = 0; i < kPieces; ++i) fetch_piece(i, 0, src);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (!(ABL & 1)) prod.prologue_finish();
@@ -338,13 +353,14 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
       for (int mt = 0; mt < MW; ++mt) ao[set][mt] = *reinterpret_cast<const u32x4*>(xa + mt * 32 * 128);
     };
     // One step; buf = step % 2 is a compile-time constant through the unrolled loops below.
-    // The step's loads are issued behind MFMAs: the producer's in k groups 0 and 1, the x tile of
-    // step + 2 in k group 3, whose operands are the last this step reads from the buffer the tile
-    // goes into (the wait in front of the first piece makes sure they have arrived, wherever the
-    // scheduler puts that piece among the group's MFMAs).
+    // The step's loads are issued behind MFMAs, one at a time, so that the address unit is fed all
+    // through the step instead of in two bursts: the x tile of step + 1 piece by piece in k groups
+    // 0 to 2 (it goes into the other buffer, which this wave read for the last time a step ago),
+    // a producer's lookups behind them in k group 3 (they fill the W slot of step + 2 and may stay
+    // in flight over the barrier), a producer's streamed bytes in k groups 0 and 1.
     auto one_step = [&](int buf, int step, int wslot) {
       read_ops(0, buf, wslot, 0);
-      const uint8_t* src = tile_src(step + 2);
+      const uint8_t* src = tile_src(step + 1);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (j < 3) read_ops((j + 1) & 1, buf, wslot, j + 1);
@@ -355,22 +371,24 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
           for (int mt = 0; mt < MW; ++mt)
             if (!(ABL & 4)) acc[mt][t] = mfma32<ACT>(ao[j & 1][mt], bo[j & 1][t], acc[mt][t]);
           if (!(ABL & 1)) {
-            if (j == 0 && t == 0) prod.template work<0, 0>(step, wslot);
-            if (j == 0 && t == 1) prod.template work<0, 1>(step, wslot);
-            if (j == 0 && t == 2) prod.template work<0, 2>(step, wslot);
-            if (j == 0 && t == 3) prod.template work<0, 3>(step, wslot);
-            if (j == 1 && t == 0) prod.template work<1, 0>(step, wslot);
-            if (j == 1 && t == 1) prod.template work<1, 1>(step, wslot);
+            if constexpr (Prod::kLoadsLast) {
+              if (j == 3 && t == 0) prod.template work<0, 0>(step, wslot);
+              if (j == 3 && t == 1) prod.template work<0, 1>(step, wslot);
+            } else {
+              if (j == 0 && t == 0) prod.template work<0, 0>(step, wslot);
+              if (j == 0 && t == 1) prod.template work<0, 1>(step, wslot);
+              if (j == 0 && t == 2) prod.template work<0, 2>(step, wslot);
+              if (j == 0 && t == 3) prod.template work<0, 3>(step, wslot);
+              if (j == 1 && t == 0) prod.template work<1, 0>(step, wslot);
+              if (j == 1 && t == 1) prod.template work<1, 1>(step, wslot);
+            }
           }
-          if (j == 3 && t < 3) {
-            if (t == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-            for (int i = t * kPieces / 3; i < (t + 1) * kPieces / 3; ++i) fetch_piece(i, buf, src);
-          }
+          if (j * 4 + t < kPieces) fetch_piece(j * 4 + t, buf ^ 1, src);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kProdLoads + ((ABL & 2) ? 0 : kPieces)) : "memory");
+      // Everything but a producer's lookups of this step has to be there when the next step starts.
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(Prod::kLoadsLast ? kProdLoads : 0) : "memory");
       block_sync_lds();
     };
     int wslot = 0;
@@ -423,13 +441,13 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
     float* const mine = pair.tiles + ((size_t)blockIdx.z * tiles + tile_id) * kTileFloats + wave * (MW * 64 * 64) + lane * 4;
     const float* const theirs =
         pair.tiles + ((size_t)(blockIdx.z ^ 1) * tiles + tile_id) * kTileFloats + wave * (MW * 64 * 64) + lane * 4;
-    uint32_t* const flag = reinterpret_cast<uint32_t*>(ws);  // outside the waves' output areas
-    uint32_t* const cnt = pair.counters + tile_id;
+    unsigned long long* const flag = reinterpret_cast<unsigned long long*>(ws);  // outside the waves' output areas
+    unsigned long long* const word = pair.words + tile_id;
     __syncthreads();  // every wave is past its last LDS read
-    if (tid == 0) flag[0] = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) flag[0] = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    uint32_t arrived = flag[0];
-    if (arrived == 0) {
+    bool arrived = flag[0] == pair.call;  // the other half is there already: nothing to write
+    if (!arrived) {
       if (wave_active) {
 #pragma unroll
         for (int mt = 0; mt < MW; ++mt)
@@ -442,13 +460,13 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the tile is where the other workgroup will read it
       __syncthreads();
-      if (tid == 0) flag[1] = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) flag[1] = __hip_atomic_exchange(word, pair.call, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
-      arrived = flag[1];
+      arrived = flag[1] == pair.call;  // it came while this half was being written
     }
-    finish = arrived != 0;
+    finish = arrived;
     if (finish) {
-      if (tid == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next call
+      if (tid == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for a replay of this call
       if (wave_active) {
 #pragma unroll
           for (int mt = 0; mt < MW; ++mt) {
@@ -507,10 +525,6 @@ int launch_tile2_mw(const GemmShape& s, const typename Prod::Args& a, const T2Pa
   const hipError_t e = enable_dynamic_lds(latch, reinterpret_cast<const void*>(&tile2_gemm_kernel<ACT, MW, Prod, ABL>), lds);
   if (e != hipSuccess)
     return fail(NPAMD_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
-  if (s.splits == 2) {
-    const int tiles = (int)(grid.x * grid.y);
-    tile2_zero_counters_kernel<<<(tiles + 255) / 256, 256, 0, st>>>(pair.counters, tiles);
-  }
   tile2_gemm_kernel<ACT, MW, Prod, ABL><<<grid, 256, lds, st>>>(s, a, pair);
   if (s.splits > 2) {
     const int64_t quads = (int64_t)s.M * ((s.N + 3) / 4);
@@ -531,11 +545,12 @@ int launch_tile2_prod(GemmShape s, const typename Prod::Args& a, hipStream_t st,
   s.split_chunks = (s.chunks + splits - 1) / splits;
   s.splits = (s.chunks + s.split_chunks - 1) / s.split_chunks;
   s.partials = (float*)workspace;
-  T2Pair pair{nullptr, nullptr};
+  T2Pair pair{nullptr, nullptr, 0ull};
   if (s.splits == 2) {
     const int64_t tiles = (int64_t)((s.N + kT2Cols - 1) / kT2Cols) * ((s.M + 128 * mw - 1) / (128 * mw));
-    pair.counters = (uint32_t*)workspace;
-    pair.tiles = (float*)((uint8_t*)workspace + ((tiles * 4 + 255) & ~(int64_t)255));
+    pair.words = (unsigned long long*)workspace;
+    pair.tiles = (float*)((uint8_t*)workspace + ((tiles * 8 + 255) & ~(int64_t)255));
+    pair.call = next_call_number();
   }
 #ifdef NPAMD_TILE2_ABLATIONS
   if (const char* e = getenv("NPAMD_T2_DEBUG_PTR")) {

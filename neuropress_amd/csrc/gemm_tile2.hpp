@@ -64,8 +64,9 @@ struct T2QArgs {
 // zero again on exit) and the f32 tile of whichever half finished first, [2][tiles][BM * 128] in
 // register order.
 struct T2Pair {
-  uint32_t* counters;
+  unsigned long long* words;  // one per tile: holds `call` while one half of the tile has arrived in this call
   float* tiles;
+  unsigned long long call;    // this call's number, drawn at random: never what memory happens to hold
 };
 
 // Splits of K for the 128-column kernel: 1 while the block tiles cover most compute units, else as
@@ -86,7 +87,7 @@ inline int64_t tile2_workspace_bytes(int M, int N, int chunks, int mw) {
   if (splits <= 1) return 0;
   if (splits > 2) return (int64_t)splits * M * N * 4;
   const int64_t tiles = (int64_t)((N + kT2Cols - 1) / kT2Cols) * ((M + 128 * mw - 1) / (128 * mw));
-  return ((tiles * 4 + 255) & ~(int64_t)255) + 2 * tiles * (128 * mw) * kT2Cols * 4;
+  return ((tiles * 8 + 255) & ~(int64_t)255) + 2 * tiles * (128 * mw) * kT2Cols * 4;
 }
 
 // Take the call when the workspace allows the planned split; return 1 when they did not take it.

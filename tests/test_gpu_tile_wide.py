@@ -149,3 +149,41 @@ def test_wide_tile_gemm_group_affine_decodes_bit_exactly(gpu, tile_wide, act, nb
         tile_wide(2, splits)
         assert torch.equal(kernels.q_gemm_tile(eye, blob, sc, nbits, gs, zp), wt), f"1024 tokens, {splits} splits"
         assert torch.equal(kernels.q_gemm_tile(eye[100:330], blob, sc, nbits, gs, zp), wt[100:330]), f"230 tokens, {splits} splits"
+
+
+@pytest.mark.parametrize("m", [130, 384])
+def test_wide_tile_gemm_meets_through_a_workspace_nobody_cleared(gpu, tile_wide, m):
+    """The two K halves of a tile meet through a word of the workspace that holds the call's own
+    random number; the workspace comes from torch's allocator as it is.  Whatever the memory held
+    before -- all ones, the words a previous call left -- the result is the same, and a graph that
+    replays one call (number included) gives it on every replay."""
+    from neuropress_amd import _lib, kernels
+
+    n, k = 520, 1024
+    tile_wide(2, 2)
+    L = cases.vq_layer(900 + m, n, k, 65536, bits=16, act=torch.bfloat16, m=m, bias=True, std=0.05)
+    x, pk, cb, bias = L["x"].to(gpu), L["packed"].to(gpu), L["cb"].bfloat16().to(gpu), L["bias"].to(gpu)
+    tile_wide(2, 1)
+    whole = kernels.vq_gemm_tile(x, pk, cb, 16, n, bias)  # K in one piece: no workspace
+    tile_wide(2, 2)
+    need = _lib.load().npamd_gemm_tile_workspace_bytes(m, n, k)
+    assert need > 0
+    expect = kernels.vq_gemm_tile(x, pk, cb, 16, n, bias)
+    assert float((expect.float() - whole.float()).abs().max()) <= 2.0 ** -6  # f32 sums in another order
+    for fill in (0xFF, 0x00, 0x5A):
+        junk = torch.full((need + (1 << 20),), fill, dtype=torch.uint8, device=gpu)
+        del junk  # back to the allocator: the next call's workspace is carved out of it
+        for _ in range(3):  # the second and third call find the words the one before left
+            assert torch.equal(kernels.vq_gemm_tile(x, pk, cb, 16, n, bias), expect)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            y = kernels.vq_gemm_tile(x, pk, cb, 16, n, bias)
+    for _ in range(4):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, expect)
+        assert torch.equal(kernels.vq_gemm_tile(x, pk, cb, 16, n, bias), expect)  # eager work between the replays
