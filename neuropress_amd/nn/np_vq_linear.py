@@ -116,11 +116,11 @@ _TILE_MAX_TOKENS: int = _env_int(
 )
 
 # Layers whose codebook LDS does not hold (more than 4096 rows of eight) and that have at least
-# _TILE_WIDE_MIN_FEATURES output or input features run the 128-column tile GEMM, which stays ahead
-# of decode + GEMM up to its 384-row block: 14336 x 4096 75-77 us at 384 tokens against 102 us,
-# 4096 x 14336 78-82 us against 117 us (the 64-column kernel: 84-97 us).
+# _TILE_WIDE_MIN_WEIGHTS weights run the 128-column tile GEMM, which stays ahead of decode + GEMM up
+# to its 384-row block: 14336 x 4096 70 us at 384 tokens against 102 us, 4096 x 14336 76 us against
+# 117 us (the 64-column kernel: 80 and 87 us).
 _TILE_WIDE_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_TILE_WIDE_MAX_TOKENS",), 384)
-_TILE_WIDE_MIN_FEATURES: int = 8192
+_TILE_WIDE_MIN_WEIGHTS: int = 1 << 25
 
 # The tile GEMM gives each workgroup 64 output columns (and up to 384 rows).  When
 # that grid covers less than this fraction of the compute units the kernel splits
@@ -968,7 +968,7 @@ class NPVQLinear(nn.Module):
             and not self.is_residual
             and self.vector_len == 8
             and self.proxy.num_centroids * self.vector_len * 2 > 65536
-            and max(self.in_features, self.out_features) >= _TILE_WIDE_MIN_FEATURES
+            and self.in_features * self.out_features >= _TILE_WIDE_MIN_WEIGHTS
         ):
             return max(_TILE_MAX_TOKENS, _TILE_WIDE_MAX_TOKENS)
         return _TILE_MAX_TOKENS

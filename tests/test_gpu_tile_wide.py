@@ -83,11 +83,11 @@ def test_wide_tile_gemm_decodes_bit_exactly(gpu, tile_wide, act, splits):
 
 
 def test_wide_and_narrow_tile_gemm_agree_on_a_large_layer(gpu, tile_wide):
-    """A layer of the size the library takes the 128-column kernel for by itself (8192 columns), K in two
+    """A layer of the size the library takes the 128-column kernel for by itself (2^25 weights), K in two
     halves: against the 64-column kernel and the dense product of the decoded weight."""
     from neuropress_amd import _lib, kernels
 
-    n, k, m = 8192, 1024, 384
+    n, k, m = 8192, 4096, 384
     g = cases.gen(5)
     cb = (torch.randn(65536, 8, generator=g) * 0.02).to(torch.float16)
     pk = torch.randint(0, 65536, (n * k // 8,), generator=g, dtype=torch.int32).to(torch.int16).view(torch.uint8).to(gpu)
