@@ -89,3 +89,47 @@ def test_nothing_but_the_lds_direct_loads_touches_m0(assembly):
                 assert in_asm, ln
                 checked += 1
     assert checked > 0
+
+
+@pytest.fixture(scope="module")
+def assembly_wide(tmp_path_factory):
+    """The gfx950 assembly of the 128-column tile GEMM (csrc/gemm_tile2.hip)."""
+    if shutil.which("hipcc") is None and not build.Path("/opt/rocm/bin/hipcc").exists():
+        pytest.skip("needs hipcc")
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    out = tmp_path_factory.mktemp("codegen") / "gemm_tile2.s"
+    cmd = [hipcc, *build.CXXFLAGS, *build.DEVICE_FLAGS, "-S", "--cuda-device-only",
+           str(build.CSRC / "gemm_tile2.hip"), "-o", str(out)]  # fmt: skip
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    return out.read_text().split("\n")
+
+
+def test_the_wide_kernel_loads_everything_into_lds_and_leaves_m0_to_its_transfers(assembly_wide):
+    """``tile2_gemm_kernel`` brings x tiles, indices, codebook rows and packed bytes into LDS with
+    ``s_mov_b32 m0, <LDS address>; global_load_lds_dword[x4]`` asm statements and counts them by hand
+    (``s_waitcnt vmcnt(n)``).  Sound only while (a) the compiler keeps nothing of its own in m0 and (b)
+    every vector-memory load of the main loop is one of those transfers, so that the hand-written counts
+    see all of a wave's loads: outside asm statements the kernels may load from global memory only where
+    the compiler's own waits cover it (bias, the handoff's first look at the tile word)."""
+    lines = assembly_wide
+    starts = [i for i, ln in enumerate(lines) if re.match(r"^_ZN5npamd17tile2_gemm_kernel\S*: ;", ln)]
+    assert len(starts) >= 20  # VQ and int4 / int8 producers x activation dtypes x row tiles
+    for i in starts:
+        name = lines[i].split(":")[0]
+        end = next(j for j in range(i, len(lines)) if lines[j].startswith(".Lfunc_end"))
+        in_asm, transfers, spills = False, 0, 0
+        for ln in lines[i:end]:
+            code = ln.split(";")[0]
+            if "#ASMSTART" in ln:
+                in_asm = True
+            elif "#ASMEND" in ln:
+                in_asm = False
+            elif re.search(r"\bm0\b", code):
+                assert in_asm, (name, ln)
+            if in_asm and "global_load_lds_dword" in code:
+                transfers += 1
+            if re.match(r"\s+scratch_(load|store)", code):
+                spills += 1
+        assert transfers >= 10, (name, transfers)
+        assert spills == 0, (name, spills)  # 512 registers per lane hold the wave tile: nothing goes to scratch
