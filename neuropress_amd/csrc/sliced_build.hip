@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <atomic>
 #include <numeric>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -87,27 +88,37 @@ inline int lds_pass_of_lane(int lane) {
   return (lane >> 5) * 2 + (first ? 0 : 1);
 }
 
-void spread_bank_groups(std::vector<uint32_t>* const* tasks, int lanes, int64_t steps) {
+// A task's entries: a run of the builder's flat entry array.
+struct TaskSpan {
+  uint32_t* e;
+  uint32_t n;
+  uint32_t size() const { return n; }
+};
+
+void spread_bank_groups(const TaskSpan* tasks, int lanes, int64_t steps) {
   constexpr int kXWeight = 1;
   int pass_lanes[4][16], pass_count[4] = {0, 0, 0, 0};
   for (int lane = 0; lane < lanes; ++lane) {
     const int p = lds_pass_of_lane(lane);
     pass_lanes[p][pass_count[p]++] = lane;
   }
+  // Lanes with the fewest entries choose first: they have the least freedom.
+  int order[4][16];
+  for (int p = 0; p < 4; ++p) {
+    for (int i = 0; i < pass_count[p]; ++i) order[p][i] = pass_lanes[p][i];
+    std::stable_sort(order[p], order[p] + pass_count[p], [&](int a, int b) { return tasks[a].size() < tasks[b].size(); });
+  }
   for (int64_t t = 0; t < steps; ++t) {
     for (int p = 0; p < 4; ++p) {
       int g_count[16] = {0}, r_count[16] = {0};
       uint8_t g_seen[kSlicedMaxGroups] = {0};
-      // Lanes with the fewest entries left choose first: they have the least freedom.
-      int order[16];
-      for (int i = 0; i < pass_count[p]; ++i) order[i] = pass_lanes[p][i];
-      std::stable_sort(order, order + pass_count[p], [&](int a, int b) { return tasks[a]->size() < tasks[b]->size(); });
       for (int i = 0; i < pass_count[p]; ++i) {
-        std::vector<uint32_t>& e = *tasks[order[i]];
-        if ((int64_t)e.size() <= t) continue;
+        const TaskSpan& task = tasks[order[p][i]];
+        uint32_t* const e = task.e;
+        if ((int64_t)task.size() <= t) continue;
         size_t best = (size_t)t;
         int best_cost = 1 << 30;
-        for (size_t j = (size_t)t; j < e.size(); ++j) {
+        for (size_t j = (size_t)t; j < task.size(); ++j) {
           const uint32_t row = e[j] & 0xFFFFu, g = e[j] >> 16;
           const int gc = g_seen[g] ? 0 : g_count[g & 15];
           const int cost = kXWeight * gc + r_count[row & 15];
@@ -222,21 +233,28 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   const int slice_rows = kSlicedMaxSliceRows;
   const int S = (nc + slice_rows - 1) / slice_rows;
 
-  // Indices transposed to [G][N] so a (group, row range) scan is contiguous.
-  std::vector<uint32_t> idx_t((size_t)n_idx);
+  // Indices as 32-bit values, row-major, clamped as the decode kernels clamp them; per-slice counts.
+  std::vector<uint32_t> idx((size_t)n_idx);
   std::vector<int64_t> slice_count((size_t)S, 0);
+  const int chunk = 64;  // rows per work item
+  const int chunks = (N + chunk - 1) / chunk;
   {
-    const int chunk = 256;  // rows per work item
-    const int chunks = (N + chunk - 1) / chunk;
     std::vector<std::vector<int64_t>> counts((size_t)chunks, std::vector<int64_t>((size_t)S, 0));
     parallel_for(chunks, [&](int c) {
-      for (int n = c * chunk; n < std::min(N, (c + 1) * chunk); ++n)
-        for (int g = 0; g < G; ++g) {
-          uint32_t v = host_read_index(packed, n_bytes, (int64_t)n * G + g, bits);
-          if (v > (uint32_t)nc - 1u) v = (uint32_t)nc - 1u;  // same clamp as the decode kernels
-          idx_t[(size_t)g * N + n] = v;
-          counts[(size_t)c][v / slice_rows]++;
+      int64_t* cnt = counts[(size_t)c].data();
+      for (int n = c * chunk; n < std::min(N, (c + 1) * chunk); ++n) {
+        uint32_t* row = &idx[(size_t)n * G];
+        if (bits == 16) {
+          const uint16_t* src = reinterpret_cast<const uint16_t*>(packed) + (size_t)n * G;  // little endian
+          for (int g = 0; g < G; ++g) row[g] = src[g];
+        } else {
+          for (int g = 0; g < G; ++g) row[g] = host_read_index(packed, n_bytes, (int64_t)n * G + g, bits);
         }
+        for (int g = 0; g < G; ++g) {
+          if (row[g] > (uint32_t)nc - 1u) row[g] = (uint32_t)nc - 1u;  // same clamp as the decode kernels
+          cnt[row[g] / (uint32_t)slice_rows]++;
+        }
+      }
     });
     for (auto& c : counts)
       for (int s = 0; s < S; ++s) slice_count[(size_t)s] += c[(size_t)s];
@@ -272,12 +290,63 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   }
   const int n_wg = (int)jobs.size();
 
-  // Pass 1, one workgroup at a time: the tasks in strip and lane order.  Pass 2 writes them at
-  // the places the layer-wide strip lengths fix.
+  // Every index is filed under its workgroup (slice, group range, row block) and row in one sweep
+  // over the rows: count, turn the counts into places in one flat entry array, fill.  A task's
+  // entries come out in ascending group order.
+  const int rpb = geo.rows_per_block;
+  std::vector<int> range_groups((size_t)S), wg_base((size_t)S);  // groups per range; first workgroup slot of a slice
+  std::vector<int> wg_of;                                        // (slice, part, row block) -> workgroup
+  {
+    int slots = 0;
+    for (int s = 0; s < S; ++s) {
+      range_groups[(size_t)s] = (G + geo.parts[(size_t)s] - 1) / geo.parts[(size_t)s];
+      wg_base[(size_t)s] = slots;
+      slots += geo.parts[(size_t)s] * geo.row_blocks;
+    }
+    wg_of.assign((size_t)slots, -1);
+    for (int w = 0; w < n_wg; ++w)
+      wg_of[(size_t)(wg_base[(size_t)jobs[w].slice] + jobs[w].part * geo.row_blocks + jobs[w].block)] = w;
+  }
+  std::vector<uint32_t> task_len((size_t)n_wg * rpb, 0u);   // entries of (workgroup, row of its block)
+  parallel_for(chunks, [&](int c) {
+    for (int n = c * chunk; n < std::min(N, (c + 1) * chunk); ++n) {
+      const uint32_t* row = &idx[(size_t)n * G];
+      const int rb = n / rpb, r = n - rb * rpb;
+      for (int g = 0; g < G; ++g) {
+        const int sl = (int)(row[g] / (uint32_t)slice_rows);
+        const int w = wg_of[(size_t)(wg_base[(size_t)sl] + (g / range_groups[(size_t)sl]) * geo.row_blocks + rb)];
+        ++task_len[(size_t)w * rpb + r];
+      }
+    }
+  });
+  std::vector<int64_t> task_begin((size_t)n_wg * rpb + 1);
+  task_begin[0] = 0;
+  for (size_t i = 0; i < (size_t)n_wg * rpb; ++i) task_begin[i + 1] = task_begin[i] + task_len[i];
+  std::vector<uint32_t> entries((size_t)n_idx);
+  parallel_for(chunks, [&](int c) {
+    std::vector<uint32_t> filled;
+    for (int n = c * chunk; n < std::min(N, (c + 1) * chunk); ++n) {
+      const uint32_t* row = &idx[(size_t)n * G];
+      const int rb = n / rpb, r = n - rb * rpb;
+      // per workgroup of this row: how many entries are in place (a row belongs to one work item)
+      filled.assign((size_t)n_wg, 0u);
+      for (int g = 0; g < G; ++g) {
+        const uint32_t v = row[g];
+        const int sl = (int)(v / (uint32_t)slice_rows);
+        const int part = g / range_groups[(size_t)sl];
+        const int w = wg_of[(size_t)(wg_base[(size_t)sl] + part * geo.row_blocks + rb)];
+        entries[(size_t)(task_begin[(size_t)w * rpb + r] + filled[(size_t)w]++)] =
+            (v % (uint32_t)slice_rows) | ((uint32_t)(g - part * range_groups[(size_t)sl]) << 16);
+      }
+    }
+  });
+  idx.clear();
+  idx.shrink_to_fit();
+
+  // One workgroup at a time: strips, lane order and the order of the entries inside a task.
   struct Built {
-    std::vector<uint32_t> entries;  // the tasks' entries, one task after the other in lane order
-    uint32_t begin[kSlicedTasks + 1];
-    int steps[kSlicedWaves];        // longest task of each strip
+    std::vector<uint16_t> order;  // task (row of the block) of every lane, strip by strip
+    int steps[kSlicedWaves];      // longest task of each strip
     int64_t real_entries;
   };
   std::vector<SlicedWorkgroup> wgs((size_t)n_wg);
@@ -287,16 +356,13 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
   const char* spread_env = getenv("NPAMD_SLICED_SPREAD");
   const bool spread = !(spread_env && *spread_env == '0');
   parallel_for(n_wg, [&](int w) {
-    std::vector<std::vector<uint32_t>> task((size_t)geo.rows_per_block);
-    std::vector<int> order;
     Built& b = built[(size_t)w];
     const Job& job = jobs[w];
     SlicedWorkgroup& wg = wgs[w];
-    const int range_groups = (G + geo.parts[job.slice] - 1) / geo.parts[job.slice];
-    const int g_begin = job.part * range_groups;
-    const int g_end = std::min(G, g_begin + range_groups);
-    const int row0 = job.block * geo.rows_per_block;
-    const int rows = std::max(0, std::min(geo.rows_per_block, N - row0));
+    const int g_begin = job.part * range_groups[(size_t)job.slice];
+    const int g_end = std::min(G, g_begin + range_groups[(size_t)job.slice]);
+    const int row0 = job.block * rpb;
+    const int rows = std::max(0, std::min(rpb, N - row0));
     wg.slice = (uint32_t)job.slice;
     wg.partial = (uint32_t)(partial_base[job.slice] + job.part);
     wg.g_begin = (uint32_t)g_begin;
@@ -305,39 +371,25 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
     wg.row_count = (uint32_t)rows;
     wg.reserved[0] = wg.reserved[1] = 0;
 
-    for (int g = g_begin; g < g_end; ++g) {
-      const uint32_t* col = &idx_t[(size_t)g * N + row0];
-      for (int r = 0; r < rows; ++r) {
-        const uint32_t v = col[r];
-        if ((int)(v / slice_rows) == job.slice)
-          task[(size_t)r].push_back((v % slice_rows) | ((uint32_t)(g - g_begin) << 16));
-      }
-    }
+    const uint32_t* len = &task_len[(size_t)w * rpb];
     // Longest tasks first; 64 neighbours in that order share a strip.
-    order.resize((size_t)rows);
-    std::iota(order.begin(), order.end(), 0);
-    std::stable_sort(order.begin(), order.end(),
-                     [&](int a, int c) { return task[(size_t)a].size() > task[(size_t)c].size(); });
+    b.order.resize((size_t)rows);
+    std::iota(b.order.begin(), b.order.end(), (uint16_t)0);
+    std::stable_sort(b.order.begin(), b.order.end(), [&](uint16_t a, uint16_t c) { return len[a] > len[c]; });
     b.real_entries = 0;
     for (int s = 0; s < kSlicedWaves; ++s) {
       const int first = s * 64;
       const int lanes = std::max(0, std::min(64, rows - first));
-      b.steps[s] = lanes ? (int)task[(size_t)order[(size_t)first]].size() : 0;
-      if (spread && lanes) {
-        std::vector<uint32_t>* strip_tasks[64];
-        for (int lane = 0; lane < lanes; ++lane) strip_tasks[lane] = &task[(size_t)order[(size_t)(first + lane)]];
-        spread_bank_groups(strip_tasks, lanes, b.steps[s]);
-      }
-      for (int lane = 0; lane < 64; ++lane) {
-        b.begin[first + lane] = (uint32_t)b.entries.size();
-        if (lane >= lanes) continue;
-        const int r = order[(size_t)(first + lane)];
+      b.steps[s] = lanes ? (int)len[b.order[(size_t)first]] : 0;
+      TaskSpan strip_tasks[64];
+      for (int lane = 0; lane < lanes; ++lane) {
+        const int r = b.order[(size_t)(first + lane)];
+        strip_tasks[lane] = TaskSpan{&entries[(size_t)task_begin[(size_t)w * rpb + r]], len[r]};
         rowmap[(size_t)w * kSlicedTasks + (size_t)first + lane] = (uint32_t)(row0 + r);
-        b.entries.insert(b.entries.end(), task[(size_t)r].begin(), task[(size_t)r].end());
+        b.real_entries += len[r];
       }
+      if (spread && lanes) spread_bank_groups(strip_tasks, lanes, b.steps[s]);
     }
-    b.begin[kSlicedTasks] = (uint32_t)b.entries.size();
-    b.real_entries = (int64_t)b.entries.size();
   });
 
   // Strip w of every workgroup gets the length of the layer's longest strip w.
@@ -400,8 +452,11 @@ extern "C" int npamd_vq_sliced_build(const uint8_t* packed, int64_t n_bytes, int
       uint8_t* strip = wg_out + wave_begin[s] * kSlicedQuadBytes;
       const int64_t slots = 4 * (int64_t)wave_quads[s];
       for (int lane = 0; lane < 64; ++lane) {
-        const uint32_t* e = b.entries.data() + b.begin[s * 64 + lane];
-        const int64_t len = (int64_t)b.begin[s * 64 + lane + 1] - (int64_t)b.begin[s * 64 + lane];
+        const size_t pos = (size_t)s * 64 + lane;
+        const bool real = pos < b.order.size();
+        const size_t task = real ? (size_t)w * rpb + b.order[pos] : 0;
+        const uint32_t* e = real ? &entries[(size_t)task_begin[task]] : nullptr;
+        const int64_t len = real ? (int64_t)task_len[task] : 0;
         for (int64_t i = 0; i < slots; ++i)
           put_entry(strip + (size_t)(i / 4) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4), i < len ? e[i] : pad);
       }
@@ -444,15 +499,26 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
   const int G = h.k / 8;
   std::vector<uint8_t> covered((size_t)h.n_partials * (size_t)h.n, 0);
   std::vector<uint8_t> filed((size_t)h.n * (size_t)G, 0);
-  for (int w = 0; w < h.n_workgroups; ++w) {
+  // One workgroup per work item; the first violation found (lowest workgroup) is the one reported.
+  std::vector<std::string> errors((size_t)h.n_workgroups);
+#define WG_REQUIRE(cond, ...)                          \
+  do {                                                 \
+    if (!(cond)) {                                     \
+      char msg[256];                                   \
+      snprintf(msg, sizeof(msg), __VA_ARGS__);         \
+      errors[(size_t)w] = msg;                         \
+      return;                                          \
+    }                                                  \
+  } while (0)
+  parallel_for(h.n_workgroups, [&](int w) {
     const SlicedWorkgroup& wg = wgs[w];
-    NPAMD_REQUIRE(wg.slice < (uint32_t)h.n_slices && wg.partial < (uint32_t)h.n_partials,
+    WG_REQUIRE(wg.slice < (uint32_t)h.n_slices && wg.partial < (uint32_t)h.n_partials,
                   "%s: workgroup %d: slice/partial out of range", what, w);
     if (h.flags & kSlicedRoundRobin) {
       // What the kernel computes instead of reading the record.
       const int parts = h.n_partials / h.n_slices;
       const int row_blocks = parts ? h.n_workgroups / (parts * h.n_slices) : 0;
-      NPAMD_REQUIRE(parts >= 1 && row_blocks >= 1 && parts * h.n_slices == h.n_partials &&
+      WG_REQUIRE(parts >= 1 && row_blocks >= 1 && parts * h.n_slices == h.n_partials &&
                         row_blocks * h.n_partials == h.n_workgroups,
                     "%s: counts do not form the regular geometry the header states", what);
       const int range_groups = (G + parts - 1) / parts;
@@ -460,16 +526,16 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
       const uint32_t part = (uint32_t)((w / h.n_slices) / row_blocks);
       const int block = (w / h.n_slices) % row_blocks;
       const int row_begin = std::min(block * rows_per_block, h.n);
-      NPAMD_REQUIRE(wg.slice == (uint32_t)(w % h.n_slices) && wg.partial == wg.slice * (uint32_t)parts + part &&
+      WG_REQUIRE(wg.slice == (uint32_t)(w % h.n_slices) && wg.partial == wg.slice * (uint32_t)parts + part &&
                         wg.g_begin == part * (uint32_t)range_groups &&
                         wg.g_count == (uint32_t)std::min(range_groups, G - (int)wg.g_begin) &&
                         wg.row_begin == (uint32_t)row_begin &&
                         wg.row_count == (uint32_t)std::max(0, std::min(rows_per_block, h.n - row_begin)),
                     "%s: workgroup %d does not follow the regular geometry the header states", what, w);
     }
-    NPAMD_REQUIRE(wg.g_count >= 1 && wg.g_count <= (uint32_t)h.groups_max && (int64_t)wg.g_begin + wg.g_count <= G,
+    WG_REQUIRE(wg.g_count >= 1 && wg.g_count <= (uint32_t)h.groups_max && (int64_t)wg.g_begin + wg.g_count <= G,
                   "%s: workgroup %d: group range out of bounds", what, w);
-    NPAMD_REQUIRE(wg.row_count <= (uint32_t)kSlicedTasks && (int64_t)wg.row_begin + wg.row_count <= h.n,
+    WG_REQUIRE(wg.row_count <= (uint32_t)kSlicedTasks && (int64_t)wg.row_begin + wg.row_count <= h.n,
                   "%s: workgroup %d: row block out of bounds", what, w);
     const uint32_t slice_len = (uint32_t)std::min(h.slice_rows, h.nc - (int)wg.slice * h.slice_rows);
     for (int s = 0; s < kSlicedWaves; ++s) {
@@ -477,28 +543,28 @@ extern "C" int npamd_vq_sliced_check(const void* blob, int64_t blob_bytes) {
       const int64_t quad_begin = (int64_t)w * wg_quads + wave_begin[s];
       for (int lane = 0; lane < 64; ++lane) {
         const uint32_t row = rowmap[(size_t)w * kSlicedTasks + (size_t)s * 64 + lane];
-        NPAMD_REQUIRE(row == kSlicedNoRow || (row >= wg.row_begin && row - wg.row_begin < wg.row_count),
+        WG_REQUIRE(row == kSlicedNoRow || (row >= wg.row_begin && row - wg.row_begin < wg.row_count),
                       "%s: workgroup %d: row outside the workgroup's row block", what, w);
         if (row != kSlicedNoRow) {
-          uint8_t& c = covered[(size_t)wg.partial * h.n + row];
-          NPAMD_REQUIRE(c == 0, "%s: partial %u row %u written twice", what, wg.partial, row);
-          c = 1;
+          const uint8_t seen = __atomic_fetch_add(&covered[(size_t)wg.partial * h.n + row], (uint8_t)1, __ATOMIC_RELAXED);
+          WG_REQUIRE(seen == 0, "%s: partial %u row %u written twice", what, wg.partial, row);
         }
         for (int64_t i = 0; i < nq * 4; ++i) {
           const uint32_t e = get_entry(quads + ((size_t)quad_begin + (size_t)(i / 4)) * kSlicedQuadBytes + (size_t)lane * 12, (int)(i % 4));
           const uint32_t local = e & 0xFFFFu, g_local = e >> 16;
-          NPAMD_REQUIRE(g_local < wg.g_count && (local < slice_len || local == (uint32_t)kSlicedPadRow),
+          WG_REQUIRE(g_local < wg.g_count && (local < slice_len || local == (uint32_t)kSlicedPadRow),
                         "%s: workgroup %d: entry field out of range", what, w);
           if (local != (uint32_t)kSlicedPadRow) {
-            NPAMD_REQUIRE(row != kSlicedNoRow, "%s: workgroup %d: live entry in a lane without a row", what, w);
-            uint8_t& f = filed[(size_t)row * G + wg.g_begin + g_local];
-            NPAMD_REQUIRE(f == 0, "%s: index (%u, %u) filed twice", what, row, wg.g_begin + g_local);
-            f = 1;
+            WG_REQUIRE(row != kSlicedNoRow, "%s: workgroup %d: live entry in a lane without a row", what, w);
+            const uint8_t seen = __atomic_fetch_add(&filed[(size_t)row * G + wg.g_begin + g_local], (uint8_t)1, __ATOMIC_RELAXED);
+            WG_REQUIRE(seen == 0, "%s: index (%u, %u) filed twice", what, row, wg.g_begin + g_local);
           }
         }
       }
     }
-  }
+  });
+#undef WG_REQUIRE
+  for (const std::string& e : errors) NPAMD_REQUIRE(e.empty(), "%s", e.c_str());
   for (uint8_t c : covered) NPAMD_REQUIRE(c == 1, "%s: some (partial, row) pair is never written", what);
   for (uint8_t f : filed) NPAMD_REQUIRE(f == 1, "%s: some index is not filed", what);
   NPAMD_REQUIRE(h.n_entries == (int64_t)h.n * G, "%s: entry count in the header is wrong", what);
