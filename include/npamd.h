@@ -245,8 +245,10 @@ int npamd_vq_gemv_sliced(const void* x, int64_t ldx, const int32_t* column_perm,
  * npamd_vq_sliced_workspace_bytes() exceeds the array are rejected with NPAMD_ERR_INVALID.
  * All calls on one GPU share the array: it starts zero-filled and every call hands it back
  * zero-filled, so calls that follow each other (on one stream, or ordered by events) are
- * fine, and calls that overlap on one GPU race.  Same arguments and results as
- * npamd_vq_gemv_sliced otherwise.
+ * fine, and calls that overlap on one GPU race.  A call that returns an error after it may have
+ * launched part of its work leaves the array suspect; the next call on that GPU zero-fills it
+ * (a kernel on the caller's stream, not a memset) before it uses it.  Same arguments and results
+ * as npamd_vq_gemv_sliced otherwise.
  */
 #define NPAMD_SLICED_STATIC_WORKSPACE_BYTES (4 * 1024 * 1024)
 int npamd_vq_gemv_sliced_static(const void* x, int64_t ldx, const int32_t* column_perm,

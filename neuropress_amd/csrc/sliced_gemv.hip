@@ -542,6 +542,15 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex scratch_mutex;
 void* scratch_of_device[kMaxDevices];  // the device address of `scratch`, per device (null: not looked up yet)
+bool scratch_suspect[kMaxDevices];     // a call on this device failed after it may have launched: zero before the next use
+
+// The kernels count on a zero-filled workspace and hand it back zero-filled; a call that fails between
+// two of its launches (more than seven tokens) cannot promise that.  A fill kernel, not a memset: the
+// caller may be capturing a graph.
+__global__ void __launch_bounds__(256) scratch_zero_kernel(u32x4* p, int n16) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) p[i] = u32x4{0u, 0u, 0u, 0u};
+}
 }  // namespace
 
 extern "C" int npamd_vq_gemv_sliced_static(const void* x, int64_t ldx, const int32_t* column_perm,
@@ -572,6 +581,18 @@ extern "C" int npamd_vq_gemv_sliced_static(const void* x, int64_t ldx, const int
       scratch_of_device[device] = ptr;
     }
     workspace = scratch_of_device[device];
+    if (scratch_suspect[device]) {
+      constexpr int n16 = NPAMD_SLICED_STATIC_WORKSPACE_BYTES / 16;
+      scratch_zero_kernel<<<(n16 + 255) / 256, 256, 0, (hipStream_t)stream>>>((u32x4*)workspace, n16);
+      const int zrc = check_launch(what);
+      if (zrc != NPAMD_OK) return zrc;
+      scratch_suspect[device] = false;
+    }
   }
-  return run_sliced(what, x, ldx, column_perm, *hp, blob, codebook, bias, y, ldy, M, act_dtype, workspace, stream);
+  const int run_rc = run_sliced(what, x, ldx, column_perm, *hp, blob, codebook, bias, y, ldy, M, act_dtype, workspace, stream);
+  if (run_rc != NPAMD_OK) {
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    scratch_suspect[device] = true;
+  }
+  return run_rc;
 }
