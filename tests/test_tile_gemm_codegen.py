@@ -133,3 +133,43 @@ def test_the_wide_kernel_loads_everything_into_lds_and_leaves_m0_to_its_transfer
                 spills += 1
         assert transfers >= 10, (name, transfers)
         assert spills == 0, (name, spills)  # 512 registers per lane hold the wave tile: nothing goes to scratch
+
+
+@pytest.fixture(scope="module")
+def assembly_gemv(tmp_path_factory):
+    """The gfx950 assembly of the fused decode GEMV (csrc/vq_gemv.hip)."""
+    if shutil.which("hipcc") is None and not build.Path("/opt/rocm/bin/hipcc").exists():
+        pytest.skip("needs hipcc")
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    out = tmp_path_factory.mktemp("codegen") / "vq_gemv.s"
+    cmd = [hipcc, *build.CXXFLAGS, *build.DEVICE_FLAGS, "-S", "--cuda-device-only",
+           str(build.CSRC / "vq_gemv.hip"), "-o", str(out)]  # fmt: skip
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    return out.read_text().split("\n")
+
+
+def test_the_gemv_leaves_m0_to_its_codebook_copy(assembly_gemv):
+    """``fused_gemv_kernel`` copies a codebook into LDS with ``s_mov_b32 m0, ...;
+    global_load_lds_dwordx4`` statements and waits for them with ``s_waitcnt vmcnt(0)`` inside the same
+    asm block sequence; nothing else in the kernels may name m0."""
+    lines = assembly_gemv
+    starts = [i for i, ln in enumerate(lines) if re.match(r"^_ZN5npamd17fused_gemv_kernel\S*: ;", ln)]
+    assert len(starts) >= 50
+    with_copy = 0
+    for i in starts:
+        name = lines[i].split(":")[0]
+        end = next(j for j in range(i, len(lines)) if lines[j].startswith(".Lfunc_end"))
+        in_asm, transfers = False, 0
+        for ln in lines[i:end]:
+            code = ln.split(";")[0]
+            if "#ASMSTART" in ln:
+                in_asm = True
+            elif "#ASMEND" in ln:
+                in_asm = False
+            elif re.search(r"\bm0\b", code):
+                assert in_asm, (name, ln)
+            if in_asm and "global_load_lds_dwordx4" in code:
+                transfers += 1
+        with_copy += transfers > 0
+    assert with_copy >= 20  # the variants that keep a table in LDS
