@@ -86,6 +86,7 @@ struct KWalk {
 struct WaveCtx {
   int wave, lane, c, h;
   int ncol;            // the lane's weight row, clamped to N - 1
+  int n_first, n_last; // the wave's first weight row (may lie past N - 1), and N - 1
   uint8_t* ws;         // W slots, kWRing x 16 KiB
   uint32_t ws_lds;     // the same as an LDS address
   uint8_t* stage;      // the block's staging area
@@ -101,46 +102,76 @@ template <int ACT>
 struct T2ProdVq16 {
   using Args = T2Args;
   static constexpr int kWRing = 3;
-  static constexpr int kLoads = 5;                 // per step: four gathers, one index load
-  static constexpr bool kLoadsLast = true;         // ... issued behind the step's x pieces, in k group 3
-  static constexpr int kStageBytes = 4 * 2 * 1024;  // per wave two staged chunks of 64 lanes x 16 bytes
+  static constexpr int kLoads = 4;                 // per step: four gathers ...
+  static constexpr int kQuadLoads = 2;             // ... and, every fourth step, two index loads behind them
+  static constexpr bool kLoadsLast = true;         // issued behind the step's x pieces, in k group 3
+  // Indices are staged four steps at a time: a column's 64 bytes of a quad of steps are half a cache
+  // line, and one load instruction fetches them for sixteen columns (16 lines; a load of one
+  // step's 16 bytes for 32 columns touches 32 lines, and the address unit's time goes with the
+  // lines).  Per wave two quads of 32 columns x 64 bytes; piece p of column r sits in slot
+  // p ^ ((r >> 2) & 3) of its row, which spreads the 8-byte reads of 32 columns over the banks.
+  static constexpr int kQuadBytes = 32 * 64;
+  static constexpr int kStageBytes = 4 * 2 * kQuadBytes;
   const Args& a;
   const KWalk& kw;
   const WaveCtx& w;
-  uint32_t idx_row_off;
-  __device__ T2ProdVq16(const Args& args, const KWalk& walk, const WaveCtx& ctx)
-      : a(args), kw(walk), w(ctx), idx_row_off((uint32_t)ctx.ncol * (uint32_t)args.chunks * 16u) {}
-  __device__ __forceinline__ void load_idx(int step, int par) const {
-    lds_load16(w.stage_lds + (uint32_t)((w.wave * 2 + par) * 1024), idx_row_off + (uint32_t)kw.chunk_of(step) * 16u, a.packed);
+  uint32_t row_off[2];  // byte offset of the index rows this lane fetches (columns lane / 4 and 16 + lane / 4 of the wave)
+  int piece;            // which of a quad's four steps the lane fetches for those columns
+  __device__ T2ProdVq16(const Args& args, const KWalk& walk, const WaveCtx& ctx) : a(args), kw(walk), w(ctx) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = 16 * i + (ctx.lane >> 2);
+      const int n = min(ctx.n_first + r, ctx.n_last);  // columns past N fetch a valid row nobody stores
+      row_off[i] = (uint32_t)n * (uint32_t)args.chunks * 16u;
+    }
+    piece = (ctx.lane & 3) ^ ((ctx.lane >> 4) & 3);  // slot ^ ((r >> 2) & 3), r = 16 i + lane / 4
   }
-  __device__ __forceinline__ void gathers(int par, int slot) const {
-    const u32x2 v = *reinterpret_cast<const u32x2*>(w.stage + (w.wave * 2 + par) * 1024 + w.lane * 16 + w.h * 8);
+  // Steps 4 quad .. 4 quad + 3 of the wave's 32 columns into staging slot quad % 2.
+  __device__ __forceinline__ void load_quad(int quad) const {
+    const uint32_t chunk = (uint32_t)kw.chunk_of(4 * quad + piece) * 16u;
+    const uint32_t dst = w.stage_lds + (uint32_t)((w.wave * 2 + (quad & 1)) * kQuadBytes);
+    lds_load16(dst, row_off[0] + chunk, a.packed);
+    lds_load16(dst + 1024u, row_off[1] + chunk, a.packed);
+  }
+  // The lookups of step `step` into W slot `slot`, from the staged indices.
+  __device__ __forceinline__ void gathers(int step, int slot) const {
+    const int q = step >> 2, p = step & 3;
+    const u32x2 v = *reinterpret_cast<const u32x2*>(w.stage + (w.wave * 2 + (q & 1)) * kQuadBytes + w.c * 64 +
+                                                    ((p ^ ((w.c >> 2) & 3)) << 4) + w.h * 8);
     const uint32_t off[4] = {(uint32_t)(min(v.x & 0xFFFFu, a.nc_minus_1) << 4), (uint32_t)(min(v.x >> 16, a.nc_minus_1) << 4),
                              (uint32_t)(min(v.y & 0xFFFFu, a.nc_minus_1) << 4), (uint32_t)(min(v.y >> 16, a.nc_minus_1) << 4)};
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       lds_load16(w.ws_lds + (uint32_t)(slot * kT2WSlotBytes + (w.wave * 4 + j) * 1024), off[j], a.cb);
   }
-  // Before the loop: W tiles of steps 0 and 1 requested, indices of steps 2 and 3 requested.
+  // Before the loop: the indices of steps 0 .. 7 staged, the W tiles of steps 0 and 1 requested.
   __device__ __forceinline__ void prologue_issue() const {
-    load_idx(0, 0);
-    load_idx(1, 1);
+    load_quad(0);
+    load_quad(1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     gathers(0, 0);
     gathers(1, 1);
-    load_idx(2, 0);
-    load_idx(3, 1);
   }
   __device__ __forceinline__ void prologue_finish() const {}
+  // In step t the wave looks up the rows of step t + 2 (W ring of three); after the lookups of
+  // t = 4 q + 2, which read quad q + 1, quad q's slot is free (its last reader was step 4 q + 1) and
+  // takes quad q + 2, first read in step 4 q + 6.
+  __device__ __forceinline__ bool loads_quad(int step) const { return (step & 3) == 2; }
   // Work behind the MFMAs of k group J, column tile T of step `step` (W slot wslot = step % 3).
   template <int J, int T>
   __device__ __forceinline__ void work(int step, int wslot) const {
-    if (J == 0 && T == 0) gathers(step & 1, wslot == 0 ? 2 : wslot - 1);
-    if (J == 0 && T == 1) load_idx(step + 4, step & 1);
+    if (J == 0 && T == 0) gathers(step + 2, wslot == 0 ? 2 : wslot - 1);
+    if (J == 0 && T == 1 && loads_quad(step)) load_quad((step >> 2) + 2);
   }
   __device__ __forceinline__ void work_all(int step, int wslot) const {
     work<0, 0>(step, wslot);
     work<0, 1>(step, wslot);
+  }
+  // Wait until everything but the loads this step issued last (its lookups, and the index quads
+  // behind them in the steps that fetch one) has landed.
+  __device__ __forceinline__ void wait_all_but_own(int step) const {
+    if (loads_quad(step)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads + kQuadLoads) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
   }
 };
 
@@ -293,6 +324,8 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
   wc.c = c;
   wc.h = h;
   wc.ncol = min(n0 + 32 * wave + c, s.N - 1);  // columns past N decode a valid row nobody stores
+  wc.n_first = n0 + 32 * wave;
+  wc.n_last = s.N - 1;
   wc.ws = ws;
   wc.ws_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)ws;
   wc.stage = stage;
@@ -388,7 +421,8 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
         }
       }
       // Everything but a producer's lookups of this step has to be there when the next step starts.
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(Prod::kLoadsLast ? kProdLoads : 0) : "memory");
+      if constexpr (Prod::kLoadsLast && !(ABL & 1)) prod.wait_all_but_own(step);
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       block_sync_lds();
     };
     int wslot = 0;
@@ -406,7 +440,8 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
     int wslot = 0;
     for (int t = 0; t < steps; ++t) {
       if (!(ABL & 1)) prod.work_all(t, wslot);
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kProdLoads) : "memory");
+      if constexpr (Prod::kLoadsLast && !(ABL & 1)) prod.wait_all_but_own(t);
+      else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kProdLoads) : "memory");
       block_sync_lds();
       wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
     }
