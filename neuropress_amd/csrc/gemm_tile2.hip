@@ -256,23 +256,26 @@ struct T2ProdQ {
     decode<1>(0);
     decode<2>(0);
     decode<3>(0);
+    fetch(1);
   }
   template <int J, int T>
   __device__ __forceinline__ void work(int step, int wslot) {
     if (J == 0 && T == 0) request(step + 3);
-    if (J == 0 && T == 1) fetch(step + 1);
     if (J == 0 && T == 2) decode<0>(wslot ^ 1);
     if (J == 0 && T == 3) decode<1>(wslot ^ 1);
     if (J == 1 && T == 0) decode<2>(wslot ^ 1);
     if (J == 1 && T == 1) decode<3>(wslot ^ 1);
+    // The bytes the next step decodes are read out of the staging ring a k group and a barrier ahead
+    // of their first use, so that the decoding never waits for LDS.
+    if (J == 3 && T == 3) fetch(step + 2);
   }
   __device__ __forceinline__ void work_all(int step, int wslot) {
     request(step + 3);
-    fetch(step + 1);
     decode<0>(wslot ^ 1);
     decode<1>(wslot ^ 1);
     decode<2>(wslot ^ 1);
     decode<3>(wslot ^ 1);
+    fetch(step + 2);
   }
 };
 
@@ -299,7 +302,6 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
   constexpr int kXBufBytes = T2Lds<MW, Prod>::kXBufBytes;
   constexpr int kPieces = 4 * MW;  // x-tile load instructions per wave and step (8 rows each)
   constexpr int kWRing = Prod::kWRing;
-  constexpr int kProdLoads = (ABL & 1) ? 0 : Prod::kLoads;
   uint8_t* const xs = lds;                              // [2][BM][128]
   uint8_t* const ws = lds + 2 * kXBufBytes;             // [kWRing][16 KiB]
   uint8_t* const stage = ws + kWRing * kT2WSlotBytes;   // the producer's staging area
@@ -414,6 +416,7 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
               if (j == 0 && t == 3) prod.template work<0, 3>(step, wslot);
               if (j == 1 && t == 0) prod.template work<1, 0>(step, wslot);
               if (j == 1 && t == 1) prod.template work<1, 1>(step, wslot);
+              if (j == 3 && t == 3) prod.template work<3, 3>(step, wslot);
             }
           }
           if (j * 4 + t < kPieces) fetch_piece(j * 4 + t, buf ^ 1, src);
@@ -441,7 +444,7 @@ tile2_gemm_kernel(const GemmShape s, const typename Prod::Args pargs, const T2Pa
     for (int t = 0; t < steps; ++t) {
       if (!(ABL & 1)) prod.work_all(t, wslot);
       if constexpr (Prod::kLoadsLast && !(ABL & 1)) prod.wait_all_but_own(t);
-      else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kProdLoads) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // as the waves with rows do
       block_sync_lds();
       wslot = wslot == kWRing - 1 ? 0 : wslot + 1;
     }
