@@ -1,40 +1,45 @@
-// Tile-decode GEMM, 128-column blocks: y = x @ W^T (+ bias) for VQ weights with 16-bit indices into a
-// codebook too large for LDS (more than 4096 rows), wave64 + MFMA 32x32x16, f32 accumulate.
+// Tile-decode GEMM, 128-column blocks: y = x @ W^T (+ bias), wave64 + MFMA 32x32x16, f32 accumulate, for VQ
+// weights with 16-bit indices into a codebook too large for LDS (more than 4096 rows) and for int4 /
+// int8 group-affine codes.
 //
 // Why a second block shape.  A block's x tile (BM rows x 64 k) passes the compute unit's vector
-// memory path once per 64-k step whatever the block's width, and that path moves 64 bytes per
-// cycle: with 64 columns it is busy with x as long as the matrix pipe is busy with the MFMAs, on
-// top of the codebook lookups that go the same way.  128 columns halve the x bytes per MFMA.
+// memory path once per 64-k step whatever the block's width, and every 128-byte line of it is a
+// request to the L2, like every codebook lookup: with 64 columns the x tile costs as many L2 requests
+// per weight as two lookups in three.  128 columns halve the x requests per MFMA.
 //
-// Block = 4 waves, one per SIMD, each with the whole register file of its SIMD (512 registers:
-// 192 accumulators for a 96 x 128 tile and two operand sets).  There are no producer waves:
-// every weight operand is one codebook row, so the decode is a gather, and the gather is issued
-// as a load that writes LDS directly (global_load_lds_dwordx4, one row per lane, 64 rows = one KiB
-// per instruction) -- no register, no LDS store instruction, no arithmetic.  The codebook the
-// caller passes is already in the activation dtype.
+// Block = 8 waves, two per SIMD.  Waves w and w + 4 own rows [32 MW (w % 4), 32 MW (w % 4 + 1)) of the
+// block tile and 64 of the 128 columns each: 2 MW accumulator tiles of 32 x 32 per wave.  There are no
+// producer waves; every job of a step is dealt over all eight, and whenever the address unit makes
+// one wave wait at a load, the other wave of its SIMD has MFMAs to issue.  Everything the kernel
+// loads lands in LDS by itself (global_load_lds_dwordx4 / _dword: no register, no LDS store
+// instruction): the x tile (rows of 128 bytes, piece p of row r in slot p ^ ((r >> 1) & 7)), the
+// staged indices or packed bytes, and for VQ the weights themselves -- a lookup is a transfer from
+// codebook + 16 index straight into the W slot the MFMAs read (the codebook the caller passes is
+// already in the activation dtype).
 //
 // Roles of wave w in every 64-k step t:
-//   MFMA:    rows [32 MW w, 32 MW (w + 1)) of the block tile x all 128 columns.
-//   x tile:  its own rows of step t + 2, loaded straight into LDS (swizzled 128-byte rows) into
-//            the buffer of step t as soon as the last operands of step t are in registers; no
-//            other wave reads those rows, so the x tile needs no barrier.
-//   W tile:  columns [32 w, 32 w + 32) of step t + 2: lane (c = l % 32, h = l / 32) reads the four
-//            indices 4h .. 4h+3 of its column's chunk from an LDS staging area of the wave (the
-//            16 bytes of a chunk were loaded there, also directly, in step t - 2) and issues four
-//            gathers; gather j lands in position l of KiB (w, j) of W slot (t + 2) % 3, which is
-//            exactly where lane l looks for B operand j of column tile w: MFMA j of a step
-//            contracts k = 64 t + 32 h + 8 j .. + 7, x and W alike.
-// All loads of a wave complete in order, and everything it requests in step t is due at the end
-// of step t + 1 (the W slot and the x buffer of step t + 2, the indices for the gathers of step
-// t + 3): one `s_waitcnt vmcnt(loads of one step)` in front of the step's only barrier.
+//   MFMA:    4 k groups x 2 column tiles x MW row tiles; the operands of k group j + 1 are read
+//            from LDS before the MFMAs of k group j.
+//   x tile:  pieces (8 rows x 128 bytes) 2 i + w / 4 of its row group, of step t + 1, into the
+//            buffer that is not being read, one piece behind each of the first 2 MW MFMA slots.
+//   W tile:  column tile w % 4, operand pair J = w / 4.  VQ: lane (c = l % 32, h = l / 32) reads its
+//            two indices of step t + 2 from the staged indices and issues two lookups; lookup j
+//            lands in position l of KiB (w % 4, j) of W slot (t + 2) % 3, which is where lane l looks
+//            for B operand j of column tile w % 4: MFMA j of a step contracts k = 64 t + 32 h + 8 j
+//            .. + 7, x and W alike.  int4 / int8: the producers' arithmetic between the MFMAs.
+// All loads of a wave complete in order and the waits are written by hand (s_waitcnt vmcnt(n) with
+// the number of younger loads that may stay in flight): everything a wave requests in step t is due
+// at the end of step t + 1 at the latest, in front of the step's only barrier.  The last two steps
+// are instantiated apart: nothing is looked up or fetched for steps past the end.
 //
 // K is split in two (blockIdx.z) when the column blocks alone leave compute units idle:
-// 14336 columns are 112 blocks of 128, so 224 workgroups each contract half of K.  The halves
-// meet without a second kernel and without spinning: whichever workgroup of a pair finishes
-// first stores its f32 tile to the workspace and counts itself in; the other adds that tile to
-// its registers, adds the bias and stores y.  Two addends commute, so the result does not
-// depend on which half was first.  More than two splits (layers of few columns) store partial
-// tiles for splitk_reduce_kernel as the 64-column kernel does.
+// 14336 columns are 112 blocks of 128, so 224 workgroups each contract half of K, the first halves
+// on four of the GPU's dies and the second halves on the other four (a die's L2 then holds half of
+// x).  The halves meet without a second kernel and without spinning: whichever workgroup of a
+// pair finishes first stores its f32 tile to the workspace and swaps the call's number into the
+// tile's word; the other adds that tile to its registers, adds the bias and stores y.  Two addends
+// commute, so the result does not depend on which half was first.  More than two splits (layers
+// of few columns) store partial tiles for splitk_reduce_kernel as the 64-column kernel does.
 #pragma once
 
 #include "gemm_tile.hpp"
@@ -60,9 +65,8 @@ struct T2QArgs {
   const uint16_t* zp;     // null: symmetric
 };
 
-// K in two halves: one arrival counter per block tile (zeroed by a fill kernel in front of the GEMM,
-// zero again on exit) and the f32 tile of whichever half finished first, [2][tiles][BM * 128] in
-// register order.
+// K in two halves: one word per block tile and the f32 tile of whichever half finished first,
+// [2][tiles][BM * 128] in register order.
 struct T2Pair {
   unsigned long long* words;  // one per tile: holds `call` while one half of the tile has arrived in this call
   float* tiles;

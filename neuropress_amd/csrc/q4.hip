@@ -658,10 +658,13 @@ static int q8_fused(const QCall& c, bool gemv) {
 // The 128-column tile GEMM (gemm_tile2.hpp) for int4 / int8: 0 when it took the call.
 static int q_tile_wide(const QCall& c) {
   const int mode = tile2_mode();
-  // Measured against the 64-column kernel, int4, us: 14336 x 4096 at 128 / 256 / 384 / 512 / 1024 tokens 36.7 / 53.5 /
-  // 67.7 / 77.2 / 155 against 37.0 / 52.5 / 75.2 / 113 / 193; 4096 x 14336 38.6 / 55.1 / 72.8 / 83.8 / 143 against
-  // 40.7 / 59.9 / 79.7 / 118 / 200; 4096 x 4096 behind at every count (more than two splits of K).
-  const bool wins = (c.K >= 8192 && c.M >= 128) || (c.N >= 8192 && c.M > 256);
+  // Measured against the 64-column kernel, int4, us at 17 / 128 / 256 / 384 / 512 tokens: 14336 x 4096 26.7 / 32.7 /
+  // 46.9 / 62.4 / 80.1 against 27.5 / 35.0 / 50.1 / 77.4 / 116; 6144 x 4096 17.9 / 26.2 / 33.9 / 49.0 / 45.4 against 20.3 /
+  // 26.4 / 35.9 / 50.9 / 66.0; 4096 x 14336 30.8 / 40.3 / 54.0 / 69.5 / 83.9 against 29.8 / 38.9 / 59.9 / 82.0 / 121 (ahead
+  // from 192 tokens: 47.4 against 51.0); 4096 x 4096 16.5 / 25.2 / 29.7 / 39.8 / 39.2 against 16.7 / 22.7 / 29.0 / 38.8 /
+  // 50.6; 8192 x 2048 14.4 / 24.2 / 31.3 / 42.8 / 31.1 against 15.7 / 22.8 / 30.9 / 40.0 / 38.6.
+  const int64_t weights = (int64_t)c.N * c.K;
+  const bool wins = (c.N >= 6144 && c.K >= 4096) || (weights >= ((int64_t)1 << 25) && c.M > 128) || c.M > 384;
   if (!(mode >= 2 || (mode == 1 && wins))) return 1;
   if (!ptr_aligned(c.scale, 4) || (c.zp && !ptr_aligned(c.zp, 4)) || (int64_t)c.N * c.K >= ((int64_t)1 << 32)) return 1;
   const GemmShape s{c.x, c.ldx, c.bias, c.y, c.ldy, c.M, c.N, c.K, c.K / 64, 0};

@@ -19,12 +19,12 @@ int run_vq(const VqCall& c, const GemmShape& s) {
     // Codebooks LDS does not hold, in the activation dtype: the 128-column kernel, whose gathers write LDS directly.
     const int mode = tile2_mode();
     const bool big = (int64_t)c.nc * 16 > kTileLdsCodebookMax;
-    // Measured against the 64-column kernel on 65536-row codebooks, 17 / 384 tokens (us): ahead on 11008 x 4096
-    // (37.6 / 63.3 against 40.7 / 73.6), 14336 x 4096 (44.4 / 70.2 against 47.1 / 80.2), 4096 x 14336 (46.3 / 76.4
-    // against 48.0 / 87.0), 8192 x 8192 (49.1 / 88.4 against 52.7 / 104.5), 28672 x 4096 (76.9 / 116 against 85.4 /
-    // 160); level or behind on 6144 x 4096 (26.8 / 56.8 against 27.8 / 54.0), 4096 x 4096 (23.0 / 43.3 against
-    // 23.6 / 40.6), 2048 x 8192 and 8192 x 2048: from 2^25 weights.
-    const bool wins = big && (int64_t)c.N * c.K >= ((int64_t)1 << 25);
+    // Measured against the 64-column kernel on 65536-row codebooks, 17 / 384 tokens (us): 14336 x 4096 40.8 / 66.6
+    // against 48.9 / 86.0, 4096 x 14336 42.8 / 75.8 against 49.5 / 92.0, 8192 x 8192 44.8 / 88.5 against 53.2 / 108,
+    // 28672 x 4096 72.3 / 112 against 84.4 / 157, 6144 x 4096 23.6 / 54.9 against 29.1 / 57.7, 4096 x 4096 20.4 / 41.6
+    // against 24.6 / 43.7, 2048 x 8192 23.8 / 43.4 against 26.4 / 44.8, 8192 x 2048 18.4 / 45.4 against 23.6 / 46.1:
+    // ahead on every layer whose codebook stays in memory.
+    const bool wins = big;
     if (c.cb_dtype == c.act && c.n_bytes < ((int64_t)1 << 32) && (mode >= 2 || (mode == 1 && wins))) {
       const T2Args t2{c.packed, c.cb, (uint32_t)c.nc - 1u, s.chunks};
       const int rc = launch_tile2(ACT, s, t2, c.st, c.what, c.ws, c.ws_bytes);

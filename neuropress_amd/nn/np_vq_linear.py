@@ -115,12 +115,17 @@ _TILE_MAX_TOKENS: int = _env_int(
     ("NEUROPRESS_VQ_TILE_MAX_TOKENS", "NEUROPRESS_VQ_TRITON_MAX_TOKENS"), 256
 )
 
-# Layers whose codebook LDS does not hold (more than 4096 rows of eight) and that have at least
-# _TILE_WIDE_MIN_WEIGHTS weights run the 128-column tile GEMM, which stays ahead of decode + GEMM up
-# to its 384-row block: 14336 x 4096 70 us at 384 tokens against 102 us, 4096 x 14336 76 us against
-# 117 us (the 64-column kernel: 80 and 87 us).
+# Layers whose codebook LDS does not hold (more than 4096 rows of eight) run the 128-column tile GEMM,
+# which splits the reduction by itself and stays ahead of decode + GEMM up to a token count that goes
+# with the layer's weights (us at 128 / 256 / 384 tokens, tile against decode + GEMM): 14336 x 4096
+# 47 / 59 / 73 against 81 / 96 / 101, 4096 x 14336 53 / 67 / 82 against 114 / 103 / 117; 6144 x 4096
+# 32 / 41 / 56 against 47 / 61 / 55, 4096 x 4096 28 / 34 / 42 against 40 / 38 / 41, 8192 x 2048 28 / 34 / 46
+# against 34 / 40 / 38; 1024 x 4096 18 / 24 / 29 against 20 / 21 / 22, 2048 x 2048 16 / 23 / 28 against 17 / 20 / 20.
 _TILE_WIDE_MAX_TOKENS: int = _env_int(("NEUROPRESS_VQ_TILE_WIDE_MAX_TOKENS",), 384)
-_TILE_WIDE_MIN_WEIGHTS: int = 1 << 25
+_TILE_WIDE_MIN_WEIGHTS: int = 1 << 25  # below: 256 tokens
+_TILE_WIDE_SMALL_WEIGHTS: int = 1 << 24  # below: 128 tokens
+_TILE_WIDE_MID_MAX_TOKENS: int = 256
+_TILE_WIDE_SMALL_MAX_TOKENS: int = 128
 
 # The tile GEMM gives each workgroup 64 output columns (and up to 384 rows).  When
 # that grid covers less than this fraction of the compute units the kernel splits
@@ -961,16 +966,24 @@ class NPVQLinear(nn.Module):
             self._derived["mfma_layer"] = ok
         return ok
 
+    def _wide_tile_layer(self) -> bool:
+        """Whether the tile GEMM of this layer is the 128-column kernel (codebook kept in memory)."""
+        return (
+            not self.is_residual
+            and self.vector_len == 8
+            and 12 < self.bits <= 16  # read as a 16-bit stream (see _kernel_stream)
+            and self.proxy.num_centroids * self.vector_len * 2 > 65536
+        )
+
     def _tile_max_tokens(self) -> int:
         """Upper end of the tile-decode GEMM band for this layer."""
-        if (
-            _TILE_MAX_TOKENS > 0
-            and not self.is_residual
-            and self.vector_len == 8
-            and self.proxy.num_centroids * self.vector_len * 2 > 65536
-            and self.in_features * self.out_features >= _TILE_WIDE_MIN_WEIGHTS
-        ):
-            return max(_TILE_MAX_TOKENS, _TILE_WIDE_MAX_TOKENS)
+        if _TILE_MAX_TOKENS > 0 and self._wide_tile_layer():
+            weights = self.in_features * self.out_features
+            if weights >= _TILE_WIDE_MIN_WEIGHTS:
+                return max(_TILE_MAX_TOKENS, _TILE_WIDE_MAX_TOKENS)
+            if weights >= _TILE_WIDE_SMALL_WEIGHTS:
+                return min(_TILE_WIDE_MAX_TOKENS, _TILE_WIDE_MID_MAX_TOKENS)
+            return min(_TILE_WIDE_MAX_TOKENS, _TILE_WIDE_SMALL_MAX_TOKENS)
         return _TILE_MAX_TOKENS
 
     def _tile_band_ok(self, x: torch.Tensor, m: int) -> bool:
@@ -981,6 +994,8 @@ class NPVQLinear(nn.Module):
             return True
         if not self._mfma_layer():
             return False  # the tile entry point would run its element-wise fallback
+        if self._wide_tile_layer():
+            return True  # the 128-column kernel fills the GPU by splitting the reduction; its band is a token count
         cus = self._derived.get("cus")
         if cus is None:
             cus = torch.cuda.get_device_properties(x.device).multi_processor_count

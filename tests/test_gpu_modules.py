@@ -281,6 +281,7 @@ def test_prefix_coded_layers_run_the_hip_bands(gpu, kind, monkeypatch):
 
     monkeypatch.setattr(vqmod, "_SLICED_MIN_INDICES", 1)
     monkeypatch.setattr(vqmod, "_TILE_MAX_TOKENS", 64)
+    monkeypatch.setattr(vqmod, "_TILE_WIDE_SMALL_MAX_TOKENS", 64)  # the band of a small layer with a codebook in memory
     monkeypatch.setattr(vqmod, "_TILE_MIN_GRID_FRACTION", 0.0)
     n, k, nc = 128, 512, 20000
     g = cases.gen(91)

@@ -47,11 +47,16 @@ def _check(y, ref):
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 17, 96, 130, 257, 300, 384, 400])
-@pytest.mark.parametrize("n,k,splits", [(300, 448, 1), (300, 448, 2), (130, 1024, 2), (264, 1088, 3), (1004, 512, 0)])
+@pytest.mark.parametrize(
+    "n,k,splits",
+    [(300, 448, 1), (300, 448, 2), (130, 1024, 2), (264, 1088, 3), (1004, 512, 0), (300, 192, 1), (300, 256, 1), (300, 128, 1)],
+)
 def test_wide_tile_gemm_against_the_oracle(gpu, oracle_lib, tile_wide, act, m, n, k, splits):
-    """Ragged N (two to eight 128-column blocks, N % 8 != 0 once: element stores), K of 7 to 17 steps, every row
-    tile count (one to three per wave, two row blocks at 400 tokens), K whole, in two halves that meet
-    in the kernel, and in three parts that meet in the reduction kernel."""
+    """Ragged N (two to eight 128-column blocks, N % 8 != 0 once: element stores), K of 3 to 17 steps (odd and
+    even counts per part: the loop ends in two steps of its own behind pairs; two steps are fewer than the
+    kernel takes, so the 64-column kernel answers), every row tile count (one to three per wave, two row
+    blocks at 400 tokens), K whole, in two halves that meet in the kernel, and in three parts that meet in
+    the reduction kernel."""
     from neuropress_amd import kernels
 
     tile_wide(2, splits)
@@ -117,12 +122,15 @@ def _q_ref(oracle_lib, L, act):
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("nbits,asym,gs", [(4, False, 32), (4, True, 32), (4, False, 128), (8, False, 32), (8, True, 64)])
 @pytest.mark.parametrize("m", [1, 17, 130, 257, 384, 400, 520])
-@pytest.mark.parametrize("n,k,splits", [(300, 512, 1), (300, 512, 2), (264, 1024, 3)])
+@pytest.mark.parametrize("n,k,splits", [(300, 512, 1), (300, 512, 2), (264, 1024, 3), (300, 448, 1), (300, 448, 2), (300, 192, 1)])
 def test_wide_tile_gemm_group_affine_against_the_oracle(gpu, oracle_lib, tile_wide, act, nbits, asym, gs, m, n, k, splits):
     """int4 / int8 codes through the 128-column kernel (packed bytes staged in LDS, decoded between the MFMAs):
     symmetric and with zero points, group sizes of 32 to 128, one to three row tiles per wave and the 256-row
-    blocks taken past 384 tokens, K whole, in two halves and in three parts."""
+    blocks taken past 384 tokens, K whole, in two halves and in three parts, odd and even step counts."""
     from neuropress_amd import kernels
+
+    if k % gs:
+        pytest.skip("K is not a multiple of the group size")
 
     tile_wide(2, splits)
     Q = cases.q4_layer(800 + m + nbits, n, k, nbits=nbits, gs=gs, act=act, m=m, asym=asym, bias=True)

@@ -111,7 +111,8 @@ def test_the_wide_kernel_loads_everything_into_lds_and_leaves_m0_to_its_transfer
     (``s_waitcnt vmcnt(n)``).  Sound only while (a) the compiler keeps nothing of its own in m0 and (b)
     every vector-memory load of the main loop is one of those transfers, so that the hand-written counts
     see all of a wave's loads: outside asm statements the kernels may load from global memory only where
-    the compiler's own waits cover it (bias, the handoff's first look at the tile word)."""
+    the compiler's own waits cover it (bias, the other half's tile, and the look at the tile word in front of
+    the last step, which only makes the hand-written waits behind it stricter)."""
     lines = assembly_wide
     starts = [i for i, ln in enumerate(lines) if re.match(r"^_ZN5npamd17tile2_gemm_kernel\S*: ;", ln)]
     assert len(starts) >= 20  # VQ and int4 / int8 producers x activation dtypes x row tiles
@@ -132,7 +133,7 @@ def test_the_wide_kernel_loads_everything_into_lds_and_leaves_m0_to_its_transfer
             if re.match(r"\s+scratch_(load|store)", code):
                 spills += 1
         assert transfers >= 10, (name, transfers)
-        assert spills == 0, (name, spills)  # 512 registers per lane hold the wave tile: nothing goes to scratch
+        assert spills == 0, (name, spills)  # 256 registers per lane hold the wave tile: nothing goes to scratch
 
 
 @pytest.fixture(scope="module")
