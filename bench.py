@@ -43,7 +43,7 @@ POOL_BYTES = 640 << 20         # rotate through more than L2 (32 MB) + Infinity 
 # in `source` holds the command, the raw counter values and the date they were taken.
 TRAFFIC = {
     "sliced_m1": {"bytes": 13577 * 1024 * 2 + 1932 * 1024, "source": "profiles/vq_sliced_gemv_cfg3_14336x4096_m1.md"},
-    "tile_m384": {"bytes": 59876 * 1024 * 2 + 45478 * 1024, "source": "profiles/vq_tile_gemm_cfg3_14336x4096_m384.md"},
+    "tile_m384": {"bytes": 35573 * 1024 * 2 + 51082 * 1024, "source": "profiles/vq_tile_gemm_cfg3_14336x4096_m384.md"},
 }
 FLUSH_BYTES = 512 << 20        # written before every timed replay: nothing a replay reads is still cached
 
@@ -455,7 +455,7 @@ def main():
         "bound": "mfma", "achieved": round(flops2 / us_tile / 1e6, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(flops2 / us_tile / 1e6 / MFMA_PEAK_TFLOPS, 4),
         "traffic": TRAFFIC["tile_m384"]["bytes"], "traffic_source": TRAFFIC["tile_m384"]["source"],
-        "kernel": "tile2_gemm_kernel<bf16, MW=3, VQ 16-bit> (128 columns, K in two halves)", "flops_per_launch": flops2,
+        "kernel": "tile2_gemm_kernel<bf16, MW=3, VQ 16-bit> (128 columns, eight waves, K in two halves)", "flops_per_launch": flops2,
         "avg_launch_us": round(us_tile, 3), "M": m2, "output_within_1e-2": ok2, "max_abs_err": max_abs2,
         # the same flops as MFMAs only, on all compute units, in this run
         "floor_us": round(us_mfma, 3), "frac_at_floor": round(flops2 / us_mfma / 1e6 / MFMA_PEAK_TFLOPS, 4),

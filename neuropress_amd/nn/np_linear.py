@@ -42,8 +42,8 @@ _Q_TILE_MAX_TOKENS: int = int(os.environ.get("NEUROPRESS_Q_TILE_MAX_TOKENS", "25
 # GEMM up to this many tokens: 4096 x 14336 80 vs 105-109 us at 320-384, 148 vs 120 us at 512.
 _Q_TILE_LONG_K_MAX_TOKENS: int = 384
 # Layers of at least _Q_TILE_WIDE_MIN_FEATURES output or input features run the 128-column fused GEMM
-# (256-row blocks past 384 tokens): 14336 x 4096 68-75 us at 384 tokens and 77-88 at 512 against 86 and 93 us
-# for decode + GEMM, 155 against about 140 at 1024; 4096 x 14336 73 / 84 us at 384 / 512.
+# (256-row blocks past 384 tokens): 14336 x 4096 61 us at 384 tokens and 78-82 at 512 against 86 and 93 us
+# for decode + GEMM, 150 against about 140 at 1024; 4096 x 14336 68 / 82 us at 384 / 512.
 _Q_TILE_WIDE_MAX_TOKENS: int = int(os.environ.get("NEUROPRESS_Q_TILE_WIDE_MAX_TOKENS", "512"))
 _Q_TILE_WIDE_MIN_FEATURES: int = 8192
 # As for the VQ path: the fused GEMM splits the reduction when the layer has few
