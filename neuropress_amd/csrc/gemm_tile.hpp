@@ -209,7 +209,8 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
   // Both software pipelines are unrolled by their depth with no branches inside
   // (a branch would make the compiler drain every outstanding load at the join),
   // so all waves run `total` iterations: steps rounded up to a multiple of kDepth.
-  // The padding iterations decode clamped addresses into buffers nobody reads.
+  // The padding iterations decode clamped addresses into buffers nobody reads (lookups for steps past
+  // the end all go to codebook row 0).
   const int total = (steps + kDepth - 1) / kDepth * kDepth;
 
   // Producer lane: column 16q + l % 16 of the tile, operand pair jp = l / 16 (see below).  Its
@@ -276,14 +277,14 @@ tile_gemm_kernel(const GemmShape s, const typename Provider::Args pargs) {
     auto advance = [&](typename Provider::PairOps& o, typename Provider::PairRaw& raw, int t, int slot) {
       store_w(o, slot);
       asm volatile("" ::: "memory");
-      prov.gather_pair(raw, jp, o);
+      prov.gather_pair(raw, jp, o, t + 2 + kDepth < steps);
       load_raw(raw, t + 2 + 2 * kDepth);
     };
 
     // Prologue: steps 0..kDepth-1 in flight, packed bytes of kDepth..2*kDepth-1 loaded; then
     // "iterations -2 and -1": store steps 0 and 1 and refill their registers.
 #pragma unroll
-    for (int p = 0; p < kDepth; ++p) prov.gather_pair(raws[p], jp, ops[p]);  // packed bytes requested above
+    for (int p = 0; p < kDepth; ++p) prov.gather_pair(raws[p], jp, ops[p], p < steps);  // packed bytes requested above
 #pragma unroll
     for (int p = 0; p < kDepth; ++p) load_raw(raws[p], p + kDepth);
     advance(ops[0], raws[0], -2, 0);

@@ -112,12 +112,15 @@ struct VqProvider {
     u32x4 b0, b1;
   };
   static constexpr int kLdsOpsPerGather = VL == 8 ? 2 : 4;  // LDS reads of one gather_pair from an LDS codebook
-  __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o) const {
+  // `live` false (a step past the end, issued to keep the pipeline free of branches): every lane looks up
+  // row 0, one cache line per instruction instead of up to 64.
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o, bool live = true) const {
     const u32x4 v = extract_idx8<BITS>(r.w);
     if constexpr (VL == 8) {
+      const uint32_t lim = live ? a.nc_minus_1 : 0u;
       const uint32_t pair = select_dword(v, jp);  // indices of operands 2*jp (low half) and 2*jp+1
-      o.b0 = cb[min(pair & 0xFFFFu, a.nc_minus_1)];
-      o.b1 = cb[min(pair >> 16, a.nc_minus_1)];
+      o.b0 = cb[min(pair & 0xFFFFu, lim)];
+      o.b1 = cb[min(pair >> 16, lim)];
     } else {
       const uint32_t pair = (jp & 1) ? v.z : v.x;   // the two rows of operand 2*jp
       const uint32_t pair1 = (jp & 1) ? v.w : v.y;  // those of operand 2*jp+1
@@ -197,13 +200,14 @@ struct RvqProvider {
     u32x4 cm0, cr0, cm1, cr1;  // main and residual rows of the two operands, as gathered
   };
   static constexpr int kLdsOpsPerGather = 2;  // with the residual codebook in LDS: its two lookups
-  __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o) const {
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int jp, PairOps& o, bool live = true) const {
     const uint32_t pm = select_dword(extract_idx8<BITS_M>(r.wm), jp);
     const uint32_t pr = select_dword(extract_idx8<BITS_R>(r.wr), jp);
-    o.cm0 = a.cb_m[min(pm & 0xFFFFu, a.ncm_minus_1)];
-    o.cm1 = a.cb_m[min(pm >> 16, a.ncm_minus_1)];
-    o.cr0 = cbr[min(pr & 0xFFFFu, a.ncr_minus_1)];
-    o.cr1 = cbr[min(pr >> 16, a.ncr_minus_1)];
+    const uint32_t lim_m = live ? a.ncm_minus_1 : 0u, lim_r = live ? a.ncr_minus_1 : 0u;  // see VqProvider::gather_pair
+    o.cm0 = a.cb_m[min(pm & 0xFFFFu, lim_m)];
+    o.cm1 = a.cb_m[min(pm >> 16, lim_m)];
+    o.cr0 = cbr[min(pr & 0xFFFFu, lim_r)];
+    o.cr1 = cbr[min(pr >> 16, lim_r)];
   }
   __device__ __forceinline__ void finish_pair(const PairOps& o, u32x4& b0, u32x4& b1) const {
     b0 = combine_rows(o.cm0, o.cr0, s2, b2);
@@ -302,7 +306,7 @@ struct Q4Provider {
     u32x4 b0, b1;  // finished operands: the dequantization waits for nothing but the packed bytes
   };
   static constexpr int kLdsOpsPerGather = 0;
-  __device__ __forceinline__ void gather_pair(const PairRaw& r, int, PairOps& o) const {
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int, PairOps& o, bool = true) const {
     o.b0 = dequant8(r.w.x, r.s2, r.z);
     o.b1 = dequant8(r.w.y, r.s2, r.z);
   }
@@ -418,7 +422,7 @@ struct Q8Provider {
     u32x4 b0, b1;  // finished operands
   };
   static constexpr int kLdsOpsPerGather = 0;
-  __device__ __forceinline__ void gather_pair(const PairRaw& r, int, PairOps& o) const {
+  __device__ __forceinline__ void gather_pair(const PairRaw& r, int, PairOps& o, bool = true) const {
     o.b0 = dequant8(r.w.x, r.w.y, r.s2, r.z);
     o.b1 = dequant8(r.w.z, r.w.w, r.s2, r.z);
   }
