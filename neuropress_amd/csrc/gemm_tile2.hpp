@@ -48,7 +48,6 @@ namespace npamd {
 
 constexpr int kT2Cols = 128;
 constexpr int kT2WSlotBytes = kT2Cols * kStepK * 2;  // 16 KiB: [column tile 4][operand j 4][lane 64][16 B]
-constexpr int kT2WRing = 3;
 
 struct T2Args {
   const uint8_t* packed;  // 16-bit indices, [N][K / 8]
@@ -80,7 +79,8 @@ int plan_tile2_splits(int M, int N, int chunks, int mw);
 int tile2_mode();
 
 // Row tiles per wave for the group-affine producers, whose decode is cheap enough to repeat per row block: past
-// 384 tokens two (256-row blocks: int4 14336 x 4096 at 512 / 1024 tokens 77 / 155 us against 97 / 173 with three).
+// 384 tokens two (256-row blocks: int4 14336 x 4096 at 512 / 1024 tokens 77 / 155 us against 97 / 173 with three,
+// measured on the four-wave form of the kernel).
 inline int plan_tile2_q_mw(int M) {
   const int mw = plan_tile_mw(M);
   return M > 384 && mw == 3 ? 2 : mw;
