@@ -118,9 +118,12 @@ int npamd_gemv_stages_activations(int M, int N, int K, int nc);
  * WMMA GEMM branch of vq_linear_wmma (neuropress/kernels/vq_linear_wmma.cu:261-394).
  * `workspace` (all three *_gemm_tile entry points): NULL, or 16-byte aligned device
  * memory of npamd_gemm_tile_workspace_bytes(M, N, K) bytes.  With it, layers
- * whose column blocks would not fill the GPU (few output features) split K over
- * more workgroups and add the f32 partial tiles in a second kernel; without it,
- * or when it is too small, K is not split.  Contents irrelevant before and after.
+ * whose column blocks would not fill the GPU split K over more workgroups, which
+ * hand their f32 partial tiles over through it: two parts meet inside the kernel
+ * (whichever finishes second adds the other's tile), more are added by a second
+ * kernel; without it, or when it is too small, K is not split.  Contents
+ * irrelevant before and after (nobody clears it); two calls that may run at the
+ * same time need a workspace each.
  */
 int npamd_vq_gemm_tile(const void* x, int64_t ldx, const uint8_t* packed, int64_t n_bytes,
                        int bits, const void* codebook, int codebook_dtype, int nc, int vl,
