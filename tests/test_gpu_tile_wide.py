@@ -68,6 +68,23 @@ def test_wide_tile_gemm_against_the_oracle(gpu, oracle_lib, tile_wide, act, m, n
     assert torch.equal(y, y2), "the result depends on which half of K finished first"
 
 
+@pytest.mark.parametrize("m", [17, 200, 384])
+def test_wide_tile_gemm_takes_activations_with_a_row_stride(gpu, tile_wide, m):
+    """x as a view of a wider buffer (row stride 2 K + 8 elements, rows 16-byte aligned): the x tile's transfers
+    take the stride from the call; the result equals the one on a contiguous copy bit for bit."""
+    from neuropress_amd import kernels
+
+    n, k = 300, 448
+    tile_wide(2, 2)
+    L = cases.vq_layer(650 + m, n, k, 65536, bits=16, act=torch.bfloat16, m=m, bias=True, std=0.05)
+    pk, cb, bias = L["packed"].to(gpu), L["cb"].bfloat16().to(gpu), L["bias"].to(gpu)
+    wide = torch.full((m, 2 * k + 8), float("nan"), dtype=torch.bfloat16, device=gpu)
+    wide[:, :k] = L["x"].to(gpu)
+    view = wide[:, :k]
+    assert view.stride(0) == 2 * k + 8 and not view.is_contiguous()
+    assert torch.equal(kernels.vq_gemm_tile(view, pk, cb, 16, n, bias), kernels.vq_gemm_tile(view.contiguous(), pk, cb, 16, n, bias))
+
+
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("splits", [1, 2, 4])
 def test_wide_tile_gemm_decodes_bit_exactly(gpu, tile_wide, act, splits):
