@@ -881,9 +881,22 @@ class NPVQLinear(nn.Module):
         if limit == 16 and 16 < m <= min(_FUSED_WIDE_MAX_TOKENS, 32):
             if self.is_residual or m * self.in_features <= _FUSED_WIDE_MAX_ACTIVATIONS:
                 return 32
-            if self._gemv_stages_activations(m):
+            if self._gemv_stages_activations(m) and not self._tile_ahead_from_17():
                 return 32
         return limit
+
+    def _tile_ahead_from_17(self) -> bool:
+        """Large layers with at least twice as many output as input features and a codebook kept in memory: the
+        128-column tile GEMM is level with the staged GEMV at 17 tokens and ahead at 24-32 (tile vs GEMV at
+        17 / 24 / 32 tokens: 14336 x 4096 40.3 / 39.0 / 40.4 vs 41.0 / 42.2 / 43.1 us, 11008 x 4096 35.4 / 35.8 / 36.1
+        vs 35.6 / 36.9 / 39.2); on 8192 x 8192 they tie, on 4096 x 14336 (44 vs 39-41.5 us) and on small layers
+        (4096 x 4096: 20.6-21.3 vs 13.3-14.0) the GEMV stays ahead."""
+        return (
+            _TILE_MAX_TOKENS > 0
+            and self._wide_tile_layer()
+            and self.out_features >= 2 * self.in_features
+            and self.in_features * self.out_features >= _TILE_WIDE_MIN_WEIGHTS
+        )
 
     def _gemv_stages_activations(self, m: int) -> bool:
         """Layers of one row tile per workgroup whose lookups go to memory run the GEMV that stages
